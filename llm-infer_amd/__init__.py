@@ -1,0 +1,31 @@
+"""llm_infer_amd: a small, whole Llama generation library for one MI355X.
+
+    engine = llm_infer_amd.load("model_dir", dtype="bfloat16", max_tokens=65536)
+    new_tokens = engine.generate([[1, 2, 3], [4, 5]], max_new_tokens=16, temperature=0.0)
+"""
+from .config import ConfigError, LlamaConfig
+from .registry import (config_from_dict, config_from_folder, register_architecture, register_block,
+                       register_embedding, register_feed_forward, register_head, register_mixer,
+                       register_norm, register_position)
+
+__version__ = "0.1.0"
+
+register_architecture("LlamaForCausalLM", LlamaConfig)
+
+
+def load(folder: str, dtype: str = "bfloat16", max_tokens: int = 8192, n_slots=None):
+    """Open a model folder (config.json + model.safetensors) on the GPU."""
+    from .engine import Engine
+    return Engine.from_folder(folder, dtype=dtype, max_tokens=max_tokens, n_slots=n_slots)
+
+
+def random_model(config, seed: int = 0, dtype: str = "bfloat16", max_tokens: int = 8192, n_slots=None):
+    """An engine with random weights made on the GPU from a configuration and a seed."""
+    from .engine import Engine
+    return Engine.from_random(config, seed=seed, dtype=dtype, max_tokens=max_tokens, n_slots=n_slots)
+
+
+def write_random_model(folder: str, config, seed: int = 0, dtype: str = "bfloat16") -> None:
+    """Write config.json and model.safetensors for a configuration and a seed."""
+    from .weights import write_random_model as _w
+    _w(folder, config, seed, dtype)

@@ -1,0 +1,368 @@
+// Causal grouped-query attention over the paged cache, compiled for one head
+// size (HEAD_DIM, a multiple of 16 up to 256).
+//
+// Formula (include/kernels_cpu.hpp:122-167, src/model/block.cpp:158-164): a query
+// at position p of head h reads the keys 0..p of KV head h / (H/K); score =
+// (q.k) * scale; softmax with the maximum subtracted; output = sum_t p_t v_t.
+// With a window w only the keys p-w+1..p count.  Scores, softmax and the
+// running sums are float32.
+//
+// 16-bit kernels: one wave owns 32 query rows.  S^T = K Q^T and O^T = V^T P^T are
+// computed with the 32x32x16 matrix instruction; keys and values come from the
+// cache already in operand order (common.h), so every operand is one contiguous
+// load and the probabilities go from the accumulators of the first product
+// straight into operand B of the second.  Pages are combined by the online
+// softmax rule (state m, l, o; src/attention.cu:12-65 holds the same merge with
+// o kept normalised).
+//   prefill: 4 waves = 128 consecutive tokens of one sequence and one query head.
+//   decode : one wave = the query heads of one KV head for one sequence and one
+//            split of the context; splits are merged by a second kernel.
+// float32 kernel: one workgroup per (token, head), keys in ascending order, so a
+// result does not depend on how the step was cut or batched.
+#include "common.h"
+
+#ifndef HEAD_DIM
+#error "compile with -DHEAD_DIM=<head size>"
+#endif
+static_assert(HEAD_DIM % 16 == 0 && HEAD_DIM >= 16 && HEAD_DIM <= 256, "head size: multiple of 16, at most 256");
+
+constexpr int HD = HEAD_DIM;
+constexpr int KS = HD / 16;              // steps of the inner index for the scores
+constexpr int DB = (HD + 31) / 32;       // 32-row blocks of the output's head dim
+constexpr float LOG2E = 1.4426950408889634f;
+
+struct CachePtrs {
+    const void* k;            // keys of this layer: page p at k + p * page_stride (elements)
+    const void* v;
+    int64_t page_stride;
+    const int* page_table;    // [n_slots, max_pages]
+    int max_pages;
+};
+
+template <class T>
+struct WaveAttn {
+    typedef typename Vec<T>::v8 v8;
+    v8 q[KS];
+    f32x16 o[DB];
+    float m, l;
+
+    __device__ __forceinline__ void init(const T* qrow) {
+        const int lane = threadIdx.x & 63;
+#pragma unroll
+        for (int s = 0; s < KS; ++s) {
+            v8 z = {};
+            q[s] = qrow ? *(const v8*)(qrow + 16 * s + 8 * (lane >> 5)) : z;
+        }
+#pragma unroll
+        for (int b = 0; b < DB; ++b)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) o[b][r] = 0.f;
+        m = -INFINITY;
+        l = 0.f;
+    }
+
+    // One page of 64 keys starting at key t0.  This lane's row sees keys lo..hi (hi < lo: none).
+    __device__ __forceinline__ void page(const T* kpage, const T* vpage, int t0, int lo, int hi, float scale2) {
+        const int lane = threadIdx.x & 63;
+        f32x16 s[2];
+#pragma unroll
+        for (int b = 0; b < 2; ++b) {
+#pragma unroll
+            for (int r = 0; r < 16; ++r) s[b][r] = 0.f;
+#pragma unroll
+            for (int ks = 0; ks < KS; ++ks) {
+                const v8 kf = *(const v8*)(kpage + ((b * KS + ks) * 64 + lane) * 8);
+                s[b] = mfma32(kf, q[ks], s[b]);
+            }
+        }
+        float mx = -INFINITY;
+#pragma unroll
+        for (int b = 0; b < 2; ++b)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) {
+                const int t = t0 + 32 * b + 8 * (r >> 2) + 4 * (lane >> 5) + (r & 3);
+                const float v = (t >= lo && t <= hi) ? s[b][r] * scale2 : -INFINITY;
+                s[b][r] = v;
+                mx = fmaxf(mx, v);
+            }
+        mx = fmaxf(mx, __shfl_xor(mx, 32, WAVE));
+        const float m_new = fmaxf(m, mx);
+        const float m_safe = (m_new == -INFINITY) ? 0.f : m_new;
+        const float alpha = exp2f(m - m_safe);
+        float psum = 0.f;
+#pragma unroll
+        for (int b = 0; b < 2; ++b)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) {
+                const float p = exp2f(s[b][r] - m_safe);
+                s[b][r] = p;
+                psum += p;
+            }
+        l = l * alpha + psum;
+        m = m_new;
+#pragma unroll
+        for (int b = 0; b < DB; ++b)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) o[b][r] *= alpha;
+#pragma unroll
+        for (int tj = 0; tj < 4; ++tj) {
+            v8 pf;
+#pragma unroll
+            for (int i = 0; i < 8; ++i) pf[i] = from_f32<T>(s[tj >> 1][8 * (tj & 1) + i]);
+#pragma unroll
+            for (int b = 0; b < DB; ++b) {
+                const v8 vf = *(const v8*)(vpage + ((b * 4 + tj) * 64 + lane) * 8);
+                o[b] = mfma32(vf, pf, o[b]);
+            }
+        }
+    }
+
+    __device__ __forceinline__ float total() const { return l + __shfl_xor(l, 32, WAVE); }
+};
+
+// ---------------------------------------------------------------------------
+// prefill
+// ---------------------------------------------------------------------------
+template <class T>
+__global__ __launch_bounds__(256) void attn_prefill_kernel(
+    const T* __restrict__ q, T* __restrict__ out, CachePtrs c, const int* __restrict__ tile_seq,
+    const int* __restrict__ tile_q0, const int* __restrict__ seq_slot, const int* __restrict__ seq_qstart,
+    const int* __restrict__ seq_qlen, const int* __restrict__ seq_ctx, int H, int K, float scale, int window) {
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int seq = tile_seq[blockIdx.x];
+    const int h = blockIdx.y, kvh = h / (H / K);
+    const int qlen = seq_qlen[seq], ctx = seq_ctx[seq];
+    const int first = tile_q0[blockIdx.x] + 32 * wave;          // this wave's first token within the step
+    if (first >= qlen) return;
+    const int qi = first + (lane & 31);
+    const bool live = qi < qlen;
+    const int base = ctx - qlen;                                 // tokens cached before this step
+    const int pos = live ? base + qi : -1;
+    const int64_t tok = seq_qstart[seq] + qi;
+    WaveAttn<T> a;
+    a.init(live ? q + (tok * H + h) * HD : nullptr);
+    const int lo = (window > 0 && live) ? max(0, pos - window + 1) : 0;
+    const int last_pos = base + min(first + 31, qlen - 1);
+    const int first_lo = window > 0 ? max(0, base + first - window + 1) : 0;
+    const int* table = c.page_table + (int64_t)seq_slot[seq] * c.max_pages;
+    const float scale2 = scale * LOG2E;
+    for (int p = first_lo / PAGE; p <= last_pos / PAGE; ++p) {
+        const int64_t page = table[p];
+        const T* kp = (const T*)c.k + page * c.page_stride + (int64_t)kvh * k_head_elems(HD);
+        const T* vp = (const T*)c.v + page * c.page_stride + (int64_t)kvh * v_head_elems(HD);
+        a.page(kp, vp, p * PAGE, lo, pos, scale2);
+    }
+    const float inv = 1.f / a.total();
+    if (!live) return;
+    T* orow = out + (tok * H + h) * HD;
+#pragma unroll
+    for (int b = 0; b < DB; ++b)
+#pragma unroll
+        for (int g = 0; g < 4; ++g) {
+            const int d = 32 * b + 8 * g + 4 * (lane >> 5);
+            if (d < HD) {
+                typename Vec<T>::v4 v = {from_f32<T>(a.o[b][4 * g] * inv), from_f32<T>(a.o[b][4 * g + 1] * inv),
+                                         from_f32<T>(a.o[b][4 * g + 2] * inv), from_f32<T>(a.o[b][4 * g + 3] * inv)};
+                *(typename Vec<T>::v4*)(orow + d) = v;
+            }
+        }
+}
+
+// ---------------------------------------------------------------------------
+// decode: one new token per sequence, q [B, H, HD]
+// ---------------------------------------------------------------------------
+template <class T>
+__global__ __launch_bounds__(64) void attn_decode_kernel(
+    const T* __restrict__ q, T* __restrict__ out, float* __restrict__ part_o, float* __restrict__ part_ml,
+    CachePtrs c, const int* __restrict__ seq_slot, const int* __restrict__ seq_ctx, int H, int K, float scale,
+    int window) {
+    const int lane = threadIdx.x & 63;
+    const int b = blockIdx.x, G = H / K, gchunks = (G + 31) / 32;
+    const int kvh = blockIdx.y / gchunks, gc = blockIdx.y % gchunks;
+    const int S = gridDim.z, split = blockIdx.z;
+    const int hg = gc * 32 + (lane & 31);
+    const bool live = hg < G;
+    const int h = kvh * G + hg;
+    const int ctx = seq_ctx[b];
+    const int pos = ctx - 1;
+    WaveAttn<T> a;
+    a.init(live ? q + ((int64_t)b * H + h) * HD : nullptr);
+    const int lo = window > 0 ? max(0, pos - window + 1) : 0;
+    const int p_first = lo / PAGE, p_end = pos / PAGE + 1;
+    const int per = (p_end - p_first + S - 1) / S;
+    const int p0 = p_first + split * per, p1 = min(p_end, p0 + per);
+    const int* table = c.page_table + (int64_t)seq_slot[b] * c.max_pages;
+    const float scale2 = scale * LOG2E;
+    for (int p = p0; p < p1; ++p) {
+        const int64_t page = table[p];
+        const T* kp = (const T*)c.k + page * c.page_stride + (int64_t)kvh * k_head_elems(HD);
+        const T* vp = (const T*)c.v + page * c.page_stride + (int64_t)kvh * v_head_elems(HD);
+        a.page(kp, vp, p * PAGE, lo, live ? pos : -1, scale2);
+    }
+    const float total = a.total();
+    if (!live) return;
+    if (S == 1) {
+        const float inv = 1.f / total;
+        T* orow = out + ((int64_t)b * H + h) * HD;
+#pragma unroll
+        for (int blk = 0; blk < DB; ++blk)
+#pragma unroll
+            for (int g = 0; g < 4; ++g) {
+                const int d = 32 * blk + 8 * g + 4 * (lane >> 5);
+                if (d < HD) {
+#pragma unroll
+                    for (int i = 0; i < 4; ++i) orow[d + i] = from_f32<T>(a.o[blk][4 * g + i] * inv);
+                }
+            }
+        return;
+    }
+    const int64_t slot = ((int64_t)b * H + h) * S + split;
+    float* po = part_o + slot * HD;
+#pragma unroll
+    for (int blk = 0; blk < DB; ++blk)
+#pragma unroll
+        for (int g = 0; g < 4; ++g) {
+            const int d = 32 * blk + 8 * g + 4 * (lane >> 5);
+            if (d < HD) {
+#pragma unroll
+                for (int i = 0; i < 4; ++i) po[d + i] = a.o[blk][4 * g + i];
+            }
+        }
+    if (lane < 32) { part_ml[slot * 2] = a.m; part_ml[slot * 2 + 1] = total; }
+}
+
+// Merge of the splits: M = max m_s, L = sum l_s 2^(m_s - M), o = sum o_s 2^(m_s - M) / L.
+template <class T>
+__global__ void attn_merge_kernel(const float* __restrict__ part_o, const float* __restrict__ part_ml,
+                                  T* __restrict__ out, int S) {
+    const int64_t row = blockIdx.x;                  // (sequence, head)
+    const float* ml = part_ml + row * S * 2;
+    float M = -INFINITY;
+    for (int s = 0; s < S; ++s) M = fmaxf(M, ml[2 * s]);
+    float L = 0.f;
+    for (int s = 0; s < S; ++s) L += (ml[2 * s] == -INFINITY) ? 0.f : ml[2 * s + 1] * exp2f(ml[2 * s] - M);
+    for (int d = threadIdx.x; d < HD; d += blockDim.x) {
+        float acc = 0.f;
+        for (int s = 0; s < S; ++s)
+            if (ml[2 * s] != -INFINITY) acc += part_o[(row * S + s) * HD + d] * exp2f(ml[2 * s] - M);
+        out[row * HD + d] = from_f32<T>(acc / L);
+    }
+}
+
+// ---------------------------------------------------------------------------
+// float32: one workgroup of 256 threads per (token, head); chunks of 256 keys.
+// ---------------------------------------------------------------------------
+__global__ __launch_bounds__(256) void attn_f32_kernel(
+    const float* __restrict__ q, float* __restrict__ out, CachePtrs c, const int* __restrict__ pos_of,
+    const int* __restrict__ tok_slot, int H, int K, float scale, int window) {
+    __shared__ float sq[HD];
+    __shared__ float sp[256];
+    __shared__ float scratch[16];
+    const int tid = threadIdx.x;
+    const int64_t tok = blockIdx.x;
+    const int h = blockIdx.y, kvh = h / (H / K);
+    const int pos = pos_of[tok];
+    const int lo = window > 0 ? max(0, pos - window + 1) : 0;
+    const int* table = c.page_table + (int64_t)tok_slot[tok] * c.max_pages;
+    for (int d = tid; d < HD; d += 256) sq[d] = q[(tok * H + h) * HD + d];
+    __syncthreads();
+    float m = -INFINITY, l = 0.f, o = 0.f;            // o: thread d < HD owns output dim d
+    for (int t0 = lo; t0 <= pos; t0 += 256) {
+        const int t = t0 + tid;
+        float s = -INFINITY;
+        if (t <= pos) {
+            const float* kp = (const float*)c.k + (int64_t)table[t / PAGE] * c.page_stride +
+                              (int64_t)kvh * k_head_elems(HD);
+            float dot = 0.f;
+            for (int d = 0; d < HD; ++d) dot = fmaf(sq[d], kp[k_offset(t % PAGE, d, HD)], dot);
+            s = dot * scale;
+        }
+        const float m_new = fmaxf(m, block_max(s, scratch));
+        const float p = (t <= pos) ? expf(s - m_new) : 0.f;
+        const float alpha = (m == -INFINITY) ? 0.f : expf(m - m_new);
+        __syncthreads();
+        sp[tid] = p;
+        __syncthreads();
+        const int n = min(256, pos - t0 + 1);
+        float psum = 0.f;
+        for (int i = 0; i < n; ++i) psum += sp[i];
+        l = l * alpha + psum;
+        m = m_new;
+        if (tid < HD) {
+            float acc = o * alpha;
+            for (int i = 0; i < n; ++i) {
+                const int tt = t0 + i;
+                const float* vp = (const float*)c.v + (int64_t)table[tt / PAGE] * c.page_stride +
+                                  (int64_t)kvh * v_head_elems(HD);
+                acc = fmaf(sp[i], vp[v_offset(tt % PAGE, tid, HD)], acc);
+            }
+            o = acc;
+        }
+        __syncthreads();
+    }
+    if (tid < HD) out[(tok * H + h) * HD + tid] = o / l;
+}
+
+// ---------------------------------------------------------------------------
+// C interface
+// ---------------------------------------------------------------------------
+extern "C" int li_attn_head_dim() { return HD; }
+
+static int check_heads(int H, int K) { return (H > 0 && K > 0 && H % K == 0) ? LI_OK : LI_BAD_ARG; }
+
+extern "C" int li_attn_prefill(const void* q, void* out, int dt, const void* k, const void* v, int64_t page_stride,
+                               const int* page_table, int max_pages, const int* tile_seq, const int* tile_q0,
+                               int n_tiles, const int* seq_slot, const int* seq_qstart, const int* seq_qlen,
+                               const int* seq_ctx, int H, int K, float scale, int window, hipStream_t stream) {
+    if (check_heads(H, K)) return LI_BAD_ARG;
+    if (n_tiles <= 0) return LI_OK;
+    CachePtrs c{k, v, page_stride, page_table, max_pages};
+    dim3 grid(n_tiles, H), block(256);
+    if (dt == DT_F16)
+        attn_prefill_kernel<f16><<<grid, block, 0, stream>>>((const f16*)q, (f16*)out, c, tile_seq, tile_q0, seq_slot,
+                                                             seq_qstart, seq_qlen, seq_ctx, H, K, scale, window);
+    else if (dt == DT_BF16)
+        attn_prefill_kernel<bf16><<<grid, block, 0, stream>>>((const bf16*)q, (bf16*)out, c, tile_seq, tile_q0,
+                                                              seq_slot, seq_qstart, seq_qlen, seq_ctx, H, K, scale,
+                                                              window);
+    else return LI_BAD_ARG;
+    LI_CHECK_LAUNCH();
+    return LI_OK;
+}
+
+// part_o: [B, H, splits, HD] float32, part_ml: [B, H, splits, 2] float32 (needed when splits > 1)
+extern "C" int li_attn_decode(const void* q, void* out, int dt, const void* k, const void* v, int64_t page_stride,
+                              const int* page_table, int max_pages, const int* seq_slot, const int* seq_ctx,
+                              int n_seqs, int H, int K, float scale, int window, int splits, float* part_o,
+                              float* part_ml, hipStream_t stream) {
+    if (check_heads(H, K) || splits < 1 || (splits > 1 && (!part_o || !part_ml))) return LI_BAD_ARG;
+    if (n_seqs <= 0) return LI_OK;
+    CachePtrs c{k, v, page_stride, page_table, max_pages};
+    const int G = H / K;
+    dim3 grid(n_seqs, K * ((G + 31) / 32), splits), block(64);
+    if (dt == DT_F16) {
+        attn_decode_kernel<f16><<<grid, block, 0, stream>>>((const f16*)q, (f16*)out, part_o, part_ml, c, seq_slot,
+                                                            seq_ctx, H, K, scale, window);
+        LI_CHECK_LAUNCH();
+        if (splits > 1) attn_merge_kernel<f16><<<n_seqs * H, 64, 0, stream>>>(part_o, part_ml, (f16*)out, splits);
+    } else if (dt == DT_BF16) {
+        attn_decode_kernel<bf16><<<grid, block, 0, stream>>>((const bf16*)q, (bf16*)out, part_o, part_ml, c,
+                                                             seq_slot, seq_ctx, H, K, scale, window);
+        LI_CHECK_LAUNCH();
+        if (splits > 1) attn_merge_kernel<bf16><<<n_seqs * H, 64, 0, stream>>>(part_o, part_ml, (bf16*)out, splits);
+    } else return LI_BAD_ARG;
+    LI_CHECK_LAUNCH();
+    return LI_OK;
+}
+
+extern "C" int li_attn_f32(const float* q, float* out, const void* k, const void* v, int64_t page_stride,
+                           const int* page_table, int max_pages, const int* pos, const int* tok_slot,
+                           int n_tokens, int H, int K, float scale, int window, hipStream_t stream) {
+    if (check_heads(H, K)) return LI_BAD_ARG;
+    if (n_tokens <= 0) return LI_OK;
+    CachePtrs c{k, v, page_stride, page_table, max_pages};
+    dim3 grid(n_tokens, H), block(256);
+    attn_f32_kernel<<<grid, block, 0, stream>>>(q, out, c, pos, tok_slot, H, K, scale, window);
+    LI_CHECK_LAUNCH();
+    return LI_OK;
+}

@@ -1,0 +1,183 @@
+// Embedding gather, RMSNorm, rotation of q/k with the write into the paged
+// cache, and the per-step bookkeeping kernel of decoding.  One kernel for each,
+// every size taken at run time.
+#include "common.h"
+
+// ---------------------------------------------------------------------------
+// x[t, :] = float(table[token[t], :])          (src/model/model.cpp:101-118)
+// ---------------------------------------------------------------------------
+template <class T>
+__global__ void embed_kernel(const T* __restrict__ table, const int* __restrict__ tokens,
+                             float* __restrict__ x, int d, int vocab) {
+    const int t = blockIdx.x;
+    int tok = tokens[t];
+    tok = tok < 0 ? 0 : (tok >= vocab ? vocab - 1 : tok);   // ids are checked on the host; never read outside
+    const T* row = table + (int64_t)tok * d;
+    float* out = x + (int64_t)t * d;
+    for (int i = threadIdx.x; i < d; i += blockDim.x) out[i] = to_f32(row[i]);
+}
+
+extern "C" int li_embed(const void* table, int table_dt, const int* tokens, float* x,
+                        int n_tokens, int d, int vocab, hipStream_t stream) {
+    if (n_tokens <= 0) return LI_OK;
+    if (d <= 0 || vocab <= 0) return LI_BAD_ARG;
+    dim3 grid(n_tokens), block(256);
+    if (table_dt == DT_F32) embed_kernel<float><<<grid, block, 0, stream>>>((const float*)table, tokens, x, d, vocab);
+    else if (table_dt == DT_F16) embed_kernel<f16><<<grid, block, 0, stream>>>((const f16*)table, tokens, x, d, vocab);
+    else if (table_dt == DT_BF16) embed_kernel<bf16><<<grid, block, 0, stream>>>((const bf16*)table, tokens, x, d, vocab);
+    else return LI_BAD_ARG;
+    LI_CHECK_LAUNCH();
+    return LI_OK;
+}
+
+// ---------------------------------------------------------------------------
+// out[r, :] = x[row(r), :] / sqrt(mean(x^2) + eps) * w     (include/kernels_cpu.hpp:43-54)
+// Sum of squares, root and scaling in float32; `rows` (may be null) picks rows.
+// ---------------------------------------------------------------------------
+template <class TO>
+__global__ void rmsnorm_kernel(const float* __restrict__ x, const float* __restrict__ w,
+                               const int* __restrict__ rows, TO* __restrict__ out, int d, float eps) {
+    __shared__ float scratch[16];
+    const int r = blockIdx.x;
+    const float* xr = x + (int64_t)(rows ? rows[r] : r) * d;
+    TO* o = out + (int64_t)r * d;
+    float ss = 0.f;
+    for (int i = threadIdx.x; i < d; i += blockDim.x) { const float v = xr[i]; ss += v * v; }
+    ss = block_sum(ss, scratch);
+    const float rms = sqrtf(ss / (float)d + eps);
+    for (int i = threadIdx.x; i < d; i += blockDim.x) o[i] = from_f32<TO>(xr[i] / rms * w[i]);
+}
+
+extern "C" int li_rmsnorm(const float* x, const float* w, const int* rows, void* out, int out_dt,
+                          int n_rows, int d, float eps, hipStream_t stream) {
+    if (n_rows <= 0) return LI_OK;
+    if (d <= 0) return LI_BAD_ARG;
+    dim3 grid(n_rows), block(d >= 2048 ? 512 : (d >= 512 ? 256 : 64));
+    if (out_dt == DT_F32) rmsnorm_kernel<float><<<grid, block, 0, stream>>>(x, w, rows, (float*)out, d, eps);
+    else if (out_dt == DT_F16) rmsnorm_kernel<f16><<<grid, block, 0, stream>>>(x, w, rows, (f16*)out, d, eps);
+    else if (out_dt == DT_BF16) rmsnorm_kernel<bf16><<<grid, block, 0, stream>>>(x, w, rows, (bf16*)out, d, eps);
+    else return LI_BAD_ARG;
+    LI_CHECK_LAUNCH();
+    return LI_OK;
+}
+
+// ---------------------------------------------------------------------------
+// Rotation of q and k by position, and the write of k and v into the cache.
+//   qkv   [T, row_stride] float32: q heads, then k heads, then v heads of one token
+//   q_out [T, H, hd]
+//   pages: k_pages/v_pages of this layer, page = page_table[slot, pos / PAGE]
+// Rotation (include/kernels_cpu.hpp:82-100): pair (a, b) <- (a cos - b sin, a sin + b cos),
+// angle = pos * inv_freq[j]; adjacent pairing rotates (2j, 2j+1), half pairing
+// (j, j + rotary_dim/2).  Dimensions at and beyond rotary_dim pass unchanged.
+// Keys are stored after the rotation (src/model/block.cpp:141-148).
+// ---------------------------------------------------------------------------
+template <class T>
+__global__ void rope_store_kernel(const float* __restrict__ qkv, int row_stride,
+                                  const float* __restrict__ inv_freq, int rotary_dim, int half_pairing,
+                                  const int* __restrict__ pos, const int* __restrict__ tok_slot,
+                                  const int* __restrict__ page_table, int max_pages,
+                                  T* __restrict__ q_out, T* __restrict__ k_pages, T* __restrict__ v_pages,
+                                  int H, int K, int hd) {
+    const int t = blockIdx.x;
+    const int p = pos[t];
+    const int half = hd >> 1;
+    const int n_pairs = (H + 2 * K) * half;
+    const float* row = qkv + (int64_t)t * row_stride;
+    int64_t page = 0;
+    if (K > 0) page = page_table[(int64_t)tok_slot[t] * max_pages + p / PAGE];
+    const int tp = p % PAGE;
+    for (int i = threadIdx.x; i < n_pairs; i += blockDim.x) {
+        const int head = i / half, j = i - head * half;
+        int d0, d1;
+        bool rotate = false;
+        if (2 * j < rotary_dim) {
+            rotate = true;
+            if (half_pairing) { d0 = j; d1 = j + (rotary_dim >> 1); }
+            else { d0 = 2 * j; d1 = 2 * j + 1; }
+        } else { d0 = 2 * j; d1 = 2 * j + 1; }
+        float a = row[head * hd + d0], b = row[head * hd + d1];
+        if (rotate && head < H + K) {
+            float s, c;
+            sincosf((float)p * inv_freq[j], &s, &c);
+            const float ra = a * c - b * s, rb = a * s + b * c;
+            a = ra; b = rb;
+        }
+        if (head < H) {
+            T* q = q_out + ((int64_t)t * H + head) * hd;
+            q[d0] = from_f32<T>(a); q[d1] = from_f32<T>(b);
+        } else if (head < H + K) {
+            T* kp = k_pages + (page * K + (head - H)) * k_head_elems(hd);
+            kp[k_offset(tp, d0, hd)] = from_f32<T>(a); kp[k_offset(tp, d1, hd)] = from_f32<T>(b);
+        } else {
+            T* vp = v_pages + (page * K + (head - H - K)) * v_head_elems(hd);
+            vp[v_offset(tp, d0, hd)] = from_f32<T>(a); vp[v_offset(tp, d1, hd)] = from_f32<T>(b);
+        }
+    }
+}
+
+extern "C" int li_rope_store(const float* qkv, int row_stride, const float* inv_freq, int rotary_dim,
+                             int half_pairing, const int* pos, const int* tok_slot, const int* page_table,
+                             int max_pages, void* q_out, void* k_pages, void* v_pages, int dt,
+                             int n_tokens, int H, int K, int hd, hipStream_t stream) {
+    if (n_tokens <= 0) return LI_OK;
+    if (hd <= 0 || (hd & 1) || H <= 0 || K < 0 || rotary_dim < 0 || rotary_dim > hd || (rotary_dim & 1) ||
+        row_stride < (H + 2 * K) * hd)
+        return LI_BAD_ARG;
+    if (K > 0 && (hd % 16 != 0)) return LI_UNSUPPORTED;
+    dim3 grid(n_tokens), block(256);
+#define LAUNCH(T)                                                                                        \
+    rope_store_kernel<T><<<grid, block, 0, stream>>>(qkv, row_stride, inv_freq, rotary_dim, half_pairing, \
+                                                     pos, tok_slot, page_table, max_pages, (T*)q_out,    \
+                                                     (T*)k_pages, (T*)v_pages, H, K, hd)
+    if (dt == DT_F32) LAUNCH(float);
+    else if (dt == DT_F16) LAUNCH(f16);
+    else if (dt == DT_BF16) LAUNCH(bf16);
+    else return LI_BAD_ARG;
+#undef LAUNCH
+    LI_CHECK_LAUNCH();
+    return LI_OK;
+}
+
+// ---------------------------------------------------------------------------
+// Bookkeeping of one decode step, on the device so that a captured step can be
+// replayed: each sequence's new token gets the position lens[slot], the
+// sequence's context grows by one.
+// ---------------------------------------------------------------------------
+__global__ void decode_prepare_kernel(const int* __restrict__ seq_slot, int* __restrict__ lens,
+                                      int* __restrict__ pos, int* __restrict__ ctx, int n) {
+    const int i = blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= n) return;
+    const int s = seq_slot[i];
+    const int l = lens[s];
+    pos[i] = l;
+    ctx[i] = l + 1;
+    lens[s] = l + 1;
+}
+
+extern "C" int li_decode_prepare(const int* seq_slot, int* lens, int* pos, int* ctx, int n, hipStream_t stream) {
+    if (n <= 0) return LI_OK;
+    decode_prepare_kernel<<<(n + 255) / 256, 256, 0, stream>>>(seq_slot, lens, pos, ctx, n);
+    LI_CHECK_LAUNCH();
+    return LI_OK;
+}
+
+// out[i] = silu(gate[i]) * up[i] for separate gate and up rows:  gu [T, 2F] float32 with
+// gate_j at column 2j and up_j at column 2j+1  ->  h [T, F].  (src/model/block.cpp:209-213)
+template <class T>
+__global__ void swiglu_kernel(const float* __restrict__ gu, T* __restrict__ h, int64_t n) {
+    const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= n) return;
+    const float g = gu[2 * i], u = gu[2 * i + 1];
+    h[i] = from_f32<T>(g / (1.f + expf(-g)) * u);
+}
+
+extern "C" int li_swiglu(const float* gu, void* h, int dt, int64_t n, hipStream_t stream) {
+    if (n <= 0) return LI_OK;
+    dim3 grid((unsigned)((n + 255) / 256)), block(256);
+    if (dt == DT_F32) swiglu_kernel<float><<<grid, block, 0, stream>>>(gu, (float*)h, n);
+    else if (dt == DT_F16) swiglu_kernel<f16><<<grid, block, 0, stream>>>(gu, (f16*)h, n);
+    else if (dt == DT_BF16) swiglu_kernel<bf16><<<grid, block, 0, stream>>>(gu, (bf16*)h, n);
+    else return LI_BAD_ARG;
+    LI_CHECK_LAUNCH();
+    return LI_OK;
+}

@@ -1,0 +1,388 @@
+// Matrix products  C[M, N] = X[M, K] . W[N, K]^T  (both operands contiguous in K,
+// the layout of the reference's matmul, include/kernels_cpu.hpp:69-80), with the
+// epilogue fused: plain store, add into the float32 residual, or SwiGLU on
+// interleaved gate/up columns.
+//
+//   gemm_fma   any element types and any sizes; float32 multiply-add in ascending k
+//              for every output, so an output does not depend on its place in the batch.
+//              It is the true 32-bit path and the fallback for K not a multiple of 8.
+//   gemm_mfma  16-bit operands on the matrix cores (32x32x16), tiles staged through
+//              LDS, optional split over K into a float32 workspace.
+//   gemv       16-bit operands, up to 8 rows of X: W is streamed once with 16-byte
+//              loads, X sits in LDS, v_dot2 accumulates in float32.
+#include "common.h"
+
+enum { EPI_STORE = 0, EPI_ADD = 1, EPI_SWIGLU = 2 };
+
+struct Epilogue {
+    void* C;        // output
+    int mode;       // EPI_*
+    int out_dt;     // DT_* of C (EPI_ADD: always float32)
+    int M, N;
+};
+
+__device__ __forceinline__ void store_one(void* C, int dt, int64_t i, float v) {
+    if (dt == DT_F32) ((float*)C)[i] = v;
+    else if (dt == DT_F16) ((f16*)C)[i] = (f16)v;
+    else ((bf16*)C)[i] = (bf16)v;
+}
+
+// v[0..3] are the results for row m and columns n..n+3 (n a multiple of 4).
+__device__ __forceinline__ void epilogue4(const Epilogue& e, int m, int n, const float* v) {
+    if (m >= e.M || n >= e.N) return;
+    if (e.mode == EPI_SWIGLU) {
+        // columns 2j (gate) and 2j+1 (up) give h[m, j] = silu(gate) * up   (src/model/block.cpp:209-213)
+        const int64_t row = (int64_t)m * (e.N >> 1);
+#pragma unroll
+        for (int j = 0; j < 4; j += 2) {
+            if (n + j + 1 < e.N) {
+                const float g = v[j], u = v[j + 1];
+                store_one(e.C, e.out_dt, row + ((n + j) >> 1), g / (1.f + expf(-g)) * u);
+            }
+        }
+        return;
+    }
+    const int64_t base = (int64_t)m * e.N + n;
+    const bool full = (n + 3 < e.N) && ((e.N & 3) == 0);
+    if (e.mode == EPI_ADD) {
+        float* c = (float*)e.C + base;
+        if (full) {
+            f32x4 o = *(f32x4*)c;
+            o[0] += v[0]; o[1] += v[1]; o[2] += v[2]; o[3] += v[3];
+            *(f32x4*)c = o;
+        } else {
+#pragma unroll
+            for (int j = 0; j < 4; ++j) if (n + j < e.N) c[j] += v[j];
+        }
+        return;
+    }
+    if (full && e.out_dt == DT_F32) {
+        f32x4 o = {v[0], v[1], v[2], v[3]};
+        *(f32x4*)((float*)e.C + base) = o;
+    } else if (full && e.out_dt == DT_F16) {
+        f16x4 o = {(f16)v[0], (f16)v[1], (f16)v[2], (f16)v[3]};
+        *(f16x4*)((f16*)e.C + base) = o;
+    } else if (full && e.out_dt == DT_BF16) {
+        bf16x4 o = {(bf16)v[0], (bf16)v[1], (bf16)v[2], (bf16)v[3]};
+        *(bf16x4*)((bf16*)e.C + base) = o;
+    } else {
+#pragma unroll
+        for (int j = 0; j < 4; ++j) if (n + j < e.N) store_one(e.C, e.out_dt, base + j, v[j]);
+    }
+}
+
+// ===========================================================================
+// gemm_fma: 64x64 tile, 256 threads, 4x4 outputs a thread, k ascending.
+// ===========================================================================
+template <class TX, class TW>
+__global__ __launch_bounds__(256) void gemm_fma_kernel(const TX* __restrict__ X, const TW* __restrict__ W,
+                                                       int K, Epilogue e) {
+    constexpr int BT = 64, BK = 16;
+    __shared__ float sX[BK][BT + 4];
+    __shared__ float sW[BK][BT + 4];
+    const int tid = threadIdx.x;
+    const int tx = tid & 15, ty = tid >> 4;
+    const int m0 = blockIdx.y * BT, n0 = blockIdx.x * BT;
+    float acc[4][4] = {};
+    const int lr = tid >> 2, lk = (tid & 3) * 4;     // row of the tile and first k this thread loads
+    for (int k0 = 0; k0 < K; k0 += BK) {
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            const int k = k0 + lk + j;
+            const int m = m0 + lr, n = n0 + lr;
+            sX[lk + j][lr] = (m < e.M && k < K) ? to_f32(X[(int64_t)m * K + k]) : 0.f;
+            sW[lk + j][lr] = (n < e.N && k < K) ? to_f32(W[(int64_t)n * K + k]) : 0.f;
+        }
+        __syncthreads();
+#pragma unroll
+        for (int k = 0; k < BK; ++k) {
+            float a[4], b[4];
+#pragma unroll
+            for (int i = 0; i < 4; ++i) { a[i] = sX[k][ty * 4 + i]; b[i] = sW[k][tx * 4 + i]; }
+#pragma unroll
+            for (int i = 0; i < 4; ++i)
+#pragma unroll
+                for (int j = 0; j < 4; ++j) acc[i][j] = fmaf(a[i], b[j], acc[i][j]);
+        }
+        __syncthreads();
+    }
+#pragma unroll
+    for (int i = 0; i < 4; ++i) epilogue4(e, m0 + ty * 4 + i, n0 + tx * 4, acc[i]);
+}
+
+// ===========================================================================
+// gemm_mfma: BN rows of W x BM rows of X per workgroup of 4 waves, BK = 64.
+// W is operand A of the matrix instruction (its rows are the instruction's rows),
+// X operand B, so that a lane ends with 4 consecutive columns n of one row m:
+// accumulator r of a 32x32 block is n = 8*(r/4) + 4*(lane/32) + r%4, m = lane%32.
+// ===========================================================================
+template <class T, int BN, int BM, int WN, int WM>
+__global__ __launch_bounds__(256) void gemm_mfma_kernel(const T* __restrict__ X, const T* __restrict__ W,
+                                                        int K, int k_per_split, float* __restrict__ ws,
+                                                        Epilogue e) {
+    typedef typename Vec<T>::v8 v8;
+    constexpr int BK = 64, LD = BK + 8;
+    constexpr int TN = BN / WN, TM = BM / WM;            // wave tile
+    constexpr int NB = TN / 32, MB = TM / 32;            // 32x32 blocks of a wave
+    constexpr int W_CHUNKS = BN * BK / 8 / 256, X_CHUNKS = BM * BK / 8 / 256;
+    static_assert(WN * WM == 4 && TN % 32 == 0 && TM % 32 == 0, "tile");
+    static_assert(W_CHUNKS >= 1 && X_CHUNKS >= 1, "tile too small for 256 threads");
+    __shared__ __attribute__((aligned(16))) T sW[BN * LD];
+    __shared__ __attribute__((aligned(16))) T sX[BM * LD];
+
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int wn = wave % WN, wm = wave / WN;
+    const int n0 = blockIdx.x * BN, m0 = blockIdx.y * BM;
+    const int k_begin = blockIdx.z * k_per_split;
+    const int k_end = min(K, k_begin + k_per_split);
+
+    f32x16 acc[NB][MB];
+#pragma unroll
+    for (int a = 0; a < NB; ++a)
+#pragma unroll
+        for (int b = 0; b < MB; ++b)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) acc[a][b][r] = 0.f;
+
+    v8 rw[W_CHUNKS], rx[X_CHUNKS];
+    auto load_tile = [&](int k0) {
+#pragma unroll
+        for (int c = 0; c < W_CHUNKS; ++c) {
+            const int chunk = tid + c * 256, row = chunk >> 3, kc = (chunk & 7) * 8;
+            const int n = n0 + row, k = k0 + kc;
+            v8 z = {};
+            rw[c] = (n < e.N && k < k_end) ? *(const v8*)(W + (int64_t)n * K + k) : z;
+        }
+#pragma unroll
+        for (int c = 0; c < X_CHUNKS; ++c) {
+            const int chunk = tid + c * 256, row = chunk >> 3, kc = (chunk & 7) * 8;
+            const int m = m0 + row, k = k0 + kc;
+            v8 z = {};
+            rx[c] = (m < e.M && k < k_end) ? *(const v8*)(X + (int64_t)m * K + k) : z;
+        }
+    };
+    auto store_tile = [&]() {
+#pragma unroll
+        for (int c = 0; c < W_CHUNKS; ++c) {
+            const int chunk = tid + c * 256, row = chunk >> 3, kc = (chunk & 7) * 8;
+            *(v8*)(sW + row * LD + kc) = rw[c];
+        }
+#pragma unroll
+        for (int c = 0; c < X_CHUNKS; ++c) {
+            const int chunk = tid + c * 256, row = chunk >> 3, kc = (chunk & 7) * 8;
+            *(v8*)(sX + row * LD + kc) = rx[c];
+        }
+    };
+
+    if (k_begin < k_end) {
+        load_tile(k_begin);
+        store_tile();
+        __syncthreads();
+        for (int k0 = k_begin; k0 < k_end; k0 += BK) {
+            const bool more = k0 + BK < k_end;
+            if (more) load_tile(k0 + BK);
+#pragma unroll
+            for (int ks = 0; ks < BK; ks += 16) {
+                v8 a[NB], b[MB];
+                const int kk = ks + 8 * (lane >> 5);
+#pragma unroll
+                for (int i = 0; i < NB; ++i) a[i] = *(const v8*)(sW + (wn * TN + i * 32 + (lane & 31)) * LD + kk);
+#pragma unroll
+                for (int j = 0; j < MB; ++j) b[j] = *(const v8*)(sX + (wm * TM + j * 32 + (lane & 31)) * LD + kk);
+#pragma unroll
+                for (int i = 0; i < NB; ++i)
+#pragma unroll
+                    for (int j = 0; j < MB; ++j) acc[i][j] = mfma32(a[i], b[j], acc[i][j]);
+            }
+            __syncthreads();
+            if (more) { store_tile(); __syncthreads(); }
+        }
+    }
+
+    const bool split = gridDim.z > 1;
+#pragma unroll
+    for (int i = 0; i < NB; ++i)
+#pragma unroll
+        for (int j = 0; j < MB; ++j) {
+            const int m = m0 + wm * TM + j * 32 + (lane & 31);
+#pragma unroll
+            for (int g = 0; g < 4; ++g) {
+                const int n = n0 + wn * TN + i * 32 + 8 * g + 4 * (lane >> 5);
+                float v[4] = {acc[i][j][4 * g], acc[i][j][4 * g + 1], acc[i][j][4 * g + 2], acc[i][j][4 * g + 3]};
+                if (!split) epilogue4(e, m, n, v);
+                else if (m < e.M) {
+                    float* p = ws + ((int64_t)blockIdx.z * e.M + m) * e.N + n;
+#pragma unroll
+                    for (int q = 0; q < 4; ++q) if (n + q < e.N) p[q] = v[q];
+                }
+            }
+        }
+}
+
+// Sum of the split-K partials in ascending split order, then the epilogue.
+__global__ void splitk_reduce_kernel(const float* __restrict__ ws, int splits, Epilogue e) {
+    const int64_t quads_per_row = (e.N + 3) >> 2;
+    const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= quads_per_row * e.M) return;
+    const int m = (int)(i / quads_per_row), n = (int)(i % quads_per_row) * 4;
+    float v[4] = {0.f, 0.f, 0.f, 0.f};
+    for (int s = 0; s < splits; ++s) {
+        const float* p = ws + ((int64_t)s * e.M + m) * e.N + n;
+#pragma unroll
+        for (int q = 0; q < 4; ++q) if (n + q < e.N) v[q] += p[q];
+    }
+    epilogue4(e, m, n, v);
+}
+
+// ===========================================================================
+// gemv: MB <= 8 rows of X against R rows of W per wave.
+// ===========================================================================
+template <class T, int MB, int R>
+__global__ __launch_bounds__(256) void gemv_kernel(const T* __restrict__ X, const T* __restrict__ W,
+                                                   int K, Epilogue e) {
+    typedef typename Vec<T>::v8 v8;
+    typedef typename Vec<T>::v2 v2;
+    constexpr int KC = 2048;                             // elements of K staged at a time
+    __shared__ __attribute__((aligned(16))) T sx[MB * KC];
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int n_base = (blockIdx.x * 4 + wave) * R;
+    float acc[R][MB];
+#pragma unroll
+    for (int r = 0; r < R; ++r)
+#pragma unroll
+        for (int m = 0; m < MB; ++m) acc[r][m] = 0.f;
+    const T* wrow[R];
+#pragma unroll
+    for (int r = 0; r < R; ++r) wrow[r] = W + (int64_t)min(n_base + r, e.N - 1) * K;
+
+    for (int kc = 0; kc < K; kc += KC) {
+        const int len = min(KC, K - kc);                 // a multiple of 8
+        __syncthreads();
+        for (int c = tid; c < MB * (KC / 8); c += 256) {
+            const int m = c / (KC / 8), k = (c % (KC / 8)) * 8;
+            v8 z = {};
+            *(v8*)(sx + m * KC + k) = (m < e.M && k < len) ? *(const v8*)(X + (int64_t)m * K + kc + k) : z;
+        }
+        __syncthreads();
+        for (int k = lane * 8; k < len; k += 64 * 8) {
+            v8 w[R];
+#pragma unroll
+            for (int r = 0; r < R; ++r) w[r] = *(const v8*)(wrow[r] + kc + k);
+#pragma unroll
+            for (int m = 0; m < MB; ++m) {
+                const v8 xv = *(const v8*)(sx + m * KC + k);
+#pragma unroll
+                for (int r = 0; r < R; ++r)
+#pragma unroll
+                    for (int p = 0; p < 4; ++p) {
+                        v2 a = {w[r][2 * p], w[r][2 * p + 1]};
+                        v2 b = {xv[2 * p], xv[2 * p + 1]};
+                        acc[r][m] = dot2(a, b, acc[r][m]);
+                    }
+            }
+        }
+    }
+#pragma unroll
+    for (int m = 0; m < MB; ++m) {
+        float v[R];
+#pragma unroll
+        for (int r = 0; r < R; ++r) v[r] = wave_sum(acc[r][m]);
+        if (lane == 0) {
+#pragma unroll
+            for (int r = 0; r < R; r += 4) epilogue4(e, m, n_base + r, v + r);
+        }
+    }
+}
+
+// ===========================================================================
+// C interface
+// ===========================================================================
+static int check_common(const void* X, const void* W, const void* C, int M, int N, int K, int mode, int out_dt) {
+    if (!X || !W || !C || M < 0 || N <= 0 || K <= 0) return LI_BAD_ARG;
+    if (mode < EPI_STORE || mode > EPI_SWIGLU) return LI_BAD_ARG;
+    if (out_dt < DT_F32 || out_dt > DT_BF16) return LI_BAD_ARG;
+    if (mode == EPI_ADD && out_dt != DT_F32) return LI_BAD_ARG;
+    if (mode == EPI_SWIGLU && (N & 1)) return LI_BAD_ARG;
+    return LI_OK;
+}
+
+extern "C" int li_gemm_fma(const void* X, int x_dt, const void* W, int w_dt, void* C, int out_dt, int mode,
+                           int M, int N, int K, hipStream_t stream) {
+    int rc = check_common(X, W, C, M, N, K, mode, out_dt);
+    if (rc) return rc;
+    if (M == 0) return LI_OK;
+    Epilogue e{C, mode, out_dt, M, N};
+    dim3 grid((N + 63) / 64, (M + 63) / 64), block(256);
+#define CASE(xd, TX, wd, TW)                                                                       \
+    if (x_dt == xd && w_dt == wd) {                                                                \
+        gemm_fma_kernel<TX, TW><<<grid, block, 0, stream>>>((const TX*)X, (const TW*)W, K, e);     \
+        LI_CHECK_LAUNCH();                                                                         \
+        return LI_OK;                                                                              \
+    }
+    CASE(DT_F32, float, DT_F32, float)
+    CASE(DT_F16, f16, DT_F16, f16)
+    CASE(DT_BF16, bf16, DT_BF16, bf16)
+    CASE(DT_F32, float, DT_F16, f16)
+    CASE(DT_F32, float, DT_BF16, bf16)
+    CASE(DT_F16, f16, DT_F32, float)
+    CASE(DT_BF16, bf16, DT_F32, float)
+#undef CASE
+    return LI_UNSUPPORTED;
+}
+
+// tile: 0 = 128x128 (W rows x X rows), 1 = 128x64, 2 = 128x32.  splits > 1 needs ws of
+// splits*M*N floats.
+extern "C" int li_gemm_mfma(const void* X, const void* W, int dt, void* C, int out_dt, int mode,
+                            int M, int N, int K, int tile, int splits, float* ws, hipStream_t stream) {
+    int rc = check_common(X, W, C, M, N, K, mode, out_dt);
+    if (rc) return rc;
+    if (dt != DT_F16 && dt != DT_BF16) return LI_BAD_ARG;
+    if (K % 8 != 0 || ((uintptr_t)X & 15) || ((uintptr_t)W & 15)) return LI_UNSUPPORTED;
+    if (splits < 1 || (splits > 1 && !ws)) return LI_BAD_ARG;
+    if (M == 0) return LI_OK;
+    Epilogue e{C, mode, out_dt, M, N};
+    int k_per_split = ((K + splits - 1) / splits + 63) / 64 * 64;
+    splits = (K + k_per_split - 1) / k_per_split;
+    const int bm = tile == 0 ? 128 : (tile == 1 ? 64 : 32);
+    dim3 grid((N + 127) / 128, (M + bm - 1) / bm, splits), block(256);
+#define LAUNCH(T)                                                                                              \
+    do {                                                                                                       \
+        if (tile == 0) gemm_mfma_kernel<T, 128, 128, 2, 2><<<grid, block, 0, stream>>>((const T*)X, (const T*)W, K, k_per_split, ws, e); \
+        else if (tile == 1) gemm_mfma_kernel<T, 128, 64, 2, 2><<<grid, block, 0, stream>>>((const T*)X, (const T*)W, K, k_per_split, ws, e); \
+        else if (tile == 2) gemm_mfma_kernel<T, 128, 32, 4, 1><<<grid, block, 0, stream>>>((const T*)X, (const T*)W, K, k_per_split, ws, e); \
+        else return LI_BAD_ARG;                                                                                \
+    } while (0)
+    if (dt == DT_F16) LAUNCH(f16); else LAUNCH(bf16);
+#undef LAUNCH
+    LI_CHECK_LAUNCH();
+    if (splits > 1) {
+        const int64_t quads = (int64_t)M * ((N + 3) / 4);
+        splitk_reduce_kernel<<<(unsigned)((quads + 255) / 256), 256, 0, stream>>>(ws, splits, e);
+        LI_CHECK_LAUNCH();
+    }
+    return LI_OK;
+}
+
+extern "C" int li_gemv(const void* X, const void* W, int dt, void* C, int out_dt, int mode,
+                       int M, int N, int K, hipStream_t stream) {
+    int rc = check_common(X, W, C, M, N, K, mode, out_dt);
+    if (rc) return rc;
+    if (dt != DT_F16 && dt != DT_BF16) return LI_BAD_ARG;
+    if (M > 8) return LI_BAD_ARG;
+    if (K % 8 != 0 || ((uintptr_t)X & 15) || ((uintptr_t)W & 15)) return LI_UNSUPPORTED;
+    if (M == 0) return LI_OK;
+    Epilogue e{C, mode, out_dt, M, N};
+    constexpr int R = 4;
+    dim3 grid((N + 4 * R - 1) / (4 * R)), block(256);
+#define LAUNCH(T)                                                                                    \
+    do {                                                                                             \
+        if (M == 1) gemv_kernel<T, 1, R><<<grid, block, 0, stream>>>((const T*)X, (const T*)W, K, e); \
+        else if (M == 2) gemv_kernel<T, 2, R><<<grid, block, 0, stream>>>((const T*)X, (const T*)W, K, e); \
+        else if (M <= 4) gemv_kernel<T, 4, R><<<grid, block, 0, stream>>>((const T*)X, (const T*)W, K, e); \
+        else gemv_kernel<T, 8, R><<<grid, block, 0, stream>>>((const T*)X, (const T*)W, K, e);       \
+    } while (0)
+    if (dt == DT_F16) LAUNCH(f16); else LAUNCH(bf16);
+#undef LAUNCH
+    LI_CHECK_LAUNCH();
+    return LI_OK;
+}

@@ -1,0 +1,111 @@
+"""The engine: a model, its cache, and the one step function."""
+from __future__ import annotations
+
+import torch
+
+from ..cache import Cache, CacheError
+from ..registry import config_from_folder
+from ..weights import load_into, place_tensor, random_tensors
+from .model import DecoderModel
+from .step import StepContext
+
+_DTYPES = {"bfloat16": torch.bfloat16, "float16": torch.float16, "float32": torch.float32,
+           "bf16": torch.bfloat16, "fp16": torch.float16, "fp32": torch.float32}
+
+
+def as_dtype(d):
+    if isinstance(d, torch.dtype):
+        return d
+    if d not in _DTYPES:
+        raise ValueError(f"dtype {d!r}: one of bfloat16, float16, float32")
+    return _DTYPES[d]
+
+
+def _require_gpu():
+    if not torch.cuda.is_available():
+        raise RuntimeError("llm_infer_amd runs on an MI355X through its HIP kernels; no GPU is visible "
+                           "and there is no CPU implementation")
+
+
+class Engine:
+    """``step`` runs a batch of sequences that started together: their prompts in one step, then
+    one token each.  It runs only the tokens it is given, against what earlier steps left in
+    the cache, and returns the logits at the wanted places."""
+
+    def __init__(self, config, model: DecoderModel, max_tokens: int, n_slots: int | None = None):
+        self.config, self.model = config, model
+        self.dtype, self.device = model.dtype, model.device
+        self.max_positions = model.spec.max_positions
+        self.vocab_size = model.spec.vocab_size
+        self.cache = Cache(model.cache_specs(), max_tokens, self.max_positions, model.dtype, model.device, n_slots)
+        self._graphs = {}
+        self._graph_bufs = None
+
+    # -- construction ----------------------------------------------------------
+    @classmethod
+    def from_folder(cls, folder: str, dtype="bfloat16", max_tokens: int = 8192, n_slots=None, device="cuda"):
+        _require_gpu()
+        config = config_from_folder(folder)
+        model = DecoderModel(config.model_spec(), as_dtype(dtype), device)
+        load_into(model, folder)
+        return cls(config, model, max_tokens, n_slots)
+
+    @classmethod
+    def from_random(cls, config, seed: int = 0, dtype="bfloat16", max_tokens: int = 8192, n_slots=None,
+                    device="cuda", stored_dtype=None):
+        """Random weights made on the device (no folder): matrices as ``stored_dtype`` would store them."""
+        _require_gpu()
+        dt = as_dtype(dtype)
+        model = DecoderModel(config.model_spec(), dt, device)
+        stored = as_dtype(stored_dtype) if stored_dtype else (dt if dt != torch.float32 else torch.bfloat16)
+        params = model.params()
+        tensors = {}
+        for name, spec in params.items():
+            t = random_tensors({name: spec}, seed, stored, device)[name]
+            tensors[name] = place_tensor(t, spec.kind, dt, device)
+        model.bind(tensors)
+        return cls(config, model, max_tokens, n_slots)
+
+    # -- sequences -----------------------------------------------------------------
+    def alloc_slot(self) -> int:
+        return self.cache.alloc_slot()
+
+    def free_slot(self, slot: int) -> None:
+        self.cache.free_slot(slot)
+
+    def length(self, slot: int) -> int:
+        return self.cache.lens[slot]
+
+    def decode_runner(self, sampler, use_graph: bool = True):
+        from .decode import GraphDecodeRunner, PlainDecodeRunner
+        return GraphDecodeRunner(self, sampler) if use_graph else PlainDecodeRunner(self, sampler)
+
+    def generate(self, prompts, **kw):
+        from .generate import generate
+        return generate(self, prompts, **kw)
+
+    # -- the step ----------------------------------------------------------------------
+    def step(self, slots, tokens, want=None) -> torch.Tensor:
+        """slots[i]: a held slot; tokens[i]: that sequence's next tokens (at least one);
+        want[i]: places among these tokens whose logits are returned (default: the last).
+        Returns float32 [sum(len(want[i])), vocab] in the order of the sequences and of want."""
+        ctx = self.prepare(slots, tokens, want)
+        logits = self.model.forward(ctx, self.cache)
+        self.cache.trim_windows(slots)
+        return logits
+
+    def prepare(self, slots, tokens, want=None) -> StepContext:
+        if len(slots) != len(tokens) or len(set(slots)) != len(slots):
+            raise ValueError("step: one token list for each slot, each slot once")
+        if want is None:
+            want = [[len(t) - 1] for t in tokens]
+        for s, t, w in zip(slots, tokens, want):
+            if len(t) == 0:
+                raise ValueError(f"step: sequence in slot {s} brings no token")
+            if min(t) < 0 or max(t) >= self.vocab_size:
+                raise ValueError(f"step: token id outside [0, {self.vocab_size}) in slot {s}")
+            if any(not 0 <= i < len(t) for i in w):
+                raise ValueError(f"step: wanted place outside the {len(t)} tokens of slot {s}")
+        before = [self.cache.lens[s] for s in slots]
+        self.cache.grow(slots, [b + len(t) for b, t in zip(before, tokens)])
+        return StepContext(self.device, slots, tokens, before, want)

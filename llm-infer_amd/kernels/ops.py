@@ -1,0 +1,297 @@
+"""Python face of the HIP kernels: argument checks on the host, then one launch
+on torch's current stream.  Every shape that a kernel and its grid assume is
+checked here before the launch; nothing falls back to another implementation.
+"""
+from __future__ import annotations
+
+import ctypes
+from ctypes import c_float, c_int, c_int64, c_uint64, c_void_p
+
+import torch
+
+from . import build
+
+PAGE = 64
+DT = {torch.float32: 0, torch.float16: 1, torch.bfloat16: 2}
+EPI_STORE, EPI_ADD, EPI_SWIGLU = 0, 1, 2
+_STATUS = {1: "bad argument", 2: "unsupported size or alignment", 3: "HIP launch error"}
+
+
+class KernelError(RuntimeError):
+    pass
+
+
+def _ptr(t):
+    return c_void_p(t.data_ptr()) if t is not None else c_void_p(0)
+
+
+def _stream():
+    return c_void_p(torch.cuda.current_stream().cuda_stream)
+
+
+def _check(rc: int, what: str):
+    if rc != 0:
+        raise KernelError(f"{what}: {_STATUS.get(rc, rc)}")
+
+
+def _need(cond: bool, msg: str):
+    if not cond:
+        raise KernelError(msg)
+
+
+def _dev(*tensors):
+    for t in tensors:
+        if t is not None:
+            _need(t.is_cuda, "kernel operands must lie on the GPU")
+            _need(t.is_contiguous(), "kernel operands must be contiguous")
+
+
+_core = None
+
+
+def core():
+    global _core
+    if _core is None:
+        lib = build.core_library()
+        lib.li_uniform01.restype = c_float
+        lib.li_uniform01.argtypes = [c_uint64, c_uint64]
+        _core = lib
+    return _core
+
+
+# ---------------------------------------------------------------------------
+def embed(table: torch.Tensor, tokens: torch.Tensor, out: torch.Tensor | None = None) -> torch.Tensor:
+    """x[t] = float32(table[tokens[t]])"""
+    _dev(table, tokens)
+    _need(tokens.dtype == torch.int32 and tokens.dim() == 1, "tokens: int32 [T]")
+    _need(table.dim() == 2 and table.dtype in DT, "table: [V, d] float")
+    n, (vocab, d) = tokens.numel(), table.shape
+    if out is None:
+        out = torch.empty((n, d), dtype=torch.float32, device=table.device)
+    _need(out.dtype == torch.float32 and out.shape == (n, d), "out: float32 [T, d]")
+    _check(core().li_embed(_ptr(table), DT[table.dtype], _ptr(tokens), _ptr(out), n, d, vocab, _stream()), "embed")
+    return out
+
+
+def rmsnorm(x: torch.Tensor, w: torch.Tensor, eps: float, out_dtype, rows: torch.Tensor | None = None,
+            n_rows: int | None = None) -> torch.Tensor:
+    """out[r] = x[rows[r]] / sqrt(mean(x^2) + eps) * w, float32 inside."""
+    _dev(x, w, rows)
+    _need(x.dtype == torch.float32 and x.dim() == 2, "x: float32 [T, d]")
+    _need(w.dtype == torch.float32 and w.shape == (x.shape[1],), "norm weight: float32 [d]")
+    if rows is not None:
+        _need(rows.dtype == torch.int32, "rows: int32")
+        n = rows.numel() if n_rows is None else n_rows
+    else:
+        n = x.shape[0]
+    out = torch.empty((n, x.shape[1]), dtype=out_dtype, device=x.device)
+    _check(core().li_rmsnorm(_ptr(x), _ptr(w), _ptr(rows), _ptr(out), DT[out_dtype], n, x.shape[1],
+                             c_float(eps), _stream()), "rmsnorm")
+    return out
+
+
+_ws_cache: dict = {}
+
+
+def _workspace(n_floats: int, device) -> torch.Tensor:
+    key = (device, torch.cuda.current_stream().cuda_stream)
+    ws = _ws_cache.get(key)
+    if ws is None or ws.numel() < n_floats:
+        ws = torch.empty(max(n_floats, 1 << 22), dtype=torch.float32, device=device)
+        _ws_cache[key] = ws
+    return ws
+
+
+def linear(x: torch.Tensor, w: torch.Tensor, mode: int = EPI_STORE, out: torch.Tensor | None = None,
+           out_dtype=None, force: str | None = None) -> torch.Tensor:
+    """C = X W^T with the epilogue ``mode``: store, add into ``out`` (float32), or SwiGLU over
+    interleaved gate/up rows of W (C has N/2 columns).  ``force`` picks a kernel for tests."""
+    _dev(x, w, out)
+    _need(x.dim() == 2 and w.dim() == 2 and x.shape[1] == w.shape[1], f"linear: x {tuple(x.shape)} w {tuple(w.shape)}")
+    m, k = x.shape
+    n = w.shape[0]
+    n_out = n // 2 if mode == EPI_SWIGLU else n
+    if mode == EPI_ADD:
+        _need(out is not None and out.dtype == torch.float32, "add epilogue needs a float32 output")
+    if out is None:
+        out = torch.empty((m, n_out), dtype=out_dtype or x.dtype, device=x.device)
+    _need(out.shape == (m, n_out), f"linear: out {tuple(out.shape)}, expected {(m, n_out)}")
+    if mode == EPI_SWIGLU:
+        _need(n % 2 == 0, "SwiGLU epilogue needs an even number of rows of W")
+    if m == 0:
+        return out
+    lib = core()
+    same16 = x.dtype == w.dtype and x.dtype in (torch.float16, torch.bfloat16)
+    fast_ok = same16 and k % 8 == 0 and x.data_ptr() % 16 == 0 and w.data_ptr() % 16 == 0
+    kind = force or ("fma" if not fast_ok else ("gemv" if m <= 8 else "mfma"))
+    if kind == "fma":
+        _check(lib.li_gemm_fma(_ptr(x), DT[x.dtype], _ptr(w), DT[w.dtype], _ptr(out), DT[out.dtype], mode,
+                               m, n, k, _stream()), "gemm_fma")
+    elif kind == "gemv":
+        _need(fast_ok and m <= 8, "gemv: 16-bit operands, K a multiple of 8, at most 8 rows")
+        _check(lib.li_gemv(_ptr(x), _ptr(w), DT[x.dtype], _ptr(out), DT[out.dtype], mode, m, n, k, _stream()), "gemv")
+    else:
+        _need(fast_ok, "gemm_mfma: 16-bit operands and K a multiple of 8")
+        tile = 0 if m > 64 else (1 if m > 32 else 2)
+        bm = (128, 64, 32)[tile]
+        blocks = ((n + 127) // 128) * ((m + bm - 1) // bm)
+        splits = 1
+        if blocks < 256:
+            splits = max(1, min(512 // blocks, k // 256, 16))
+        if kind.startswith("mfma:"):                       # "mfma:<tile>:<splits>" for tests
+            _, t_, s_ = kind.split(":")
+            tile, splits = int(t_), int(s_)
+        ws = _workspace(splits * m * n, x.device) if splits > 1 else None
+        _check(lib.li_gemm_mfma(_ptr(x), _ptr(w), DT[x.dtype], _ptr(out), DT[out.dtype], mode, m, n, k,
+                                tile, splits, _ptr(ws), _stream()), "gemm_mfma")
+    return out
+
+
+def swiglu(gu: torch.Tensor, out_dtype) -> torch.Tensor:
+    """h[:, j] = silu(gu[:, 2j]) * gu[:, 2j+1] for float32 gu."""
+    _dev(gu)
+    _need(gu.dtype == torch.float32 and gu.dim() == 2 and gu.shape[1] % 2 == 0, "gu: float32 [T, 2F]")
+    h = torch.empty((gu.shape[0], gu.shape[1] // 2), dtype=out_dtype, device=gu.device)
+    _check(core().li_swiglu(_ptr(gu), _ptr(h), DT[out_dtype], c_int64(h.numel()), _stream()), "swiglu")
+    return h
+
+
+def rope_store(qkv, inv_freq, rotary_dim, half_pairing, pos, tok_slot, page_table, k_pages, v_pages,
+               n_heads, n_kv_heads, head_dim, out_dtype) -> torch.Tensor:
+    """Rotate q and k by position, write k and v into the pages; returns q [T, H, hd].
+    With n_kv_heads == 0 only q is rotated (a layer that reads another layer's cache)."""
+    _dev(qkv, inv_freq, pos, tok_slot, page_table, k_pages, v_pages)
+    t = qkv.shape[0]
+    _need(qkv.dtype == torch.float32 and qkv.dim() == 2, "qkv: float32 [T, (H+2K) hd]")
+    _need(qkv.shape[1] >= (n_heads + 2 * n_kv_heads) * head_dim, "qkv row too short")
+    _need(pos.dtype == torch.int32 and pos.numel() >= t, "pos: int32 [T]")
+    if rotary_dim > 0:
+        _need(inv_freq is not None and inv_freq.dtype == torch.float32 and inv_freq.numel() >= rotary_dim // 2,
+              "inv_freq: float32 [rotary_dim / 2]")
+    if n_kv_heads > 0:
+        _need(tok_slot.dtype == torch.int32 and tok_slot.numel() >= t, "tok_slot: int32 [T]")
+        _need(page_table.dtype == torch.int32 and page_table.dim() == 2, "page_table: int32 [slots, pages]")
+        _need(k_pages.dtype == out_dtype and v_pages.dtype == out_dtype, "cache dtype differs from q dtype")
+    q = torch.empty((t, n_heads, head_dim), dtype=out_dtype, device=qkv.device)
+    _check(core().li_rope_store(
+        _ptr(qkv), qkv.shape[1], _ptr(inv_freq), rotary_dim, int(half_pairing), _ptr(pos), _ptr(tok_slot),
+        _ptr(page_table), page_table.shape[1] if page_table is not None else 0, _ptr(q), _ptr(k_pages),
+        _ptr(v_pages), DT[out_dtype], t, n_heads, n_kv_heads, head_dim, _stream()), "rope_store")
+    return q
+
+
+def decode_prepare(seq_slot, lens, pos, ctx, n):
+    _dev(seq_slot, lens, pos, ctx)
+    for a in (seq_slot, lens, pos, ctx):
+        _need(a.dtype == torch.int32, "decode_prepare: int32 arrays")
+    _need(seq_slot.numel() >= n and pos.numel() >= n and ctx.numel() >= n, "decode_prepare: arrays too short")
+    _check(core().li_decode_prepare(_ptr(seq_slot), _ptr(lens), _ptr(pos), _ptr(ctx), n, _stream()), "decode_prepare")
+
+
+# ---------------------------------------------------------------------------
+# attention
+# ---------------------------------------------------------------------------
+_attn: dict = {}
+
+
+def _attn_lib(head_dim: int):
+    lib = _attn.get(head_dim)
+    if lib is None:
+        lib = build.attention_library(head_dim)
+        _need(lib.li_attn_head_dim() == head_dim, "attention library built for another head size")
+        _attn[head_dim] = lib
+    return lib
+
+
+def _check_pages(k_pages, v_pages, page_table, n_kv_heads, head_dim, dtype):
+    _need(k_pages.dtype == dtype and v_pages.dtype == dtype, "cache dtype differs from q dtype")
+    _need(page_table.dtype == torch.int32 and page_table.dim() == 2, "page_table: int32 [slots, pages]")
+
+
+def attention_prefill(q, kv, meta, n_heads, n_kv_heads, head_dim, scale, window) -> torch.Tensor:
+    """16-bit attention for a step with whole prompts.  ``kv``: (k_pages, v_pages, page_stride,
+    page_table); ``meta``: dict of int32 device arrays tile_seq, tile_q0, seq_slot, seq_qstart,
+    seq_qlen, seq_ctx and the int n_tiles."""
+    k_pages, v_pages, page_stride, page_table = kv
+    _dev(q, k_pages, v_pages, page_table)
+    _need(q.dtype in (torch.float16, torch.bfloat16) and q.shape[1:] == (n_heads, head_dim), "q: 16-bit [T, H, hd]")
+    _check_pages(k_pages, v_pages, page_table, n_kv_heads, head_dim, q.dtype)
+    out = torch.empty_like(q)
+    _check(_attn_lib(head_dim).li_attn_prefill(
+        _ptr(q), _ptr(out), DT[q.dtype], _ptr(k_pages), _ptr(v_pages), c_int64(page_stride), _ptr(page_table),
+        page_table.shape[1], _ptr(meta["tile_seq"]), _ptr(meta["tile_q0"]), meta["n_tiles"], _ptr(meta["seq_slot"]),
+        _ptr(meta["seq_qstart"]), _ptr(meta["seq_qlen"]), _ptr(meta["seq_ctx"]), n_heads, n_kv_heads,
+        c_float(scale), int(window or 0), _stream()), "attn_prefill")
+    return out
+
+
+def attention_decode(q, kv, seq_slot, seq_ctx, n_seqs, n_heads, n_kv_heads, head_dim, scale, window,
+                     splits: int = 1) -> torch.Tensor:
+    """16-bit attention for one new token per sequence; q [B, H, hd]."""
+    k_pages, v_pages, page_stride, page_table = kv
+    _dev(q, k_pages, v_pages, page_table, seq_slot, seq_ctx)
+    _need(q.dtype in (torch.float16, torch.bfloat16) and q.shape == (n_seqs, n_heads, head_dim), "q: 16-bit [B, H, hd]")
+    _check_pages(k_pages, v_pages, page_table, n_kv_heads, head_dim, q.dtype)
+    _need(seq_slot.numel() >= n_seqs and seq_ctx.numel() >= n_seqs, "per-sequence arrays too short")
+    out = torch.empty_like(q)
+    part_o = part_ml = None
+    if splits > 1:
+        part_o = torch.empty((n_seqs, n_heads, splits, head_dim), dtype=torch.float32, device=q.device)
+        part_ml = torch.empty((n_seqs, n_heads, splits, 2), dtype=torch.float32, device=q.device)
+    _check(_attn_lib(head_dim).li_attn_decode(
+        _ptr(q), _ptr(out), DT[q.dtype], _ptr(k_pages), _ptr(v_pages), c_int64(page_stride), _ptr(page_table),
+        page_table.shape[1], _ptr(seq_slot), _ptr(seq_ctx), n_seqs, n_heads, n_kv_heads, c_float(scale),
+        int(window or 0), splits, _ptr(part_o), _ptr(part_ml), _stream()), "attn_decode")
+    return out
+
+
+def attention_f32(q, kv, pos, tok_slot, n_heads, n_kv_heads, head_dim, scale, window) -> torch.Tensor:
+    """float32 attention for any step: every token reads its sequence's cache up to its position."""
+    k_pages, v_pages, page_stride, page_table = kv
+    _dev(q, k_pages, v_pages, page_table, pos, tok_slot)
+    _need(q.dtype == torch.float32 and q.shape[1:] == (n_heads, head_dim), "q: float32 [T, H, hd]")
+    _check_pages(k_pages, v_pages, page_table, n_kv_heads, head_dim, torch.float32)
+    _need(pos.numel() >= q.shape[0] and tok_slot.numel() >= q.shape[0], "per-token arrays too short")
+    out = torch.empty_like(q)
+    _check(_attn_lib(head_dim).li_attn_f32(
+        _ptr(q), _ptr(out), _ptr(k_pages), _ptr(v_pages), c_int64(page_stride), _ptr(page_table),
+        page_table.shape[1], _ptr(pos), _ptr(tok_slot), q.shape[0], n_heads, n_kv_heads, c_float(scale),
+        int(window or 0), _stream()), "attn_f32")
+    return out
+
+
+# ---------------------------------------------------------------------------
+# sampling
+# ---------------------------------------------------------------------------
+def argmax(logits: torch.Tensor, out: torch.Tensor | None = None) -> torch.Tensor:
+    _dev(logits, out)
+    _need(logits.dtype == torch.float32 and logits.dim() == 2, "logits: float32 [B, V]")
+    if out is None:
+        out = torch.empty((logits.shape[0],), dtype=torch.int32, device=logits.device)
+    _need(out.dtype == torch.int32 and out.numel() >= logits.shape[0], "out: int32 [B]")
+    _check(core().li_argmax(_ptr(logits), logits.shape[0], logits.shape[1], _ptr(out), _stream()), "argmax")
+    return out
+
+
+def sample(logits, temperature: float, seq_slot=None, state=None, forced_r=None, out=None) -> torch.Tensor:
+    """Temperature sampling; ``state`` is the [slots, 2] int64 (key, counter) table, ``forced_r``
+    (float32 [B]) replaces the generator for tests."""
+    _dev(logits, seq_slot, state, forced_r, out)
+    _need(logits.dtype == torch.float32 and logits.dim() == 2, "logits: float32 [B, V]")
+    b = logits.shape[0]
+    if out is None:
+        out = torch.empty((b,), dtype=torch.int32, device=logits.device)
+    if temperature > 0 and forced_r is None:
+        _need(seq_slot is not None and seq_slot.dtype == torch.int32 and seq_slot.numel() >= b, "seq_slot: int32 [B]")
+        _need(state is not None and state.dtype == torch.int64 and state.dim() == 2 and state.shape[1] == 2,
+              "state: int64 [slots, 2]")
+    if forced_r is not None:
+        _need(forced_r.dtype == torch.float32 and forced_r.numel() >= b, "forced_r: float32 [B]")
+    _check(core().li_sample(_ptr(logits), b, logits.shape[1], c_float(temperature), _ptr(seq_slot), _ptr(state),
+                            _ptr(forced_r), _ptr(out), _stream()), "sample")
+    return out
+
+
+def uniform01(key: int, counter: int) -> float:
+    """The generator's value for (key, counter), computed on the host by the same function."""
+    return float(core().li_uniform01(c_uint64(key & (2 ** 64 - 1)), c_uint64(counter & (2 ** 64 - 1))))

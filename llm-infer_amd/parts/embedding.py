@@ -1,0 +1,54 @@
+from __future__ import annotations
+
+import torch
+
+from ..kernels import ops
+from ..registry import register_embedding, register_head
+from ..weights.loader import ParamSpec
+from .base import Part
+
+
+@register_embedding("embedding")
+class Embedding(Part):
+    """x = float32(table[token]), unscaled (src/model/model.cpp:101-118)."""
+
+    def __init__(self, *, vocab_size, hidden_size, prefix, dtype, device):
+        self.vocab_size, self.hidden_size = vocab_size, hidden_size
+        self.prefix, self.dtype, self.device = prefix, dtype, device
+        self.weight = None
+
+    def params(self):
+        return {"weight": ParamSpec((self.vocab_size, self.hidden_size))}
+
+    def bind(self, tensors):
+        self.weight = tensors["weight"]
+
+    def forward(self, tokens):
+        return ops.embed(self.weight, tokens)
+
+
+@register_head("lm_head")
+class LMHead(Part):
+    """logits = h W^T in float32 (src/model/model.cpp:93-98).  ``tied``: W is the embedding
+    table (the reference has no tied models: it requires output.weight, model.cpp:35-38)."""
+
+    def __init__(self, *, vocab_size, hidden_size, tied, prefix, dtype, device):
+        self.vocab_size, self.hidden_size, self.tied = vocab_size, hidden_size, tied
+        self.prefix, self.dtype, self.device = prefix, dtype, device
+        self.weight = None
+
+    def params(self):
+        return {} if self.tied else {"weight": ParamSpec((self.vocab_size, self.hidden_size))}
+
+    def ignorable(self):
+        return [self.prefix + "weight"] if self.tied else []
+
+    def bind(self, tensors):
+        if not self.tied:
+            self.weight = tensors["weight"]
+
+    def tie(self, table):
+        self.weight = table
+
+    def forward(self, h):
+        return ops.linear(h, self.weight, out_dtype=torch.float32)

@@ -1,0 +1,27 @@
+from __future__ import annotations
+
+import torch
+
+from ..kernels import ops
+from ..registry import register_norm
+from ..weights.loader import ParamSpec
+from .base import Part
+
+
+@register_norm("rmsnorm")
+class RMSNorm(Part):
+    """out = x / sqrt(mean(x^2) + eps) * weight, in float32; the weight is kept in float32
+    (include/kernels_cpu.hpp:43-54, src/model/block.cpp:81-83)."""
+
+    def __init__(self, *, size: int, eps: float, prefix: str, dtype, device):
+        self.size, self.eps, self.prefix, self.dtype, self.device = size, float(eps), prefix, dtype, device
+        self.weight = None
+
+    def params(self):
+        return {"weight": ParamSpec((self.size,), "vector", "ones")}
+
+    def bind(self, tensors):
+        self.weight = tensors["weight"]
+
+    def forward(self, x: torch.Tensor, rows: torch.Tensor | None = None) -> torch.Tensor:
+        return ops.rmsnorm(x, self.weight, self.eps, self.dtype, rows)

@@ -1,0 +1,49 @@
+from __future__ import annotations
+
+import torch
+
+from ..kernels import ops
+from ..registry import register_position
+
+
+@register_position("rope")
+class RotaryPosition:
+    """Rotation of q and k by position: angle = pos * theta^(-i / rotary_dim) for the pair
+    that starts at dimension i (include/kernels_cpu.hpp:82-100).  ``pairing`` "adjacent"
+    rotates (i, i+1) as the reference does; "half" rotates (i/2, i/2 + rotary_dim/2).
+
+    A position encoding owns a table of one frequency per rotated pair; another
+    encoding of this family (scaled, interpolated) only fills the table differently.
+    Its one duty towards a mixer is ``rotate_store``: rotate q and k of the step's
+    tokens, write k and v into the layer's pages, and return q.
+    """
+
+    def __init__(self, *, theta: float, rotary_dim: int, head_dim: int, pairing: str = "adjacent", dtype, device):
+        self.rotary_dim, self.head_dim, self.pairing = rotary_dim, head_dim, pairing
+        i = torch.arange(0, rotary_dim, 2, dtype=torch.float32)
+        # 1 / powf(theta, i / rotary_dim) in float32, as kernels_cpu.hpp:87
+        inv = 1.0 / torch.pow(torch.tensor(float(theta), dtype=torch.float32), i / float(rotary_dim))
+        self.inv_freq = inv.to(device) if device is not None else inv
+        self.dtype = dtype
+
+    def rotate_store(self, qkv, ctx, kv_view, n_heads, n_kv_heads, head_dim):
+        k = v = table = None
+        if n_kv_heads > 0:
+            k, v, table = kv_view.k, kv_view.v, kv_view.page_table
+        return ops.rope_store(qkv, self.inv_freq, self.rotary_dim, self.pairing == "half", ctx.pos, ctx.tok_slot,
+                              table, k, v, n_heads, n_kv_heads, head_dim, self.dtype)
+
+
+@register_position("none")
+class NoPosition:
+    """No position encoding: q passes unrotated, k and v are written as they are."""
+
+    def __init__(self, *, dtype, device, **_):
+        self.dtype = dtype
+
+    def rotate_store(self, qkv, ctx, kv_view, n_heads, n_kv_heads, head_dim):
+        k = v = table = None
+        if n_kv_heads > 0:
+            k, v, table = kv_view.k, kv_view.v, kv_view.page_table
+        return ops.rope_store(qkv, None, 0, False, ctx.pos, ctx.tok_slot, table, k, v, n_heads, n_kv_heads,
+                              head_dim, self.dtype)

@@ -1,0 +1,121 @@
+"""Weights by tensor name.
+
+A model states which tensors it needs (``ParamSpec`` for each name); the loader
+compares that table with what a checkpoint folder holds and raises ONE error that
+lists every missing tensor, every unexpected tensor and every wrong shape
+(the reference stops at the first: include/model/tensor.hpp:18-24, 112-137).
+
+Kept dtypes: matrices in the compute dtype (bfloat16 or float16; float32 in the
+32-bit path), norm vectors in float32 (the reference requires F32 norm weights,
+src/model/block.cpp:81-83), integer tables as int32, and a tensor that is stored
+in 32-bit stays 32-bit.
+"""
+from __future__ import annotations
+
+import json
+import os
+from dataclasses import dataclass
+
+import torch
+
+from .safetensors_io import SafetensorsFile
+
+
+class WeightError(ValueError):
+    pass
+
+
+@dataclass(frozen=True)
+class ParamSpec:
+    shape: tuple
+    kind: str = "matrix"        # "matrix" | "vector" | "int"
+    init: str = "normal"        # random-weights mode: "normal" N(0, 0.02) | "ones" 1 + N(0, 0.01)
+
+
+class Checkpoint:
+    """The tensors of a model folder: one ``model.safetensors`` or the shards that
+    ``model.safetensors.index.json`` names."""
+
+    def __init__(self, folder: str):
+        self.folder = folder
+        single = os.path.join(folder, "model.safetensors")
+        index = os.path.join(folder, "model.safetensors.index.json")
+        self._where = {}
+        self._files = {}
+        if os.path.isfile(single):
+            self._files[single] = SafetensorsFile(single)
+        elif os.path.isfile(index):
+            with open(index) as f:
+                for name, shard in json.load(f)["weight_map"].items():
+                    path = os.path.join(folder, shard)
+                    if path not in self._files:
+                        self._files[path] = SafetensorsFile(path)
+        else:
+            raise WeightError(f"no model.safetensors (or model.safetensors.index.json) in {folder}")
+        for path, f in self._files.items():
+            for name in f.names():
+                self._where[name] = f
+
+    def names(self) -> list:
+        return list(self._where)
+
+    def info(self, name: str):
+        return self._where[name].info(name)
+
+    def tensor(self, name: str) -> torch.Tensor:
+        return self._where[name].tensor(name)
+
+
+def read_checkpoint(folder: str) -> Checkpoint:
+    return Checkpoint(folder)
+
+
+def check_tensors(needed: dict, found, ignorable=()) -> None:
+    """``needed``: name -> ParamSpec; ``found``: object with names() and info(name).
+    Raises one WeightError listing all that is missing, unexpected or misshapen."""
+    have = set(found.names())
+    missing = [n for n in needed if n not in have]
+    unexpected = sorted(n for n in have if n not in needed and n not in ignorable)
+    wrong = []
+    for n, spec in needed.items():
+        if n in have:
+            dtype, shape = found.info(n)
+            if tuple(shape) != tuple(spec.shape):
+                wrong.append(f"{n}: expected {list(spec.shape)}, got {list(shape)}")
+            elif spec.kind == "int" and dtype.is_floating_point:
+                wrong.append(f"{n}: expected an integer table, got {dtype}")
+            elif spec.kind != "int" and not dtype.is_floating_point:
+                wrong.append(f"{n}: expected floating point, got {dtype}")
+    if missing or unexpected or wrong:
+        parts = ["the checkpoint does not fit the model:"]
+        if missing:
+            parts.append(f"  missing tensors ({len(missing)}): " + ", ".join(missing))
+        if unexpected:
+            parts.append(f"  unexpected tensors ({len(unexpected)}): " + ", ".join(unexpected))
+        if wrong:
+            parts.append(f"  wrong shapes or types ({len(wrong)}): " + "; ".join(wrong))
+        raise WeightError("\n".join(parts))
+
+
+def kept_dtype(stored: torch.dtype, kind: str, compute: torch.dtype) -> torch.dtype:
+    if kind == "int":
+        return torch.int32
+    if kind == "vector" or compute == torch.float32:
+        return torch.float32
+    if stored in (torch.float32, torch.float64):
+        return torch.float32                      # stored in 32-bit stays so
+    return compute
+
+
+def place_tensor(t: torch.Tensor, kind: str, compute: torch.dtype, device) -> torch.Tensor:
+    """Move one tensor to the device in the dtype the engine keeps it in."""
+    return t.to(device=device, dtype=kept_dtype(t.dtype, kind, compute)).contiguous()
+
+
+def load_into(model, folder: str) -> None:
+    """Check the folder's tensors against ``model.params()`` and hand each part its tensors."""
+    ckpt = read_checkpoint(folder)
+    needed = model.params()
+    check_tensors(needed, ckpt, model.ignorable_names())
+    model.bind({name: place_tensor(ckpt.tensor(name), spec.kind, model.dtype, model.device)
+                for name, spec in needed.items()})

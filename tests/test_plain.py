@@ -1,0 +1,211 @@
+"""Pins the plain implementation by what fixes it beside the reference's text.
+
+The reference holds no test vectors, so each formula is pinned by special cases
+that reduce to a library routine and by invariants, chosen so that a plausible
+mistake (wrong sign or pairing, eps outside the root, swapped gate and up, a norm
+in the wrong place) fails.
+"""
+import math
+
+import pytest
+import torch
+
+import plain_llama as P
+from tiny_configs import ALL, TINY_A, TINY_B, TINY_C
+
+torch.manual_seed(0)
+F64 = torch.float64
+
+
+def test_rmsnorm_library_formula_and_eps_place():
+    x = torch.randn(5, 96, dtype=F64)
+    w = torch.randn(96, dtype=F64)
+    ref = x * torch.rsqrt((x * x).mean(-1, keepdim=True) + 1e-5) * w
+    assert torch.allclose(P.rmsnorm(x, w, 1e-5), ref, rtol=1e-12, atol=0)
+    # eps is added to the mean inside the root: at mean-square 1e-6, eps 1e-5 dominates
+    x = torch.full((1, 64), 1e-3, dtype=F64)
+    out = P.rmsnorm(x, torch.ones(64, dtype=F64), 1e-5)
+    assert torch.allclose(out, torch.full_like(out, 1e-3 / math.sqrt(1e-6 + 1e-5)), rtol=1e-12)
+    # the weight multiplies, it is not (1 + w)
+    assert P.rmsnorm(torch.randn(3, 8, dtype=F64), torch.zeros(8, dtype=F64), 1e-5).abs().max() == 0
+    # mean-square of the output with w=1
+    x = torch.randn(4, 128, dtype=F64)
+    ms = (x * x).mean(-1)
+    out = P.rmsnorm(x, torch.ones(128, dtype=F64), 1e-5)
+    assert torch.allclose((out * out).mean(-1), ms / (ms + 1e-5), rtol=1e-12)
+
+
+def test_linear_is_x_wt():
+    x, w = torch.randn(3, 7, dtype=F64), torch.randn(5, 7, dtype=F64)
+    assert torch.allclose(P.linear(x, w), torch.nn.functional.linear(x, w))
+    assert P.linear(x, w).shape == (3, 5)
+
+
+def test_rope_identity_norm_pairing_theta_sign():
+    v = torch.randn(6, 3, 32, dtype=F64)
+    pos = torch.tensor([0, 1, 2, 50, 51, 1000])
+    out = P.rope(v, pos, 10000.0, 32)
+    assert torch.equal(out[0], v[0])                      # position 0 is the identity
+    a = v.view(6, 3, 16, 2).norm(dim=-1)
+    b = out.view(6, 3, 16, 2).norm(dim=-1)
+    assert torch.allclose(a, b, rtol=1e-12)               # every adjacent pair keeps its norm
+    # a one-hot at 2j moves mass only to 2j+1, with (cos a, +sin a)
+    j = 3
+    e = torch.zeros(1, 1, 32, dtype=F64)
+    e[0, 0, 2 * j] = 1.0
+    r = P.rope(e, torch.tensor([7]), 500000.0, 32)
+    ang = 7.0 * 500000.0 ** (-(2 * j) / 32)
+    want = torch.zeros(32, dtype=F64)
+    want[2 * j], want[2 * j + 1] = math.cos(ang), math.sin(ang)
+    assert torch.allclose(r[0, 0], want, atol=1e-12)
+    # the exponent's denominator is rotary_dim, not head_dim
+    e = torch.zeros(1, 1, 32, dtype=F64)
+    e[0, 0, 2] = 1.0
+    r = P.rope(e, torch.tensor([1]), 10000.0, 16)
+    assert abs(r[0, 0, 2].item() - math.cos(10000.0 ** (-2 / 16))) < 1e-12
+    # dimensions beyond rotary_dim are left alone
+    out = P.rope(v, pos, 10000.0, 16)
+    assert torch.equal(out[..., 16:], v[..., 16:])
+    assert not torch.equal(out[1:, :, :16], v[1:, :, :16])
+
+
+def test_rope_scores_depend_on_distance_only():
+    q = torch.randn(1, 2, 16, dtype=F64)
+    k = torch.randn(1, 2, 16, dtype=F64)
+    def score(m, n):
+        return (P.rope(q, torch.tensor([m]), 1e4, 16) * P.rope(k, torch.tensor([n]), 1e4, 16)).sum(-1)
+    assert torch.allclose(score(5, 2), score(105, 102), atol=1e-10)
+    assert not torch.allclose(score(5, 2), score(5, 3), atol=1e-6)
+
+
+def _library_attention(q, k, v):
+    n, H, hd = q.shape
+    g = H // k.shape[1]
+    kk = k.repeat_interleave(g, dim=1).transpose(0, 1)
+    vv = v.repeat_interleave(g, dim=1).transpose(0, 1)
+    o = torch.nn.functional.scaled_dot_product_attention(q.transpose(0, 1), kk, vv, is_causal=True)
+    return o.transpose(0, 1)
+
+
+@pytest.mark.parametrize("H,K,hd", [(4, 2, 16), (3, 1, 32), (5, 5, 48), (8, 2, 64)])
+def test_attention_equals_library(H, K, hd):
+    n = 11
+    q, k, v = torch.randn(n, H, hd, dtype=F64), torch.randn(n, K, hd, dtype=F64), torch.randn(n, K, hd, dtype=F64)
+    assert torch.allclose(P.attention(q, k, v), _library_attention(q, k, v), atol=1e-12)
+
+
+def test_attention_special_cases():
+    n, H, K, hd = 6, 4, 2, 16
+    q, v = torch.randn(n, H, hd, dtype=F64), torch.randn(n, K, hd, dtype=F64)
+    k = torch.randn(n, K, hd, dtype=F64)
+    out = P.attention(q, k, v)
+    # the first token sees only itself
+    assert torch.allclose(out[0], v[0].repeat_interleave(2, dim=0))
+    # equal keys: the output is the running mean of the values
+    ku = torch.ones(n, K, hd, dtype=F64)
+    out = P.attention(q, ku, v)
+    means = torch.cumsum(v, 0) / torch.arange(1, n + 1, dtype=F64)[:, None, None]
+    assert torch.allclose(out, means.repeat_interleave(2, dim=1), atol=1e-12)
+    # consecutive query heads share a KV head: h // (H // K)
+    q2 = q.clone()
+    q2[:, 1] = q2[:, 0]
+    out = P.attention(q2, k, v)
+    assert torch.allclose(out[:, 0], out[:, 1])
+    assert not torch.allclose(out[:, 1], P.attention(q2[:, [0, 2, 1, 3]], k, v)[:, 1])
+    # the scale is 1/sqrt(hd): with one outstanding key the weights are known in closed form
+    hd = 32
+    q = torch.zeros(2, 1, hd, dtype=F64)
+    q[1, 0, 0] = 3.0
+    k = torch.zeros(2, 1, hd, dtype=F64)
+    k[1, 0, 0] = 2.0
+    v = torch.tensor([[[0.0] * hd], [[1.0] * hd]], dtype=F64)
+    p1 = math.exp(6.0 / math.sqrt(hd)) / (1.0 + math.exp(6.0 / math.sqrt(hd)))
+    assert abs(P.attention(q, k, v)[1, 0, 0].item() - p1) < 1e-12
+    # window: only the last w keys
+    n = 9
+    q, k, v = (torch.randn(n, 2, 16, dtype=F64) for _ in range(3))
+    w = P.attention(q, k, v, window=3)
+    assert torch.allclose(w[:3], P.attention(q, k, v)[:3])
+    assert torch.allclose(w[8], P.attention(q[6:9], k[6:9], v[6:9])[2])
+
+
+def test_silu_and_swiglu():
+    x = torch.tensor([0.0, 30.0, -2.0, 2.0], dtype=F64)
+    s = P.silu(x)
+    assert s[0] == 0 and abs(s[1] - 30.0) < 1e-9
+    assert torch.allclose(s[2], -2.0 * torch.sigmoid(torch.tensor(-2.0, dtype=F64)))
+    assert torch.allclose(s, torch.nn.functional.silu(x))
+    d, f = 8, 12
+    xx = torch.randn(3, d, dtype=F64)
+    wg, wu, wd = torch.randn(f, d, dtype=F64), torch.randn(f, d, dtype=F64), torch.randn(d, f, dtype=F64)
+    assert P.swiglu(xx, torch.zeros_like(wg), wu, wd).abs().max() == 0
+    assert P.swiglu(xx, wg, torch.zeros_like(wu), wd).abs().max() == 0
+    ref = torch.nn.functional.linear(torch.nn.functional.silu(xx @ wg.t()) * (xx @ wu.t()), wd)
+    assert torch.allclose(P.swiglu(xx, wg, wu, wd), ref)
+    assert not torch.allclose(P.swiglu(xx, wu, wg, wd), ref)       # gate and up are not interchangeable
+
+
+@pytest.mark.parametrize("name", list(ALL))
+def test_block_is_identity_without_output_matrices(name):
+    cfg = ALL[name]
+    s = P.sizes(cfg)
+    w = {k: v.double() for k, v in P.random_weights(cfg, 3).items()}
+    w["model.layers.0.self_attn.o_proj.weight"].zero_()
+    w["model.layers.0.mlp.down_proj.weight"].zero_()
+    x = torch.randn(5, s["d"], dtype=F64)
+    assert torch.equal(P.block(x, w, 0, s, torch.arange(5)), x)
+
+
+def test_attention_part_shift_invariance():
+    s = P.sizes(TINY_A)
+    w = {k: v.double() for k, v in P.random_weights(TINY_A, 1, std=0.3).items()}
+    x = torch.randn(7, s["d"], dtype=F64)
+    a = P.attention_part(x, w, "model.layers.0.self_attn.", s, torch.arange(7))
+    b = P.attention_part(x, w, "model.layers.0.self_attn.", s, torch.arange(7) + 40)
+    assert torch.allclose(a, b, atol=1e-10)
+
+
+def test_sizes_defaults():
+    s = P.sizes({"hidden_size": 64, "num_attention_heads": 4, "num_hidden_layers": 1,
+                 "intermediate_size": 8, "vocab_size": 10})
+    assert s["n_kv"] == 4 and s["hd"] == 16 and s["theta"] == 10000.0 and s["eps"] == 1e-5
+    assert s["rotary"] == 16 and not s["tied"]
+    assert P.sizes(TINY_C)["rotary"] == 24 and P.sizes(TINY_C)["hd"] == 48
+
+
+def test_head_tied_and_untied_and_prefix_property():
+    for cfg in (TINY_A, TINY_B):
+        w = P.random_weights(cfg, 5, std=0.2)
+        toks = list(range(3, 14))
+        full = P.forward(w, cfg, toks, F64)
+        # causal: the logits of a prefix equal the prefix of the logits
+        part = P.forward(w, cfg, toks[:6], F64)
+        assert torch.allclose(full[:6], part, atol=1e-10)
+        assert full.shape == (11, cfg["vocab_size"])
+    assert "lm_head.weight" not in P.random_weights(TINY_B, 0)
+    w = P.random_weights(TINY_A, 5, std=0.2)
+    a = P.forward(w, TINY_A, [1, 2, 3], F64)
+    w["lm_head.weight"] = w["lm_head.weight"] * 2
+    assert torch.allclose(P.forward(w, TINY_A, [1, 2, 3], F64), 2 * a, atol=1e-10)
+
+
+def test_sampling_rules():
+    l = torch.tensor([1.0, 5.0, 5.0, 2.0])
+    assert P.sample_greedy(l) == 1                                  # the first maximum wins
+    assert P.sample_temperature(l, 0.0, 0.3) == 1
+    assert P.sample_temperature(l, -1.0, 0.3) == 1
+    p = P.probabilities(l, 0.8)
+    assert torch.allclose(p, torch.softmax(l / 0.8, 0))
+    assert P.sample_temperature(l, 0.8, 0.0) == 0
+    assert P.sample_temperature(l, 0.8, float(p[0]) + 1e-4) == 1
+    assert P.sample_temperature(l, 0.8, 0.99999999) == 3
+    assert P.sample_temperature(l, 1e-4, 0.9) in (1, 2)
+
+
+def test_generate_stops_before_keeping_the_stop_token():
+    w = P.random_weights(TINY_A, 2, std=0.2)
+    out = P.generate_greedy(w, TINY_A, [4, 5, 6], 6)
+    assert len(out) == 6
+    cut = P.generate_greedy(w, TINY_A, [4, 5, 6], 6, stop=(out[2],))
+    first = out.index(out[2])
+    assert cut == out[:first]

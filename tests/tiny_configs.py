@@ -1,0 +1,29 @@
+"""Small configurations of the architecture that differ in every size and option."""
+
+# 2 layers, GQA 4/2, head 16, ffn 172 (no multiple of 8), untied
+TINY_A = {
+    "architectures": ["LlamaForCausalLM"], "model_type": "llama",
+    "num_hidden_layers": 2, "hidden_size": 64, "num_attention_heads": 4, "num_key_value_heads": 2,
+    "intermediate_size": 172, "vocab_size": 256, "rope_theta": 10000.0, "rms_norm_eps": 1e-5,
+    "max_position_embeddings": 128, "tie_word_embeddings": False, "hidden_act": "silu",
+}
+
+# 3 layers, MQA 3/1, head 32, tied head, other theta and eps
+TINY_B = {
+    "architectures": ["LlamaForCausalLM"], "model_type": "llama",
+    "num_hidden_layers": 3, "hidden_size": 96, "num_attention_heads": 3, "num_key_value_heads": 1,
+    "intermediate_size": 256, "vocab_size": 384, "rope_theta": 500000.0, "rms_norm_eps": 1e-6,
+    "max_position_embeddings": 256, "tie_word_embeddings": True, "hidden_act": "silu",
+}
+
+# 1 layer, MHA 5/5, explicit head_dim 48 != hidden/heads, half of each head rotated,
+# odd vocabulary, long context
+TINY_C = {
+    "architectures": ["LlamaForCausalLM"], "model_type": "llama",
+    "num_hidden_layers": 1, "hidden_size": 80, "num_attention_heads": 5, "head_dim": 48,
+    "intermediate_size": 136, "vocab_size": 331, "rope_theta": 1000.0, "rms_norm_eps": 1e-4,
+    "partial_rotary_factor": 0.5,
+    "max_position_embeddings": 1024, "tie_word_embeddings": False, "hidden_act": "silu",
+}
+
+ALL = {"A": TINY_A, "B": TINY_B, "C": TINY_C}
