@@ -75,7 +75,7 @@ template <class T>
 __global__ void rope_store_kernel(const float* __restrict__ qkv, int row_stride,
                                   const float* __restrict__ inv_freq, int rotary_dim, int half_pairing,
                                   const int* __restrict__ pos, const int* __restrict__ tok_slot,
-                                  const int* __restrict__ page_table, int max_pages,
+                                  const int* __restrict__ page_table, int max_pages, int64_t page_stride,
                                   T* __restrict__ q_out, T* __restrict__ k_pages, T* __restrict__ v_pages,
                                   int H, int K, int hd) {
     const int t = blockIdx.x;
@@ -106,10 +106,10 @@ __global__ void rope_store_kernel(const float* __restrict__ qkv, int row_stride,
             T* q = q_out + ((int64_t)t * H + head) * hd;
             q[d0] = from_f32<T>(a); q[d1] = from_f32<T>(b);
         } else if (head < H + K) {
-            T* kp = k_pages + (page * K + (head - H)) * k_head_elems(hd);
+            T* kp = k_pages + page * page_stride + (int64_t)(head - H) * k_head_elems(hd);
             kp[k_offset(tp, d0, hd)] = from_f32<T>(a); kp[k_offset(tp, d1, hd)] = from_f32<T>(b);
         } else {
-            T* vp = v_pages + (page * K + (head - H - K)) * v_head_elems(hd);
+            T* vp = v_pages + page * page_stride + (int64_t)(head - H - K) * v_head_elems(hd);
             vp[v_offset(tp, d0, hd)] = from_f32<T>(a); vp[v_offset(tp, d1, hd)] = from_f32<T>(b);
         }
     }
@@ -117,7 +117,7 @@ __global__ void rope_store_kernel(const float* __restrict__ qkv, int row_stride,
 
 extern "C" int li_rope_store(const float* qkv, int row_stride, const float* inv_freq, int rotary_dim,
                              int half_pairing, const int* pos, const int* tok_slot, const int* page_table,
-                             int max_pages, void* q_out, void* k_pages, void* v_pages, int dt,
+                             int max_pages, int64_t page_stride, void* q_out, void* k_pages, void* v_pages, int dt,
                              int n_tokens, int H, int K, int hd, hipStream_t stream) {
     if (n_tokens <= 0) return LI_OK;
     if (hd <= 0 || (hd & 1) || H <= 0 || K < 0 || rotary_dim < 0 || rotary_dim > hd || (rotary_dim & 1) ||
@@ -127,7 +127,7 @@ extern "C" int li_rope_store(const float* qkv, int row_stride, const float* inv_
     dim3 grid(n_tokens), block(256);
 #define LAUNCH(T)                                                                                        \
     rope_store_kernel<T><<<grid, block, 0, stream>>>(qkv, row_stride, inv_freq, rotary_dim, half_pairing, \
-                                                     pos, tok_slot, page_table, max_pages, (T*)q_out,    \
+                                                     pos, tok_slot, page_table, max_pages, page_stride, (T*)q_out, \
                                                      (T*)k_pages, (T*)v_pages, H, K, hd)
     if (dt == DT_F32) LAUNCH(float);
     else if (dt == DT_F16) LAUNCH(f16);

@@ -156,7 +156,7 @@ def swiglu(gu: torch.Tensor, out_dtype) -> torch.Tensor:
     return h
 
 
-def rope_store(qkv, inv_freq, rotary_dim, half_pairing, pos, tok_slot, page_table, k_pages, v_pages,
+def rope_store(qkv, inv_freq, rotary_dim, half_pairing, pos, tok_slot, page_table, page_stride, k_pages, v_pages,
                n_heads, n_kv_heads, head_dim, out_dtype) -> torch.Tensor:
     """Rotate q and k by position, write k and v into the pages; returns q [T, H, hd].
     With n_kv_heads == 0 only q is rotated (a layer that reads another layer's cache)."""
@@ -175,7 +175,8 @@ def rope_store(qkv, inv_freq, rotary_dim, half_pairing, pos, tok_slot, page_tabl
     q = torch.empty((t, n_heads, head_dim), dtype=out_dtype, device=qkv.device)
     _check(core().li_rope_store(
         _ptr(qkv), qkv.shape[1], _ptr(inv_freq), rotary_dim, int(half_pairing), _ptr(pos), _ptr(tok_slot),
-        _ptr(page_table), page_table.shape[1] if page_table is not None else 0, _ptr(q), _ptr(k_pages),
+        _ptr(page_table), page_table.shape[1] if page_table is not None else 0, c_int64(page_stride or 0),
+        _ptr(q), _ptr(k_pages),
         _ptr(v_pages), DT[out_dtype], t, n_heads, n_kv_heads, head_dim, _stream()), "rope_store")
     return q
 

@@ -27,11 +27,11 @@ class RotaryPosition:
         self.dtype = dtype
 
     def rotate_store(self, qkv, ctx, kv_view, n_heads, n_kv_heads, head_dim):
-        k = v = table = None
+        k = v = table = stride = None
         if n_kv_heads > 0:
-            k, v, table = kv_view.k, kv_view.v, kv_view.page_table
+            k, v, table, stride = kv_view.k, kv_view.v, kv_view.page_table, kv_view.page_stride
         return ops.rope_store(qkv, self.inv_freq, self.rotary_dim, self.pairing == "half", ctx.pos, ctx.tok_slot,
-                              table, k, v, n_heads, n_kv_heads, head_dim, self.dtype)
+                              table, stride, k, v, n_heads, n_kv_heads, head_dim, self.dtype)
 
 
 @register_position("none")
@@ -42,8 +42,8 @@ class NoPosition:
         self.dtype = dtype
 
     def rotate_store(self, qkv, ctx, kv_view, n_heads, n_kv_heads, head_dim):
-        k = v = table = None
+        k = v = table = stride = None
         if n_kv_heads > 0:
-            k, v, table = kv_view.k, kv_view.v, kv_view.page_table
-        return ops.rope_store(qkv, None, 0, False, ctx.pos, ctx.tok_slot, table, k, v, n_heads, n_kv_heads,
+            k, v, table, stride = kv_view.k, kv_view.v, kv_view.page_table, kv_view.page_stride
+        return ops.rope_store(qkv, None, 0, False, ctx.pos, ctx.tok_slot, table, stride, k, v, n_heads, n_kv_heads,
                               head_dim, self.dtype)

@@ -83,7 +83,14 @@ def rope(v: torch.Tensor, positions: torch.Tensor, theta: float, rotary_dim: int
     return out
 
 
-def attention(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, window: int | None = None) -> torch.Tensor:
+def _r(t: torch.Tensor, act_dtype) -> torch.Tensor:
+    """Rounds an activation to the dtype an engine stores it in (None: no rounding).  Only used to
+    measure what 16-bit storage of activations itself costs; the formulas are unchanged."""
+    return t if act_dtype is None else t.to(act_dtype).to(t.dtype)
+
+
+def attention(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, window: int | None = None,
+              act_dtype=None) -> torch.Tensor:
     """Causal grouped-query attention over one whole sequence.
 
     q [n, H, hd], k and v [n, K, hd] -> [n, H, hd].  Query head h reads KV head
@@ -103,7 +110,7 @@ def attention(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, window: int | N
             keys = k[lo:t + 1, g, :]
             s = (keys @ q[t, h, :]) / math.sqrt(hd)          # hpp:146-154
             s = torch.exp(s - s.max())                        # hpp:122-133
-            p = s / s.sum()                                   # hpp:135-137
+            p = _r(s, act_dtype) / s.sum()                    # hpp:135-137
             out[t, h, :] = p @ v[lo:t + 1, g, :]             # hpp:159-166
     return out
 
@@ -113,44 +120,46 @@ def silu(x: torch.Tensor) -> torch.Tensor:
     return x / (1.0 + torch.exp(-x))
 
 
-def swiglu(x: torch.Tensor, w_gate: torch.Tensor, w_up: torch.Tensor, w_down: torch.Tensor) -> torch.Tensor:
+def swiglu(x: torch.Tensor, w_gate: torch.Tensor, w_up: torch.Tensor, w_down: torch.Tensor,
+           act_dtype=None) -> torch.Tensor:
     """down(silu(gate(x)) * up(x)) (src/model/block.cpp:200-217)."""
-    return linear(silu(linear(x, w_gate)) * linear(x, w_up), w_down)
+    return linear(_r(silu(linear(x, w_gate)) * linear(x, w_up), act_dtype), w_down)
 
 
-def attention_part(x, w, prefix, s, positions, window=None):
+def attention_part(x, w, prefix, s, positions, window=None, act_dtype=None):
     """Projections, rotation of q and k, attention, output projection (block.cpp:125-167)."""
     n = x.shape[0]
     q = linear(x, w[prefix + "q_proj.weight"]).view(n, s["n_heads"], s["hd"])
     k = linear(x, w[prefix + "k_proj.weight"]).view(n, s["n_kv"], s["hd"])
     v = linear(x, w[prefix + "v_proj.weight"]).view(n, s["n_kv"], s["hd"])
-    q = rope(q, positions, s["theta"], s["rotary"])          # block.cpp:141
-    k = rope(k, positions, s["theta"], s["rotary"])          # block.cpp:142
-    a = attention(q, k, v, window).reshape(n, s["n_heads"] * s["hd"])
-    return linear(a, w[prefix + "o_proj.weight"])             # block.cpp:167
+    q = _r(rope(q, positions, s["theta"], s["rotary"]), act_dtype)          # block.cpp:141
+    k = _r(rope(k, positions, s["theta"], s["rotary"]), act_dtype)          # block.cpp:142
+    a = attention(q, k, _r(v, act_dtype), window, act_dtype).reshape(n, s["n_heads"] * s["hd"])
+    return linear(_r(a, act_dtype), w[prefix + "o_proj.weight"])            # block.cpp:167
 
 
-def block(x, w, i, s, positions):
+def block(x, w, i, s, positions, act_dtype=None):
     """Pre-norm decoder layer: x += attn(norm(x)); x += ffn(norm(x)) (block.cpp:106-224)."""
     p = f"model.layers.{i}."
-    h = rmsnorm(x, w[p + "input_layernorm.weight"], s["eps"])                     # block.cpp:113-119
-    x = x + attention_part(h, w, p + "self_attn.", s, positions)                  # block.cpp:170-172
-    h = rmsnorm(x, w[p + "post_attention_layernorm.weight"], s["eps"])            # block.cpp:177-183
+    h = _r(rmsnorm(x, w[p + "input_layernorm.weight"], s["eps"]), act_dtype)      # block.cpp:113-119
+    x = x + attention_part(h, w, p + "self_attn.", s, positions, None, act_dtype)  # block.cpp:170-172
+    h = _r(rmsnorm(x, w[p + "post_attention_layernorm.weight"], s["eps"]), act_dtype)   # block.cpp:177-183
     x = x + swiglu(h, w[p + "mlp.gate_proj.weight"], w[p + "mlp.up_proj.weight"],
-                   w[p + "mlp.down_proj.weight"])                                  # block.cpp:220-222
+                   w[p + "mlp.down_proj.weight"], act_dtype)                       # block.cpp:220-222
     return x
 
 
-def forward(weights: dict, cfg: dict, tokens, dtype=torch.float32) -> torch.Tensor:
-    """Logits [n, vocab] at every position of one whole sequence (model.cpp:60-99)."""
+def forward(weights: dict, cfg: dict, tokens, dtype=torch.float32, act_dtype=None) -> torch.Tensor:
+    """Logits [n, vocab] at every position of one whole sequence (model.cpp:60-99).
+    ``act_dtype`` rounds the activations that a 16-bit engine stores between its kernels."""
     s = sizes(cfg)
     w = {k: v.to(dtype) for k, v in weights.items()}
     tokens = torch.as_tensor(tokens, dtype=torch.long)
     positions = torch.arange(tokens.numel())
     x = embed(w["model.embed_tokens.weight"], tokens)
     for i in range(s["n_layers"]):
-        x = block(x, w, i, s, positions)
-    x = rmsnorm(x, w["model.norm.weight"], s["eps"])                               # model.cpp:79-90
+        x = block(x, w, i, s, positions, act_dtype)
+    x = _r(rmsnorm(x, w["model.norm.weight"], s["eps"]), act_dtype)                # model.cpp:79-90
     head = w["model.embed_tokens.weight"] if s["tied"] or "lm_head.weight" not in w else w["lm_head.weight"]
     return linear(x, head)                                                          # model.cpp:93-98
 
