@@ -1,0 +1,159 @@
+#!/usr/bin/env python3
+"""Decode and prefill throughput of the Llama-3.1-8B shape with random weights on one MI355X.
+
+    python bench.py --gpus 1 --steps K --warmup W
+
+A step is one decode step of the generation loop's own runner (bookkeeping, the
+model's forward pass from the cache, sampling, tokens back to the host) for a
+batch of 8 sequences whose contexts end at the benchmark's context length.  The
+line printed also holds the prefill of one 2,048-token prompt, the decode step's
+share of the HBM roofline, and decode throughput at batch 1 and 64.
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+# MI355X published peaks
+HBM_BYTES_S = 8.0e12
+PEAK_FLOPS = {"fp16": 2.5e15, "bf16": 2.5e15, "fp32": 157.3e12}
+
+# Llama-3.1-8B shape
+SHAPE = dict(num_hidden_layers=32, hidden_size=4096, num_attention_heads=32, num_key_value_heads=8,
+             head_dim=128, intermediate_size=14336, vocab_size=128256, rope_theta=500000.0,
+             rms_norm_eps=1e-5, max_position_embeddings=8192, tie_word_embeddings=False,
+             hidden_act="silu", architectures=["LlamaForCausalLM"])
+
+
+def main() -> int:
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=64)
+    ap.add_argument("--warmup", type=int, default=8)
+    ap.add_argument("--batch", type=int, default=8)
+    ap.add_argument("--context", type=int, default=8192)
+    ap.add_argument("--layers", type=int, default=32, help="fewer layers than the shape has (named in config)")
+    ap.add_argument("--dtype", default="fp16", choices=["fp16", "bf16"])
+    ap.add_argument("--prefill-tokens", type=int, default=2048)
+    ap.add_argument("--points", default="1,64", help="further decode batch sizes, comma separated ('' for none)")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print(f"bench.py: this library runs on one GPU; --gpus {args.gpus} is not supported")
+        return 2
+
+    import torch
+
+    import llm_infer_amd
+    from llm_infer_amd.sampling import Sampler
+
+    raw = dict(SHAPE, num_hidden_layers=args.layers, max_position_embeddings=args.context)
+    cfg = llm_infer_amd.config_from_dict(raw)
+    points = [int(p) for p in args.points.split(",") if p]
+    batches = [args.batch] + [p for p in points if p != args.batch]
+    max_tokens = max(max(batches) * args.context, args.prefill_tokens) + 64 * max(batches)
+    t0 = time.time()
+    engine = llm_infer_amd.random_model(cfg, seed=0, dtype=args.dtype, max_tokens=max_tokens,
+                                        n_slots=max(batches))
+    torch.cuda.synchronize()
+    print(f"[bench] model ready in {time.time() - t0:.1f} s", file=sys.stderr, flush=True)
+    model, cache = engine.model, engine.cache
+    elem = 2
+
+    # bytes a decode step has to read: every matrix once, the norms, and the cache of the live requests
+    weight_bytes = 0
+    for name, spec in model.params().items():
+        n = 1
+        for s in spec.shape:
+            n *= s
+        if name.startswith("model.embed_tokens"):
+            continue                                   # only the batch's rows are read
+        weight_bytes += n * (4 if spec.kind == "vector" else elem)
+    kv_bytes_per_token = cache.bytes_per_token()
+
+    def decode_run(batch, steps, warmup):
+        """Fills `batch` sequences to just below the context length with random keys and values,
+        then times `steps` decode steps."""
+        start = args.context - steps - warmup - 1
+        slots = [engine.alloc_slot() for _ in range(batch)]
+        cache.grow(slots, [start] * batch)
+        for g in cache.groups:
+            g.storage.normal_(0.0, 1.0)
+        sampler = Sampler(temperature=0.0, seed=0)
+        sampler.start(cache, slots, list(range(batch)))
+        runner = engine.decode_runner(sampler, use_graph=True)
+        gen = torch.Generator().manual_seed(batch)
+        toks = torch.randint(0, cfg.vocab_size, (batch,), generator=gen).tolist()
+        for _ in range(warmup):
+            toks = runner.run(slots, toks)
+        torch.cuda.synchronize()
+        t = time.perf_counter()
+        for _ in range(steps):
+            toks = runner.run(slots, toks)
+        torch.cuda.synchronize()
+        dt = time.perf_counter() - t
+        ctx_mid = start + warmup + steps // 2
+        for s in slots:
+            engine.free_slot(s)
+        return dt, ctx_mid
+
+    results = {}
+    for b in batches:
+        dt, ctx_mid = decode_run(b, args.steps, args.warmup)
+        results[b] = (dt, ctx_mid)
+        print(f"[bench] decode batch {b}: {dt / args.steps * 1e3:.3f} ms/step, "
+              f"{b * args.steps / dt:.1f} tok/s", file=sys.stderr, flush=True)
+
+    # prefill of one prompt
+    T = args.prefill_tokens
+    gen = torch.Generator().manual_seed(1)
+    prompt = torch.randint(0, cfg.vocab_size, (T,), generator=gen).tolist()
+    times = []
+    for i in range(4):
+        slot = engine.alloc_slot()
+        torch.cuda.synchronize()
+        t = time.perf_counter()
+        engine.step([slot], [prompt])
+        torch.cuda.synchronize()
+        times.append(time.perf_counter() - t)
+        engine.free_slot(slot)
+    prefill_s = min(times[1:])
+    L, d, H, K, hd, F, V = (cfg.num_hidden_layers, cfg.hidden_size, cfg.num_attention_heads,
+                            cfg.num_key_value_heads, cfg.head_dim, cfg.intermediate_size, cfg.vocab_size)
+    gemm = 2 * T * (d * (H + 2 * K) * hd + H * hd * d + 3 * d * F) * L + 2 * V * d
+    attn = 2 * H * hd * T * (T + 1) * L
+    prefill_flops = gemm + attn
+
+    dt, ctx_mid = results[args.batch]
+    ms = dt / args.steps * 1e3
+    step_bytes = weight_bytes + args.batch * d * elem + kv_bytes_per_token * ctx_mid * args.batch
+    achieved = step_bytes / (dt / args.steps)
+    line = {
+        "metric": f"decode tokens/s, Llama-3.1-8B shape, batch {args.batch}, context {args.context}",
+        "value": round(args.batch * args.steps / dt, 2), "unit": "tokens/s", "n_gpus": 1,
+        "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(ms, 4),
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": args.dtype,
+        "data": "synthetic: random weights N(0, 0.02), uniform random token ids, cache filled with random "
+                "keys and values up to the context length",
+        "config": {
+            "model": "Llama-3.1-8B shape", "layers": L, "layers_of_shape": SHAPE["num_hidden_layers"],
+            "hidden": d, "heads": H, "kv_heads": K, "head_dim": hd, "intermediate": F, "vocab": V,
+            "rope_theta": cfg.rope_theta, "rms_norm_eps": cfg.rms_norm_eps, "tied": cfg.tie_word_embeddings,
+            "global_batch": args.batch, "seq_len": args.context, "context": args.context,
+            "prefill_tokens": T, "parallelism": "1 GPU", "sampling": "greedy",
+        },
+        "prefill": {"value": round(T / prefill_s, 1), "tokens": T, "ms": round(prefill_s * 1e3, 3),
+                    "frac": round(prefill_flops / prefill_s / PEAK_FLOPS[args.dtype], 4)},
+        "roofline": {"bound": "hbm", "achieved": round(achieved / 1e9, 1), "peak": HBM_BYTES_S / 1e9,
+                     "unit": "GB/s", "frac": round(achieved / HBM_BYTES_S, 4)},
+        "points": {f"decode_b{b}": round(b * args.steps / results[b][0], 2) for b in batches if b != args.batch},
+    }
+    print(json.dumps(line))
+    return 0
+
+
+if __name__ == "__main__":
+    sys.exit(main())

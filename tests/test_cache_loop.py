@@ -1,0 +1,195 @@
+"""The cache's bookkeeping and the generation loop's decisions (no GPU)."""
+import random
+
+import pytest
+import torch
+
+from llm_infer_amd.cache import Cache, CacheError, KVSpec, PagePool, SlotAllocator, StateSpec
+from llm_infer_amd.config.spec import ConfigError, ModelSpec, PartSpec, ScheduleEntry
+from llm_infer_amd.engine.generate import BatchTracker, RequestError, plan_batches
+from llm_infer_amd.engine.step import decode_splits
+from llm_infer_amd.cli import parse_args
+from llm_infer_amd.tokenizer import Tokenizer
+
+
+def test_slots_are_neither_lost_nor_held_twice_nor_freed_twice():
+    a = SlotAllocator(4)
+    got = [a.alloc() for _ in range(4)]
+    assert sorted(got) == [0, 1, 2, 3] and a.n_free == 0
+    with pytest.raises(CacheError, match="in use"):
+        a.alloc()
+    a.free(2)
+    with pytest.raises(CacheError, match="not held"):
+        a.free(2)
+    with pytest.raises(CacheError, match="not held"):
+        a.free(7)
+    assert a.alloc() == 2
+    rng = random.Random(0)
+    held = set(got)
+    for _ in range(2000):
+        if held and (rng.random() < 0.5 or a.n_free == 0):
+            s = rng.choice(sorted(held))
+            a.free(s)
+            held.remove(s)
+        else:
+            s = a.alloc()
+            assert s not in held
+            held.add(s)
+        assert a.held() == held and a.n_free + len(held) == 4
+
+
+def test_a_following_batch_uses_the_same_slots_again():
+    a = SlotAllocator(8)
+    first = [a.alloc() for _ in range(3)]
+    for s in first:
+        a.free(s)
+    assert [a.alloc() for _ in range(3)] == first
+
+
+def test_pages():
+    p = PagePool(6, first=1)
+    x = p.alloc(3)
+    assert len(set(x)) == 3 and 0 not in x and p.n_free == 2
+    with pytest.raises(CacheError, match="cache is full"):
+        p.alloc(3)
+    p.free(x[:1])
+    with pytest.raises(CacheError, match="not held"):
+        p.free(x[:1])
+    assert p.n_free == 3 and p.held() == set(x[1:])
+
+
+def _cache(specs, max_tokens=640, max_pos=512, slots=4):
+    return Cache(specs, max_tokens, max_pos, torch.bfloat16, None, slots)
+
+
+def test_cache_groups_lengths_and_page_accounting():
+    full, win = KVSpec(2, 16), KVSpec(2, 16, window=100)
+    c = _cache([full, win, None, full, StateSpec((3, 4))])
+    assert len(c.groups) == 3
+    kv_full = next(g for g in c.groups if getattr(g, "spec", None) == full)
+    kv_win = next(g for g in c.groups if getattr(g, "spec", None) == win)
+    assert kv_full.entries == [0, 3] and kv_win.entries == [1] and c.view(2) is None
+    assert kv_full.page_elems == 2 * (2 * 64 * 16 + 2 * 64 * 32)       # values padded to 32 dims
+    s0, s1 = c.alloc_slot(), c.alloc_slot()
+    c.grow([s0, s1], [130, 1])
+    assert c.lens[s0] == 130 and c.lens[s1] == 1
+    assert len(kv_full.pages_of[s0]) == 3 and len(kv_full.pages_of[s1]) == 1
+    assert kv_full.table_host[s0, :3].tolist() == [kv_full.pages_of[s0][i] for i in range(3)]
+    assert c.tokens_free() == 640 - 4 * 64
+    # a window group gives back pages that no later token can read
+    c.grow([s0], [300])
+    c.trim_windows([s0])
+    assert sorted(kv_win.pages_of[s0]) == [3, 4] and kv_win.table_host[s0, 0] == 0
+    assert sorted(kv_full.pages_of[s0]) == [0, 1, 2, 3, 4]
+    with pytest.raises(CacheError, match="exceeds the model's 512 positions"):
+        c.grow([s0], [513])
+    with pytest.raises(CacheError, match="cache is full"):
+        c.grow([s1], [500])
+    c.free_slot(s0)
+    assert kv_full.pool.n_free == 10 - 1 and kv_win.pool.n_free == 10 - 1 and c.lens[s0] == 0
+    with pytest.raises(CacheError, match="not held"):
+        c.free_slot(s0)
+    with pytest.raises(CacheError, match="not held"):
+        c.grow([s0], [5])
+    c.free_slot(s1)
+    assert kv_full.pool.n_free == 10 and not kv_full.pool.held() and c.slots.n_free == 4
+
+
+def test_random_sequences_never_share_a_page():
+    c = _cache([KVSpec(1, 16)], max_tokens=64 * 40, max_pos=64 * 12, slots=6)
+    g = c.groups[0]
+    rng = random.Random(1)
+    live = {}
+    for _ in range(600):
+        if live and rng.random() < 0.3:
+            s = rng.choice(sorted(live))
+            c.free_slot(s)
+            del live[s]
+        elif len(live) < 6 and rng.random() < 0.5:
+            live[c.alloc_slot()] = 0
+        elif live:
+            s = rng.choice(sorted(live))
+            n = min(64 * 12, live[s] + rng.randint(1, 90))
+            try:
+                c.grow([s], [n])
+                live[s] = n
+            except CacheError:
+                pass
+        pages = [p for s in live for p in g.pages_of[s].values()]
+        assert len(pages) == len(set(pages)) and 0 not in pages
+        assert set(pages) == g.pool.held()
+        for s, n in live.items():
+            assert len(g.pages_of[s]) == -(-n // 64) and c.lens[s] == n
+
+
+def test_schedule_validation():
+    def spec(schedule, n_layers=2):
+        ps = PartSpec("x")
+        from llm_infer_amd.config.spec import LayerSpec
+        layer = LayerSpec("pre_norm", ps, ps, ps, ps)
+        return ModelSpec(8, 8, 8, ps, tuple([layer] * n_layers), tuple(schedule), ps, ps)
+    spec([ScheduleEntry(0), ScheduleEntry(1), ScheduleEntry(0), ScheduleEntry(1, cache_from=1)]).validate()
+    with pytest.raises(ConfigError, match="names layer 5"):
+        spec([ScheduleEntry(5)]).validate()
+    with pytest.raises(ConfigError, match="does not run before"):
+        spec([ScheduleEntry(0, cache_from=1), ScheduleEntry(1)]).validate()
+    with pytest.raises(ConfigError, match="keeps none of its own"):
+        spec([ScheduleEntry(0), ScheduleEntry(1, cache_from=0), ScheduleEntry(0, cache_from=1)]).validate()
+
+
+def test_plan_batches():
+    assert plan_batches([5, 6, 7, 8, 9], 10, 2, 10_000, 100) == [[0, 1], [2, 3], [4]]
+    assert plan_batches([60, 60, 60], 10, 8, 256, 1000) == [[0, 1], [2]]         # 128 tokens each
+    assert plan_batches([10, 10], 1000, 8, 128, 64) == [[0, 1]]                  # capped by the context
+    with pytest.raises(RequestError, match="Prompt too long: 100 tokens \\(max: 100\\)"):
+        plan_batches([100], 1, 1, 10_000, 100)
+    with pytest.raises(RequestError, match="empty prompt"):
+        plan_batches([3, 0], 1, 1, 10_000, 100)
+    with pytest.raises(RequestError, match="needs room"):
+        plan_batches([200], 100, 1, 256, 1000)
+
+
+def test_the_loop_decisions():
+    t = BatchTracker([3, 5, 2], max_new_tokens=3, stop_token_ids={9}, max_positions=6)
+    assert t.live() == [0, 1, 2]
+    go = t.accept([0, 1, 2], [4, 9, 7])           # request 1 samples the stop token at once
+    assert go == [0, 2] and t.outputs == [[4], [], [7]] and t.reason[1] == "stop"
+    go = t.accept([0, 2], [5, 8])
+    assert go == [0, 2]
+    go = t.accept([0, 2], [6, 9])                 # request 0 reaches its budget: no forward after the last
+    assert go == [] and t.outputs == [[4, 5, 6], [], [7, 8]] and t.reason == ["length", "stop", "stop"]
+    with pytest.raises(RuntimeError):
+        t.accept([0], [1])
+    t = BatchTracker([5], 10, (), max_positions=6)
+    assert t.accept([0], [1]) == [0]              # the token fits at position 5
+    assert t.accept([0], [2]) == [] and t.reason == ["context"] and t.outputs == [[1, 2]]
+    t = BatchTracker([5], 0, (), 100)
+    assert t.live() == [] and t.reason == ["length"]
+
+
+def test_decode_splits_fill_the_chip_and_are_powers_of_two():
+    assert decode_splits(1, 8, 32, 8192) == 64
+    assert decode_splits(8, 8, 32, 8192) == 16
+    assert decode_splits(64, 8, 32, 8192) == 2
+    assert decode_splits(64, 32, 32, 4096) == 1
+    assert decode_splits(1, 8, 32, 100) == 1 and decode_splits(1, 1, 64, 640) == 4
+
+
+def test_command_line_follows_the_reference():
+    c = parse_args(["m", "-i", "hi", "-n", "5", "-t", "0.5", "--seed", "7", "-T", "99"])
+    assert (c["model"], c["prompt"], c["max_tokens"], c["temperature"], c["seed"], c["context"]) == \
+        ("m", "hi", 5, 0.5, 7, 99)
+    c = parse_args(["m", "--tokens", "1,2,3", "--tokens", "4 5"])
+    assert c["tokens"] == [[1, 2, 3], [4, 5]] and c["max_tokens"] == 256 and c["temperature"] == 1.0
+    assert parse_args(["m"]) is None and parse_args([]) is None
+    assert parse_args(["m", "-i", "a", "-f", "b"]) is None and parse_args(["m", "-i", "a", "--bogus"]) is None
+    assert parse_args(["m", "-i", "a", "-d", "cuda"]) is None and parse_args(["-h"])["help"]
+
+
+def test_tokenizer_longest_match_and_bytes():
+    vocab = {"<s>": 0, "</s>": 1, "a": 2, "ab": 3, "abc": 4, "▁b": 5, "c": 6, "<|eot_id|>": 300}
+    vocab.update({f"<0x{i:02X}>": 10 + i for i in range(256)})
+    t = Tokenizer(vocab, bos_id=0, eos_id=1)
+    assert t.encode("abcab b", True) == [0, 4, 3, 5] and t.encode("abd", False) == [3, 10 + ord("d")]
+    assert t.eot_id == 300 and t.decode([0, 5, 4, 10 + ord("!")]) == "<s>babc!"    # no blank after BOS
+    assert t.decode(t.encode("cab é", False)) == "cab é"

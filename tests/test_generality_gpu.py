@@ -1,0 +1,440 @@
+"""Each part alone against the plain implementation; long decoding; the first tokens; slots and
+pages used again; batch composition; sampling through the entry points; and a toy architecture
+(a mixer with state of its own, a layer named twice, a layer that reads another's cache) that is
+registered, built and stepped without touching the framework's files."""
+import json
+import os
+import subprocess
+import sys
+
+import numpy as np
+import pytest
+import torch
+
+import plain_llama as P
+from tiny_configs import TINY_A, TINY_B, TINY_C
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda"
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def sharp_weights(cfg, seed):
+    w = P.random_weights(cfg, seed, std=0.05)
+    for name in w:
+        if "q_proj" in name or "k_proj" in name:
+            w[name] = (w[name].float() * 2).to(w[name].dtype)
+    return w
+
+
+@pytest.fixture(scope="module")
+def lib():
+    import llm_infer_amd
+    return llm_infer_amd
+
+
+@pytest.fixture(scope="module")
+def folders(tmp_path_factory):
+    out = {}
+    for name, cfg in (("A", TINY_A), ("B", TINY_B), ("C", TINY_C)):
+        d = str(tmp_path_factory.mktemp(f"gen_{name}"))
+        P.write_model(d, cfg, sharp_weights(cfg, 11 + ord(name)))
+        out[name] = d
+    return out
+
+
+def _ctx(lens_before, tokens):
+    from llm_infer_amd.engine.step import StepContext
+    return StepContext(DEV, list(range(len(tokens))), tokens, lens_before, [[] for _ in tokens])
+
+
+# ---------------------------------------------------------------------------
+# the parts, each alone, at sizes of their own
+# ---------------------------------------------------------------------------
+@pytest.mark.parametrize("dt", [torch.float32, torch.bfloat16])
+def test_parts_alone(lib, dt):
+    from llm_infer_amd.cache import Cache
+    from llm_infer_amd.parts import Attention, Embedding, GatedMLP, LMHead, PreNormBlock, RMSNorm, RotaryPosition
+    d, H, K, hd, F, V, eps, theta, rot = 112, 6, 3, 32, 200, 77, 1e-3, 777.0, 16
+    g = torch.Generator().manual_seed(4)
+    tol = 2e-5 if dt == torch.float32 else 3e-2
+
+    def mat(*shape, s=0.1):
+        return (torch.randn(*shape, generator=g) * s).to(torch.bfloat16)
+
+    w = {"n1.weight": 1 + 0.1 * torch.randn(d, generator=g), "n2.weight": 1 + 0.1 * torch.randn(d, generator=g),
+         "a.q_proj.weight": mat(H * hd, d), "a.k_proj.weight": mat(K * hd, d), "a.v_proj.weight": mat(K * hd, d),
+         "a.o_proj.weight": mat(d, H * hd), "f.gate_proj.weight": mat(F, d), "f.up_proj.weight": mat(F, d),
+         "f.down_proj.weight": mat(d, F), "e.weight": mat(V, d, s=1.0)}
+    dev = {k: v.to(DEV).to(torch.float32 if (v.dim() == 1 or dt == torch.float32) else dt) for k, v in w.items()}
+    w64 = {k: v.double() for k, v in w.items()}
+    norm1 = RMSNorm(size=d, eps=eps, prefix="n1.", dtype=dt, device=DEV)
+    norm2 = RMSNorm(size=d, eps=eps, prefix="n2.", dtype=dt, device=DEV)
+    pos = RotaryPosition(theta=theta, rotary_dim=rot, head_dim=hd, dtype=dt, device=DEV)
+    attn = Attention(hidden_size=d, n_heads=H, n_kv_heads=K, head_dim=hd, scale=hd ** -0.5, position=pos,
+                     prefix="a.", dtype=dt, device=DEV)
+    ffn = GatedMLP(hidden_size=d, intermediate_size=F, prefix="f.", dtype=dt, device=DEV)
+    emb = Embedding(vocab_size=V, hidden_size=d, prefix="e.", dtype=dt, device=DEV)
+    head = LMHead(vocab_size=V, hidden_size=d, tied=True, prefix="h.", dtype=dt, device=DEV)
+    for part in (norm1, norm2, attn, ffn, emb):
+        assert all(tuple(dev[part.prefix + n].shape) == tuple(s.shape) for n, s in part.params().items())
+        part.bind({n: dev[part.prefix + n] for n in part.params()})
+    head.tie(emb.weight)
+    assert head.params() == {} and head.ignorable() == ["h.weight"]
+
+    lens = [70, 3]
+    toks = [torch.randint(0, V, (n,), generator=g).tolist() for n in lens]
+    ctx = _ctx([0, 0], toks)
+    # embedding
+    x = emb.forward(ctx.token_ids)
+    x_ref = torch.cat([w64["e.weight"][t] for t in toks])
+    assert torch.equal(x.double().cpu(), x_ref)
+    # norm
+    h = norm1.forward(x)
+    h_ref = P.rmsnorm(x_ref, w64["n1.weight"], eps)
+    assert h.dtype == dt and (h.double().cpu() - h_ref).abs().max() < tol * 4
+    # feed-forward (adds into the residual)
+    res = x.clone()
+    ffn.forward(h, res)
+    f_ref = P.swiglu(h.double().cpu(), w64["f.gate_proj.weight"], w64["f.up_proj.weight"], w64["f.down_proj.weight"])
+    assert (res.double().cpu() - (x_ref + f_ref)).abs().max() < tol * (1 + f_ref.abs().max())
+    # attention over a fresh cache, two sequences of unequal length in one step
+    cache = Cache([attn.cache_spec()], 256, 128, dt, DEV, 2)
+    slots = [cache.alloc_slot(), cache.alloc_slot()]
+    cache.grow(slots, lens)
+    res = x.clone()
+    attn.forward(h, ctx, cache.view(0), res)
+    s = dict(n_heads=H, n_kv=K, hd=hd, theta=theta, rotary=rot)
+    wa = {k: v for k, v in w64.items()}
+    off, a_ref = 0, []
+    for n in lens:
+        a_ref.append(P.attention_part(h.double().cpu()[off:off + n], wa, "a.", s, torch.arange(n)))
+        off += n
+    a_ref = torch.cat(a_ref)
+    assert (res.double().cpu() - (x_ref + a_ref)).abs().max() < tol * (1 + a_ref.abs().max())
+    # the whole block on fresh slots equals norm -> attention -> norm -> feed-forward
+    for sl in slots:
+        cache.free_slot(sl)
+    slots = [cache.alloc_slot(), cache.alloc_slot()]
+    cache.grow(slots, lens)
+    blk = PreNormBlock(norm1, attn, norm2, ffn)
+    xb = x.clone()
+    blk.forward(xb, ctx, cache.view(0))
+    wb = {"model.layers.0.input_layernorm.weight": w64["n1.weight"],
+          "model.layers.0.post_attention_layernorm.weight": w64["n2.weight"]}
+    for k in ("q_proj", "k_proj", "v_proj", "o_proj"):
+        wb[f"model.layers.0.self_attn.{k}.weight"] = w64[f"a.{k}.weight"]
+    for k in ("gate_proj", "up_proj", "down_proj"):
+        wb[f"model.layers.0.mlp.{k}.weight"] = w64[f"f.{k}.weight"]
+    s.update(eps=eps)
+    off, b_ref = 0, []
+    for n in lens:
+        b_ref.append(P.block(x_ref[off:off + n], wb, 0, s, torch.arange(n)))
+        off += n
+    b_ref = torch.cat(b_ref)
+    assert (xb.double().cpu() - b_ref).abs().max() < tol * (1 + b_ref.abs().max()) * 2
+    # head on chosen rows
+    rows = torch.tensor([69, 72, 0], dtype=torch.int32, device=DEV)
+    logits = head.forward(norm2.forward(xb, rows))
+    l_ref = P.linear(P.rmsnorm(xb.double().cpu()[rows.long().cpu()], w64["n2.weight"], eps), w64["e.weight"])
+    assert logits.dtype == torch.float32 and (logits.double().cpu() - l_ref).abs().max() < tol * (1 + l_ref.abs().max())
+
+
+# ---------------------------------------------------------------------------
+# long decoding, the first tokens, graph replay
+# ---------------------------------------------------------------------------
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_long_decoding_and_first_tokens(lib, folders, dtype):
+    cfg, folder = TINY_C, folders["C"]
+    weights = P.load_weights(folder)
+    n = 700
+    toks = torch.randint(0, cfg["vocab_size"], (n,), generator=torch.Generator().manual_seed(2)).tolist()
+    ref = P.forward(weights, cfg, toks, torch.float64)
+    own = (P.forward(weights, cfg, toks, torch.float32) if dtype == "float32"
+           else P.forward(weights, cfg, toks, torch.float64, torch.bfloat16))
+    tol = 3 * (own.double() - ref).abs().max().item() + 1e-6
+    eng = lib.load(folder, dtype=dtype, max_tokens=2048)
+    s = eng.alloc_slot()
+    got = [eng.step([s], [toks[:1]])[0]]                       # the very first token alone
+    for p in range(1, n):                                      # then 699 tokens one by one, across 11 pages
+        got.append(eng.step([s], [[toks[p]]])[0])
+    got = torch.stack(got).double().cpu()
+    err = (got - ref).abs().max(dim=1).values
+    assert err.max().item() < tol, f"first wrong place: {int((err >= tol).nonzero()[0])}"
+    assert err[:4].max().item() < tol                          # positions 0..3
+    eng.free_slot(s)
+    # a 2-token prompt in one step: both places
+    s = eng.alloc_slot()
+    two = eng.step([s], [toks[:2]], [[0, 1]]).double().cpu()
+    assert (two - ref[:2]).abs().max().item() < tol
+    eng.free_slot(s)
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_recorded_steps_replay_like_eager_steps(lib, folders, dtype):
+    """Greedy generation of 150 tokens for a ragged batch whose sequences end at different times:
+    the recorded (graph) runner and the eager runner must give the same tokens, replay after replay."""
+    eng = lib.load(folders["C"], dtype=dtype, max_tokens=8192)
+    g = torch.Generator().manual_seed(3)
+    prompts = [torch.randint(0, 331, (n,), generator=g).tolist() for n in (5, 90, 33, 64)]
+    plain_tokens = eng.generate(prompts, max_new_tokens=150, temperature=0.0, use_graph=False)
+    stop = {plain_tokens[1][40], plain_tokens[2][100]}          # make two sequences end early
+    a = eng.generate(prompts, max_new_tokens=150, temperature=0.0, use_graph=False, stop_token_ids=stop)
+    b = eng.generate(prompts, max_new_tokens=150, temperature=0.0, use_graph=True, stop_token_ids=stop)
+    c = eng.generate(prompts, max_new_tokens=150, temperature=0.0, use_graph=True, stop_token_ids=stop)
+    assert a == b == c
+    assert len(a[1]) <= 40 and len(a[2]) <= 100 and len(a[0]) <= 150
+    assert all(t not in stop for o in a for t in o)
+    t1 = eng.generate(prompts, max_new_tokens=40, temperature=0.7, seed=5, use_graph=False)
+    t2 = eng.generate(prompts, max_new_tokens=40, temperature=0.7, seed=5, use_graph=True)
+    assert t1 == t2
+    assert eng.cache.slots.n_free == eng.cache.n_slots and eng.cache.tokens_free() == (eng.cache.n_pages - 1) * 64
+
+
+# ---------------------------------------------------------------------------
+# slots and pages used again, batch composition
+# ---------------------------------------------------------------------------
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_reused_slots_and_batch_composition(lib, folders, dtype):
+    cfg, folder = TINY_B, folders["B"]
+    eng = lib.load(folder, dtype=dtype, max_tokens=64 * 6, n_slots=3)
+    g = torch.Generator().manual_seed(9)
+    reqs = [torch.randint(0, cfg["vocab_size"], (n,), generator=g).tolist() for n in (100, 17, 64, 65, 1, 30)]
+
+    def alone(toks):
+        s = eng.alloc_slot()
+        out = eng.step([s], [toks], [list(range(len(toks)))]).clone()
+        eng.free_slot(s)
+        return out
+
+    base = [alone(t) for t in reqs]
+    # poison everything that is free: a sequence that starts in a used slot and used pages sees none of it
+    for grp in eng.cache.groups:
+        grp.storage.fill_(float("nan"))
+    again = [alone(t) for t in reqs]
+    for x, y in zip(base, again):
+        assert torch.equal(x, y)
+    # batches of three with unequal lengths, in two orders: same logits for every request
+    for order in ([0, 1, 2, 3, 4, 5], [4, 3, 5, 2, 0, 1]):
+        for b in range(0, 6, 3):
+            ids = order[b:b + 3]
+            slots = [eng.alloc_slot() for _ in ids]
+            out = eng.step(slots, [reqs[i] for i in ids], [list(range(len(reqs[i]))) for i in ids])
+            off = 0
+            for i in ids:
+                part = out[off:off + len(reqs[i])]
+                off += len(reqs[i])
+                if dtype == "float32":
+                    assert torch.equal(part, base[i]), "32-bit results do not depend on the batch"
+                else:
+                    assert (part - base[i]).abs().max().item() < 2e-2 * base[i].std().item()
+            for s in slots:
+                eng.free_slot(s)
+    with pytest.raises(Exception, match="cache is full|in use"):
+        slots = [eng.alloc_slot() for _ in range(3)]
+        eng.step(slots, [reqs[0] + reqs[0], reqs[0] + reqs[0], reqs[0] + reqs[0]])
+
+
+def test_requests_are_checked(lib, folders):
+    eng = lib.load(folders["A"], dtype="bfloat16", max_tokens=256)
+    s = eng.alloc_slot()
+    with pytest.raises(ValueError, match="token id outside"):
+        eng.step([s], [[1, 256]])
+    with pytest.raises(ValueError, match="brings no token"):
+        eng.step([s], [[]])
+    with pytest.raises(ValueError, match="wanted place"):
+        eng.step([s], [[1, 2]], [[2]])
+    with pytest.raises(Exception, match="exceeds the model's 128 positions"):
+        eng.step([s], [list(range(129))])
+    from llm_infer_amd.engine.generate import RequestError
+    with pytest.raises(RequestError, match="Prompt too long: 128 tokens \\(max: 128\\)"):
+        eng.generate([list(range(128))], max_new_tokens=1)
+
+
+# ---------------------------------------------------------------------------
+# sampling through the entry points
+# ---------------------------------------------------------------------------
+def test_temperature_sampling_follows_the_plain_sampler(lib, folders):
+    """float32 engine, T = 0.8: every token equals the plain sampler's choice for the same uniform
+    number, unless that number falls within rounding of a boundary of the cumulative distribution."""
+    from llm_infer_amd.sampling import Sampler
+    cfg, folder = TINY_B, folders["B"]
+    weights = P.load_weights(folder)
+    eng = lib.load(folder, dtype="float32", max_tokens=1024)
+    prompts = [[5], [1, 2, 3, 4], list(range(10, 19)), list(range(40, 56)), list(range(100, 131))]
+    T, seed, n_new = 0.8, 1, 12
+    out = eng.generate(prompts, max_new_tokens=n_new, temperature=T, seed=seed, stop_token_ids=())
+    sampler = Sampler(T, seed)
+    for r_idx, (p, o) in enumerate(zip(prompts, out)):
+        assert len(o) == n_new
+        toks = list(p)
+        for k, t in enumerate(o):
+            logits = P.forward(weights, cfg, toks, torch.float64)[-1]
+            r = sampler.uniform(r_idx, k)
+            c = torch.cumsum(P.probabilities(logits, T), 0)
+            if (c - r).abs().min().item() > 1e-5:
+                assert t == P.sample_temperature(logits, T, r), (r_idx, k)
+            toks.append(t)
+    # a request's tokens do not depend on the batch it runs in, only on (seed, request index)
+    alone = eng.generate([prompts[0]], max_new_tokens=n_new, temperature=T, seed=seed, stop_token_ids=())
+    assert alone[0] == out[0]
+    other = eng.generate(prompts, max_new_tokens=n_new, temperature=T, seed=seed + 1, stop_token_ids=())
+    assert other != out
+    # one batch after another: a single slot serves all five requests
+    small = lib.load(folder, dtype="float32", max_tokens=64, n_slots=1)
+    serial, stats = small.generate(prompts, max_new_tokens=n_new, temperature=T, seed=seed, stop_token_ids=(),
+                                   return_stats=True)
+    assert serial == out and stats.batches == 5
+
+
+def test_command_line_generates_greedily(folders):
+    cfg, folder = TINY_A, folders["A"]
+    weights = P.load_weights(folder)
+    prompts = [[3, 14, 15, 92, 65, 35, 89], [7], list(range(20, 33))]
+    cmd = [sys.executable, os.path.join(ROOT, "bin", "infer"), folder, "-n", "8", "-t", "0", "--dtype", "float32"]
+    for p in prompts:
+        cmd += ["--tokens", ",".join(map(str, p))]
+    res = subprocess.run(cmd, capture_output=True, text=True, timeout=300)
+    assert res.returncode == 0, res.stderr
+    got = [json.loads(line.split("tokens: ", 1)[1]) for line in res.stdout.splitlines() if " tokens: [" in line]
+    assert got == [P.generate_greedy(weights, cfg, p, 8) for p in prompts]
+    for word in ("Loading model:", "Layers: 2", "KV Heads: 2", "Prefilling...", "Generation Statistics:",
+                 "Prompt tokens: 21", "Generated tokens: 24", "Temperature: 0.00"):
+        assert word in res.stdout
+    bad = subprocess.run([sys.executable, os.path.join(ROOT, "bin", "infer"), folder + "_nope", "--tokens", "1"],
+                         capture_output=True, text=True, timeout=300)
+    assert bad.returncode == 1 and "Error:" in bad.stderr
+
+
+# ---------------------------------------------------------------------------
+# a toy architecture, defined here
+# ---------------------------------------------------------------------------
+def test_toy_architecture_with_a_stateful_mixer(lib):
+    from llm_infer_amd.cache import StateSpec
+    from llm_infer_amd.config.spec import LayerSpec, ModelSpec, PartSpec, ScheduleEntry
+    from llm_infer_amd.engine import Engine
+    from llm_infer_amd.parts.base import Part
+    from llm_infer_amd.weights.loader import ParamSpec
+
+    @lib.register_mixer("toy_decay")
+    class DecayMixer(Part):
+        """s <- decay * s + W_in h ;  out = W_out s, with s kept per sequence in the cache."""
+
+        def __init__(self, *, hidden_size, state_size, decay, position=None, prefix, dtype, device):
+            self.d, self.n, self.decay, self.prefix, self.dtype = hidden_size, state_size, decay, prefix, dtype
+
+        def params(self):
+            return {"in.weight": ParamSpec((self.n, self.d)), "out.weight": ParamSpec((self.d, self.n))}
+
+        def bind(self, tensors):
+            self.w_in, self.w_out = tensors["in.weight"].float(), tensors["out.weight"].float()
+
+        def cache_spec(self):
+            return StateSpec((self.n,), "float32")
+
+        def forward(self, h, ctx, cache_view, residual, owns_cache=True):
+            u = h.float() @ self.w_in.t()
+            y = torch.empty_like(u)
+            row = 0
+            for slot, n in zip(ctx.host_slots, ctx.host_qlens):
+                s = cache_view.state[slot].clone()
+                for _ in range(n):
+                    s = self.decay * s + u[row]
+                    y[row] = s
+                    row += 1
+                cache_view.state[slot] = s
+            residual += y @ self.w_out.t()
+
+    class ToyConfig:
+        def __init__(self, raw):
+            self.raw = raw
+
+        @classmethod
+        def from_dict(cls, raw):
+            return cls(raw)
+
+        def model_spec(self):
+            r = self.raw
+            d, hd = r["width"], r["head"]
+            norm = PartSpec("rmsnorm", {"size": d, "eps": r["eps"]})
+            ffn = PartSpec("gated_mlp", {"hidden_size": d, "intermediate_size": r["ffn"]})
+            toy = LayerSpec("pre_norm", PartSpec("toy_decay", {"hidden_size": d, "state_size": r["state"],
+                                                               "decay": r["decay"]}, "l0.mix."),
+                            ffn.with_prefix("l0.ffn."), norm.with_prefix("l0.n1."), norm.with_prefix("l0.n2."))
+            att = LayerSpec("pre_norm", PartSpec("attention", {"hidden_size": d, "n_heads": 2, "n_kv_heads": 1,
+                                                               "head_dim": hd, "scale": hd ** -0.5}, "l1.mix."),
+                            ffn.with_prefix("l1.ffn."), norm.with_prefix("l1.n1."), norm.with_prefix("l1.n2."),
+                            PartSpec("rope", {"theta": 100.0, "rotary_dim": hd, "head_dim": hd}))
+            # the toy layer runs twice (two states), the attention layer runs twice, its second run
+            # reading the keys and values that its first run stored
+            schedule = (ScheduleEntry(0), ScheduleEntry(1), ScheduleEntry(0), ScheduleEntry(1, cache_from=1))
+            return ModelSpec(d, r["vocab"], r["positions"],
+                             PartSpec("embedding", {"vocab_size": r["vocab"], "hidden_size": d}, "emb."),
+                             (toy, att), schedule, norm.with_prefix("final."),
+                             PartSpec("lm_head", {"vocab_size": r["vocab"], "hidden_size": d, "tied": True}, "head."))
+
+    lib.register_architecture("ToyForCausalLM", ToyConfig)
+    raw = {"architectures": ["ToyForCausalLM"], "width": 48, "head": 16, "ffn": 40, "state": 24, "decay": 0.9,
+           "eps": 1e-5, "vocab": 50, "positions": 256}
+    cfg = lib.config_from_dict(raw)
+    eng = Engine.from_random(cfg, seed=1, dtype="float32", max_tokens=512, stored_dtype="float32")
+    model = eng.model
+    assert sorted(type(g).__name__ for g in eng.cache.groups) == ["KVGroup", "StateGroup"]
+    assert [s is None for s in model.cache_specs()] == [False, False, False, True]
+
+    # plain float64 reference of this toy model, whole sequence
+    W = {}
+    for layer, p in zip(model.layers, ("l0.", "l1.")):
+        W[p + "n1"], W[p + "n2"] = layer.mixer_norm.weight.double().cpu(), layer.feed_forward_norm.weight.double().cpu()
+        gu = layer.feed_forward.w_gate_up.double().cpu()
+        W[p + "gate"], W[p + "up"], W[p + "down"] = gu[0::2], gu[1::2], layer.feed_forward.w_down.double().cpu()
+    toy, att = model.layers[0].mixer, model.layers[1].mixer
+    wq, wk, wv = att.wqkv.double().cpu().split([32, 16, 16])
+    wo = att.wo.double().cpu()
+
+    def ref_forward(toks):
+        n = len(toks)
+        x = model.embedding.weight.double().cpu()[toks]
+        posn = torch.arange(n)
+        kv = None
+        for entry in (0, 1, 2, 3):
+            p = "l0." if entry in (0, 2) else "l1."
+            h = P.rmsnorm(x, W[p + "n1"], 1e-5)
+            if p == "l0.":
+                u = h @ toy.w_in.double().cpu().t()
+                s, ys = torch.zeros(24, dtype=torch.float64), []
+                for t in range(n):
+                    s = 0.9 * s + u[t]
+                    ys.append(s)
+                x = x + torch.stack(ys) @ toy.w_out.double().cpu().t()
+            else:
+                q = P.rope((h @ wq.t()).view(n, 2, 16), posn, 100.0, 16)
+                if entry == 1:
+                    kv = (P.rope((h @ wk.t()).view(n, 1, 16), posn, 100.0, 16), (h @ wv.t()).view(n, 1, 16))
+                x = x + P.attention(q, kv[0], kv[1]).reshape(n, 32) @ wo.t()
+            x = x + P.swiglu(P.rmsnorm(x, W[p + "n2"], 1e-5), W[p + "gate"], W[p + "up"], W[p + "down"])
+        return P.rmsnorm(x, model.final_norm.weight.double().cpu(), 1e-5) @ model.embedding.weight.double().cpu().t()
+
+    g = torch.Generator().manual_seed(0)
+    seqs = [torch.randint(0, 50, (n,), generator=g).tolist() for n in (70, 9, 130)]
+    refs = [ref_forward(t) for t in seqs]
+    # whole, in one ragged batch
+    slots = [eng.alloc_slot() for _ in seqs]
+    out = eng.step(slots, seqs, [list(range(len(t))) for t in seqs]).double().cpu()
+    assert (out - torch.cat(refs)).abs().max().item() < 2e-5
+    for s in slots:
+        eng.free_slot(s)
+    # cut: a first part, then token by token; the state is carried from step to step and reset on reuse
+    slots = [eng.alloc_slot() for _ in seqs]
+    heads = [len(t) - 5 for t in seqs]
+    out = eng.step(slots, [t[:h] for t, h in zip(seqs, heads)]).double().cpu()
+    for i, (r, h) in enumerate(zip(refs, heads)):
+        assert (out[i] - r[h - 1]).abs().max().item() < 2e-5
+    for k in range(5):
+        out = eng.step(slots, [[t[h + k]] for t, h in zip(seqs, heads)]).double().cpu()
+        for i, (r, h) in enumerate(zip(refs, heads)):
+            assert (out[i] - r[h + k]).abs().max().item() < 2e-5
+    for s in slots:
+        eng.free_slot(s)
+    toks = eng.generate([seqs[1]], max_new_tokens=4, temperature=0.0, use_graph=False)[0]
+    assert toks[0] == int(refs[1][-1].argmax())
