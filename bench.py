@@ -108,11 +108,11 @@ def main() -> int:
               f"{b * args.steps / dt:.1f} tok/s", file=sys.stderr, flush=True)
 
     # prefill of one prompt
-    T = args.prefill_tokens
+    T = max(1, args.prefill_tokens)
     gen = torch.Generator().manual_seed(1)
     prompt = torch.randint(0, cfg.vocab_size, (T,), generator=gen).tolist()
     times = []
-    for i in range(4):
+    for i in range(4 if args.prefill_tokens > 0 else 2):
         slot = engine.alloc_slot()
         torch.cuda.synchronize()
         t = time.perf_counter()

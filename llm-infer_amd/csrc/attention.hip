@@ -61,19 +61,30 @@ struct WaveAttn {
         l = 0.f;
     }
 
-    // One page of 64 keys starting at key t0.  This lane's row sees keys lo..hi (hi < lo: none).
-    __device__ __forceinline__ void page(const T* kpage, const T* vpage, int t0, int lo, int hi, float scale2) {
+    // The work on one page of 64 keys is cut into phases so that a kernel can keep the loads of
+    // one phase in flight while the matrix cores work on another.
+    __device__ __forceinline__ void load_k(const T* kpage, v8 (&kf)[2 * KS]) const {
         const int lane = threadIdx.x & 63;
-        f32x16 s[2];
+#pragma unroll
+        for (int i = 0; i < 2 * KS; ++i) kf[i] = *(const v8*)(kpage + (i * 64 + lane) * 8);
+    }
+    __device__ __forceinline__ void load_v(const T* vpage, v8 (&vf)[DB * 4]) const {
+        const int lane = threadIdx.x & 63;
+#pragma unroll
+        for (int i = 0; i < DB * 4; ++i) vf[i] = *(const v8*)(vpage + (i * 64 + lane) * 8);
+    }
+
+    // Scores of the page's keys (starting at key t0) against this wave's rows, mask, running
+    // maximum and sum; leaves the probabilities in s.  This lane's row sees keys lo..hi.
+    __device__ __forceinline__ void scores(const v8 (&kf)[2 * KS], f32x16 (&s)[2], int t0, int lo, int hi,
+                                           float scale2) {
+        const int lane = threadIdx.x & 63;
 #pragma unroll
         for (int b = 0; b < 2; ++b) {
 #pragma unroll
             for (int r = 0; r < 16; ++r) s[b][r] = 0.f;
 #pragma unroll
-            for (int ks = 0; ks < KS; ++ks) {
-                const v8 kf = *(const v8*)(kpage + ((b * KS + ks) * 64 + lane) * 8);
-                s[b] = mfma32(kf, q[ks], s[b]);
-            }
+            for (int ks = 0; ks < KS; ++ks) s[b] = mfma32(kf[b * KS + ks], q[ks], s[b]);
         }
         float mx = -INFINITY;
 #pragma unroll
@@ -104,6 +115,28 @@ struct WaveAttn {
         for (int b = 0; b < DB; ++b)
 #pragma unroll
             for (int r = 0; r < 16; ++r) o[b][r] *= alpha;
+    }
+
+    // o += V^T P^T: the probabilities go from the score accumulators into operand B as they lie.
+    __device__ __forceinline__ void mix(const v8 (&vf)[DB * 4], const f32x16 (&s)[2]) {
+#pragma unroll
+        for (int tj = 0; tj < 4; ++tj) {
+            v8 pf;
+#pragma unroll
+            for (int i = 0; i < 8; ++i) pf[i] = from_f32<T>(s[tj >> 1][8 * (tj & 1) + i]);
+#pragma unroll
+            for (int b = 0; b < DB; ++b) o[b] = mfma32(vf[b * 4 + tj], pf, o[b]);
+        }
+    }
+
+    // One page, phases in order; the values are fetched where they are used, which keeps the
+    // register count low enough for several waves per SIMD.
+    __device__ __forceinline__ void page(const T* kpage, const T* vpage, int t0, int lo, int hi, float scale2) {
+        const int lane = threadIdx.x & 63;
+        v8 kf[2 * KS];
+        f32x16 s[2];
+        load_k(kpage, kf);
+        scores(kf, s, t0, lo, hi, scale2);
 #pragma unroll
         for (int tj = 0; tj < 4; ++tj) {
             v8 pf;
@@ -193,11 +226,18 @@ __global__ __launch_bounds__(64) void attn_decode_kernel(
     const int p0 = p_first + split * per, p1 = min(p_end, p0 + per);
     const int* table = c.page_table + (int64_t)seq_slot[b] * c.max_pages;
     const float scale2 = scale * LOG2E;
+    // keys of page p+1 are loaded while the values of page p are mixed, values of page p while
+    // its scores are computed
+    typename WaveAttn<T>::v8 kf[2 * KS], vf[DB * 4];
+    f32x16 s[2];
+    const T* kbase = (const T*)c.k + (int64_t)kvh * k_head_elems(HD);
+    const T* vbase = (const T*)c.v + (int64_t)kvh * v_head_elems(HD);
+    if (p0 < p1) a.load_k(kbase + (int64_t)table[p0] * c.page_stride, kf);
     for (int p = p0; p < p1; ++p) {
-        const int64_t page = table[p];
-        const T* kp = (const T*)c.k + page * c.page_stride + (int64_t)kvh * k_head_elems(HD);
-        const T* vp = (const T*)c.v + page * c.page_stride + (int64_t)kvh * v_head_elems(HD);
-        a.page(kp, vp, p * PAGE, lo, live ? pos : -1, scale2);
+        a.load_v(vbase + (int64_t)table[p] * c.page_stride, vf);
+        a.scores(kf, s, p * PAGE, lo, live ? pos : -1, scale2);
+        if (p + 1 < p1) a.load_k(kbase + (int64_t)table[p + 1] * c.page_stride, kf);
+        a.mix(vf, s);
     }
     const float total = a.total();
     if (!live) return;
@@ -235,16 +275,20 @@ __global__ __launch_bounds__(64) void attn_decode_kernel(
 template <class T>
 __global__ void attn_merge_kernel(const float* __restrict__ part_o, const float* __restrict__ part_ml,
                                   T* __restrict__ out, int S) {
+    __shared__ float wgt[64];                        // at most 64 splits
+    __shared__ float scratch[16];
     const int64_t row = blockIdx.x;                  // (sequence, head)
     const float* ml = part_ml + row * S * 2;
-    float M = -INFINITY;
-    for (int s = 0; s < S; ++s) M = fmaxf(M, ml[2 * s]);
-    float L = 0.f;
-    for (int s = 0; s < S; ++s) L += (ml[2 * s] == -INFINITY) ? 0.f : ml[2 * s + 1] * exp2f(ml[2 * s] - M);
-    for (int d = threadIdx.x; d < HD; d += blockDim.x) {
+    const int tid = threadIdx.x;
+    const float ms = tid < S ? ml[2 * tid] : -INFINITY;
+    const float M = block_max(ms, scratch);
+    const float w = (tid < S && ms != -INFINITY) ? exp2f(ms - M) : 0.f;
+    const float L = block_sum(tid < S ? ml[2 * tid + 1] * w : 0.f, scratch);
+    if (tid < 64) wgt[tid] = w;
+    __syncthreads();
+    for (int d = tid; d < HD; d += blockDim.x) {
         float acc = 0.f;
-        for (int s = 0; s < S; ++s)
-            if (ml[2 * s] != -INFINITY) acc += part_o[(row * S + s) * HD + d] * exp2f(ml[2 * s] - M);
+        for (int s = 0; s < S; ++s) acc += part_o[(row * S + s) * HD + d] * wgt[s];
         out[row * HD + d] = from_f32<T>(acc / L);
     }
 }
@@ -335,7 +379,7 @@ extern "C" int li_attn_decode(const void* q, void* out, int dt, const void* k, c
                               const int* page_table, int max_pages, const int* seq_slot, const int* seq_ctx,
                               int n_seqs, int H, int K, float scale, int window, int splits, float* part_o,
                               float* part_ml, hipStream_t stream) {
-    if (check_heads(H, K) || splits < 1 || (splits > 1 && (!part_o || !part_ml))) return LI_BAD_ARG;
+    if (check_heads(H, K) || splits < 1 || splits > 64 || (splits > 1 && (!part_o || !part_ml))) return LI_BAD_ARG;
     if (n_seqs <= 0) return LI_OK;
     CachePtrs c{k, v, page_stride, page_table, max_pages};
     const int G = H / K;
@@ -344,12 +388,12 @@ extern "C" int li_attn_decode(const void* q, void* out, int dt, const void* k, c
         attn_decode_kernel<f16><<<grid, block, 0, stream>>>((const f16*)q, (f16*)out, part_o, part_ml, c, seq_slot,
                                                             seq_ctx, H, K, scale, window);
         LI_CHECK_LAUNCH();
-        if (splits > 1) attn_merge_kernel<f16><<<n_seqs * H, 64, 0, stream>>>(part_o, part_ml, (f16*)out, splits);
+        if (splits > 1) attn_merge_kernel<f16><<<n_seqs * H, 128, 0, stream>>>(part_o, part_ml, (f16*)out, splits);
     } else if (dt == DT_BF16) {
         attn_decode_kernel<bf16><<<grid, block, 0, stream>>>((const bf16*)q, (bf16*)out, part_o, part_ml, c,
                                                              seq_slot, seq_ctx, H, K, scale, window);
         LI_CHECK_LAUNCH();
-        if (splits > 1) attn_merge_kernel<bf16><<<n_seqs * H, 64, 0, stream>>>(part_o, part_ml, (bf16*)out, splits);
+        if (splits > 1) attn_merge_kernel<bf16><<<n_seqs * H, 128, 0, stream>>>(part_o, part_ml, (bf16*)out, splits);
     } else return LI_BAD_ARG;
     LI_CHECK_LAUNCH();
     return LI_OK;

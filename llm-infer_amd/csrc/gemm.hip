@@ -294,6 +294,92 @@ __global__ __launch_bounds__(256) void gemv_kernel(const T* __restrict__ X, cons
     }
 }
 
+
+// ===========================================================================
+// gemv_mfma: up to 16 rows of X on the matrix cores (16x16x32), W streamed from
+// global memory straight into operand A.  A wave owns NT tiles of 16 rows of W
+// and one slice of K; the KW waves of a workgroup cover K and their partial
+// tiles are summed through LDS in wave order.  A lane (row r = lane%16, group
+// g = lane/16) loads 32 contiguous bytes of its row per 64 elements of K, so
+// two back-to-back loads of a wave fetch whole 128-byte lines; X uses the same
+// assignment of k to lanes, which the sum over k does not care about.
+// ===========================================================================
+__device__ __forceinline__ f32x4 mfma16(f16x8 a, f16x8 b, f32x4 c) {
+    return __builtin_amdgcn_mfma_f32_16x16x32_f16(a, b, c, 0, 0, 0);
+}
+__device__ __forceinline__ f32x4 mfma16(bf16x8 a, bf16x8 b, f32x4 c) {
+    return __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b, c, 0, 0, 0);
+}
+
+template <class T, int NT, int KW>
+__global__ __launch_bounds__(64 * KW) void gemv_mfma_kernel(const T* __restrict__ X, const T* __restrict__ W,
+                                                            int K, Epilogue e) {
+    typedef typename Vec<T>::v8 v8;
+    constexpr int U = 4;                                  // 64-element steps of K in flight
+    __shared__ float part[KW][NT][64][4];
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int r = lane & 15, g = lane >> 4;
+    const int n0 = blockIdx.x * (16 * NT);
+    const int steps = (K + 63) >> 6;
+    const int per = (steps + KW - 1) / KW;
+    const int s_begin = wave * per, s_end = min(steps, s_begin + per);
+    const T* wrow[NT];
+#pragma unroll
+    for (int t = 0; t < NT; ++t) wrow[t] = W + (int64_t)min(n0 + 16 * t + r, e.N - 1) * K + 16 * g;
+    const bool have_x = r < e.M;
+    const T* xrow = X + (int64_t)(have_x ? r : 0) * K + 16 * g;
+    f32x4 acc[NT];
+#pragma unroll
+    for (int t = 0; t < NT; ++t) acc[t] = f32x4{0.f, 0.f, 0.f, 0.f};
+
+    for (int s0 = s_begin; s0 < s_end; s0 += U) {
+        v8 a[U][NT][2], b[U][2];
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+            const int k = (s0 + u) * 64;                  // this lane reads k + 16 g .. + 15
+            const bool in0 = (s0 + u < s_end) && (k + 16 * g < K);
+            const bool in1 = (s0 + u < s_end) && (k + 16 * g + 8 < K);
+            const v8 z = {};
+#pragma unroll
+            for (int t = 0; t < NT; ++t) {
+                a[u][t][0] = in0 ? *(const v8*)(wrow[t] + k) : z;
+                a[u][t][1] = in1 ? *(const v8*)(wrow[t] + k + 8) : z;
+            }
+            b[u][0] = (in0 && have_x) ? *(const v8*)(xrow + k) : z;
+            b[u][1] = (in1 && have_x) ? *(const v8*)(xrow + k + 8) : z;
+        }
+#pragma unroll
+        for (int u = 0; u < U; ++u)
+#pragma unroll
+            for (int t = 0; t < NT; ++t) {
+                acc[t] = mfma16(a[u][t][0], b[u][0], acc[t]);
+                acc[t] = mfma16(a[u][t][1], b[u][1], acc[t]);
+            }
+    }
+    if (KW > 1) {
+#pragma unroll
+        for (int t = 0; t < NT; ++t)
+#pragma unroll
+            for (int q = 0; q < 4; ++q) part[wave][t][lane][q] = acc[t][q];
+        __syncthreads();
+        if (wave != 0) return;
+#pragma unroll
+        for (int t = 0; t < NT; ++t)
+#pragma unroll
+            for (int q = 0; q < 4; ++q) {
+                float v = part[0][t][lane][q];
+                for (int w = 1; w < KW; ++w) v += part[w][t][lane][q];
+                acc[t][q] = v;
+            }
+    }
+    // accumulator q of a 16x16 tile: row of W n = 4 * (lane / 16) + q, row of X m = lane % 16
+#pragma unroll
+    for (int t = 0; t < NT; ++t) {
+        float v[4] = {acc[t][0], acc[t][1], acc[t][2], acc[t][3]};
+        epilogue4(e, r, n0 + 16 * t + 4 * g, v);
+    }
+}
+
 // ===========================================================================
 // C interface
 // ===========================================================================
@@ -382,6 +468,33 @@ extern "C" int li_gemv(const void* X, const void* W, int dt, void* C, int out_dt
         else gemv_kernel<T, 8, R><<<grid, block, 0, stream>>>((const T*)X, (const T*)W, K, e);       \
     } while (0)
     if (dt == DT_F16) LAUNCH(f16); else LAUNCH(bf16);
+#undef LAUNCH
+    LI_CHECK_LAUNCH();
+    return LI_OK;
+}
+
+extern "C" int li_gemv_mfma(const void* X, const void* W, int dt, void* C, int out_dt, int mode,
+                            int M, int N, int K, hipStream_t stream) {
+    int rc = check_common(X, W, C, M, N, K, mode, out_dt);
+    if (rc) return rc;
+    if (dt != DT_F16 && dt != DT_BF16) return LI_BAD_ARG;
+    if (M > 16) return LI_BAD_ARG;
+    if (K % 8 != 0 || ((uintptr_t)X & 15) || ((uintptr_t)W & 15)) return LI_UNSUPPORTED;
+    if (M == 0) return LI_OK;
+    Epilogue e{C, mode, out_dt, M, N};
+    const int nt = N >= 16384 ? 2 : 1;
+    const int tiles = (N + 16 * nt - 1) / (16 * nt);
+    const int kw = (tiles < 1024 && K >= 2048) ? 8 : 4;
+#define LAUNCH(T, NT, KW) gemv_mfma_kernel<T, NT, KW><<<tiles, 64 * KW, 0, stream>>>((const T*)X, (const T*)W, K, e)
+#define PICK(T)                                          \
+    do {                                                 \
+        if (nt == 2 && kw == 4) LAUNCH(T, 2, 4);         \
+        else if (nt == 2) LAUNCH(T, 2, 8);               \
+        else if (kw == 4) LAUNCH(T, 1, 4);               \
+        else LAUNCH(T, 1, 8);                            \
+    } while (0)
+    if (dt == DT_F16) PICK(f16); else PICK(bf16);
+#undef PICK
 #undef LAUNCH
     LI_CHECK_LAUNCH();
     return LI_OK;

@@ -123,10 +123,14 @@ def linear(x: torch.Tensor, w: torch.Tensor, mode: int = EPI_STORE, out: torch.T
     lib = core()
     same16 = x.dtype == w.dtype and x.dtype in (torch.float16, torch.bfloat16)
     fast_ok = same16 and k % 8 == 0 and x.data_ptr() % 16 == 0 and w.data_ptr() % 16 == 0
-    kind = force or ("fma" if not fast_ok else ("gemv" if m <= 8 else "mfma"))
+    kind = force or ("fma" if not fast_ok else ("gemv_mfma" if m <= 16 else "mfma"))
     if kind == "fma":
         _check(lib.li_gemm_fma(_ptr(x), DT[x.dtype], _ptr(w), DT[w.dtype], _ptr(out), DT[out.dtype], mode,
                                m, n, k, _stream()), "gemm_fma")
+    elif kind == "gemv_mfma":
+        _need(fast_ok and m <= 16, "gemv_mfma: 16-bit operands, K a multiple of 8, at most 16 rows")
+        _check(lib.li_gemv_mfma(_ptr(x), _ptr(w), DT[x.dtype], _ptr(out), DT[out.dtype], mode, m, n, k, _stream()),
+               "gemv_mfma")
     elif kind == "gemv":
         _need(fast_ok and m <= 8, "gemv: 16-bit operands, K a multiple of 8, at most 8 rows")
         _check(lib.li_gemv(_ptr(x), _ptr(w), DT[x.dtype], _ptr(out), DT[out.dtype], mode, m, n, k, _stream()), "gemv")

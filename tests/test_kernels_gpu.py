@@ -63,7 +63,7 @@ def _linear_ref(x, w, mode, res=None):
 
 
 LIN_CASES = [  # M, N, K
-    (1, 64, 64), (3, 172, 96), (8, 100, 256), (5, 6, 8), (13, 344, 64), (33, 130, 136),
+    (1, 64, 64), (2, 16400, 4096), (16, 1000, 2056), (9, 40, 4104), (3, 172, 96), (8, 100, 256), (5, 6, 8), (13, 344, 64), (33, 130, 136),
     (64, 256, 512), (70, 200, 1024), (129, 384, 320), (200, 136, 72), (256, 512, 2048),
 ]
 
@@ -79,6 +79,8 @@ def test_linear_all_kernels_and_epilogues(ops, M, N, K, dt):
     if dt != torch.float32:
         if M <= 8:
             kinds.append("gemv")
+        if M <= 16:
+            kinds.append("gemv_mfma")
         kinds += ["mfma:0:1", "mfma:1:1", "mfma:2:1", "mfma:2:3", "mfma:0:2", None]
     for kind in kinds:
         for mode in (0, 1, 2):
