@@ -27,6 +27,11 @@ __device__ __forceinline__ void store_one(void* C, int dt, int64_t i, float v) {
     else ((bf16*)C)[i] = (bf16)v;
 }
 
+// Offset of W[n, k] in the tiled order of a weight matrix (see "Tiled weights" below).
+__host__ __device__ __forceinline__ int64_t tiled_offset(int n, int k, int K) {
+    return ((((int64_t)(n >> 4) * (K >> 5) + (k >> 5)) * 64) + (((k & 31) >> 3) << 4) + (n & 15)) * 8 + (k & 7);
+}
+
 // v[0..3] are the results for row m and columns n..n+3 (n a multiple of 4).
 __device__ __forceinline__ void epilogue4(const Epilogue& e, int m, int n, const float* v) {
     if (m >= e.M || n >= e.N) return;
@@ -116,7 +121,7 @@ __global__ __launch_bounds__(256) void gemm_fma_kernel(const TX* __restrict__ X,
 // X operand B, so that a lane ends with 4 consecutive columns n of one row m:
 // accumulator r of a 32x32 block is n = 8*(r/4) + 4*(lane/32) + r%4, m = lane%32.
 // ===========================================================================
-template <class T, int BN, int BM, int WN, int WM>
+template <class T, int BN, int BM, int WN, int WM, bool TILED>
 __global__ __launch_bounds__(256) void gemm_mfma_kernel(const T* __restrict__ X, const T* __restrict__ W,
                                                         int K, int k_per_split, float* __restrict__ ws,
                                                         Epilogue e) {
@@ -145,13 +150,18 @@ __global__ __launch_bounds__(256) void gemm_mfma_kernel(const T* __restrict__ X,
             for (int r = 0; r < 16; ++r) acc[a][b][r] = 0.f;
 
     v8 rw[W_CHUNKS], rx[X_CHUNKS];
+    const int n_padded = (e.N + 15) & ~15;
     auto load_tile = [&](int k0) {
 #pragma unroll
         for (int c = 0; c < W_CHUNKS; ++c) {
-            const int chunk = tid + c * 256, row = chunk >> 3, kc = (chunk & 7) * 8;
+            const int chunk = tid + c * 256;
+            // row-major: 8 threads a row; tiled: 64 threads a (16 rows x 32 k) block, as it lies in memory
+            const int row = TILED ? ((chunk >> 7) << 4) + (chunk & 15) : chunk >> 3;
+            const int kc = TILED ? (((chunk >> 6) & 1) << 5) + (((chunk >> 4) & 3) << 3) : (chunk & 7) * 8;
             const int n = n0 + row, k = k0 + kc;
             v8 z = {};
-            rw[c] = (n < e.N && k < k_end) ? *(const v8*)(W + (int64_t)n * K + k) : z;
+            if (TILED) rw[c] = (n < n_padded && k < k_end) ? *(const v8*)(W + tiled_offset(n, k, K)) : z;
+            else rw[c] = (n < e.N && k < k_end) ? *(const v8*)(W + (int64_t)n * K + k) : z;
         }
 #pragma unroll
         for (int c = 0; c < X_CHUNKS; ++c) {
@@ -164,7 +174,9 @@ __global__ __launch_bounds__(256) void gemm_mfma_kernel(const T* __restrict__ X,
     auto store_tile = [&]() {
 #pragma unroll
         for (int c = 0; c < W_CHUNKS; ++c) {
-            const int chunk = tid + c * 256, row = chunk >> 3, kc = (chunk & 7) * 8;
+            const int chunk = tid + c * 256;
+            const int row = TILED ? ((chunk >> 7) << 4) + (chunk & 15) : chunk >> 3;
+            const int kc = TILED ? (((chunk >> 6) & 1) << 5) + (((chunk >> 4) & 3) << 3) : (chunk & 7) * 8;
             *(v8*)(sW + row * LD + kc) = rw[c];
         }
 #pragma unroll
@@ -380,6 +392,89 @@ __global__ __launch_bounds__(64 * KW) void gemv_mfma_kernel(const T* __restrict_
     }
 }
 
+
+// ===========================================================================
+// Tiled weights.  A matrix W[N, K] (K a multiple of 32) may be kept in the order in
+// which the 16x16x32 matrix instruction takes operand A:
+//   [tile = n / 16][step = k / 32][lane = 16 * ((k % 32) / 8) + n % 16][k % 8]
+// (rows padded to a multiple of 16).  A wave then reads each operand as one
+// contiguous 1 KiB load.  gemv_tiled is gemv_mfma on that layout.
+// ===========================================================================
+template <class T>
+__global__ void tile_weight_kernel(const T* __restrict__ W, T* __restrict__ out, int N, int K, int64_t total) {
+    // one thread per 8 elements of the output
+    const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= total) return;
+    const int lane = (int)(i & 63);
+    const int64_t blk = i >> 6;
+    const int steps = K >> 5;
+    const int step = (int)(blk % steps);
+    const int tile = (int)(blk / steps);
+    const int n = tile * 16 + (lane & 15), k = step * 32 + (lane >> 4) * 8;
+    typedef typename Vec<T>::v8 v8;
+    v8 z = {};
+    *(v8*)(out + i * 8) = n < N ? *(const v8*)(W + (int64_t)n * K + k) : z;
+}
+
+template <class T, int NT, int KW>
+__global__ __launch_bounds__(64 * KW) void gemv_tiled_kernel(const T* __restrict__ X, const T* __restrict__ Wt,
+                                                             int K, Epilogue e) {
+    typedef typename Vec<T>::v8 v8;
+    constexpr int U = 8;                                  // 32-element steps of K in flight
+    __shared__ float part[KW][NT][64][4];
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int r = lane & 15, g = lane >> 4;
+    const int tile0 = blockIdx.x * NT;
+    const int n_tiles = (e.N + 15) >> 4;
+    const int steps = K >> 5;
+    const int per = (steps + KW - 1) / KW;
+    const int s_begin = wave * per, s_end = min(steps, s_begin + per);
+    const T* wt[NT];
+#pragma unroll
+    for (int t = 0; t < NT; ++t) wt[t] = Wt + ((int64_t)min(tile0 + t, n_tiles - 1) * steps * 64 + lane) * 8;
+    const bool have_x = r < e.M;
+    const T* xrow = X + (int64_t)(have_x ? r : 0) * K + 8 * g;
+    f32x4 acc[NT];
+#pragma unroll
+    for (int t = 0; t < NT; ++t) acc[t] = f32x4{0.f, 0.f, 0.f, 0.f};
+    for (int s0 = s_begin; s0 < s_end; s0 += U) {
+        v8 a[U][NT], b[U];
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+            const bool in = s0 + u < s_end;
+            const v8 z = {};
+#pragma unroll
+            for (int t = 0; t < NT; ++t) a[u][t] = in ? *(const v8*)(wt[t] + (int64_t)(s0 + u) * 512) : z;
+            b[u] = (in && have_x) ? *(const v8*)(xrow + (s0 + u) * 32) : z;
+        }
+#pragma unroll
+        for (int u = 0; u < U; ++u)
+#pragma unroll
+            for (int t = 0; t < NT; ++t) acc[t] = mfma16(a[u][t], b[u], acc[t]);
+    }
+    if (KW > 1) {
+#pragma unroll
+        for (int t = 0; t < NT; ++t)
+#pragma unroll
+            for (int q = 0; q < 4; ++q) part[wave][t][lane][q] = acc[t][q];
+        __syncthreads();
+        if (wave != 0) return;
+#pragma unroll
+        for (int t = 0; t < NT; ++t)
+#pragma unroll
+            for (int q = 0; q < 4; ++q) {
+                float v = part[0][t][lane][q];
+                for (int w = 1; w < KW; ++w) v += part[w][t][lane][q];
+                acc[t][q] = v;
+            }
+    }
+#pragma unroll
+    for (int t = 0; t < NT; ++t) {
+        float v[4] = {acc[t][0], acc[t][1], acc[t][2], acc[t][3]};
+        epilogue4(e, r, (tile0 + t) * 16 + 4 * g, v);
+    }
+}
+
 // ===========================================================================
 // C interface
 // ===========================================================================
@@ -418,12 +513,13 @@ extern "C" int li_gemm_fma(const void* X, int x_dt, const void* W, int w_dt, voi
 
 // tile: 0 = 128x128 (W rows x X rows), 1 = 128x64, 2 = 128x32.  splits > 1 needs ws of
 // splits*M*N floats.
-extern "C" int li_gemm_mfma(const void* X, const void* W, int dt, void* C, int out_dt, int mode,
+extern "C" int li_gemm_mfma(const void* X, const void* W, int tiled, int dt, void* C, int out_dt, int mode,
                             int M, int N, int K, int tile, int splits, float* ws, hipStream_t stream) {
     int rc = check_common(X, W, C, M, N, K, mode, out_dt);
     if (rc) return rc;
     if (dt != DT_F16 && dt != DT_BF16) return LI_BAD_ARG;
     if (K % 8 != 0 || ((uintptr_t)X & 15) || ((uintptr_t)W & 15)) return LI_UNSUPPORTED;
+    if (tiled && K % 32 != 0) return LI_UNSUPPORTED;
     if (splits < 1 || (splits > 1 && !ws)) return LI_BAD_ARG;
     if (M == 0) return LI_OK;
     Epilogue e{C, mode, out_dt, M, N};
@@ -431,15 +527,18 @@ extern "C" int li_gemm_mfma(const void* X, const void* W, int dt, void* C, int o
     splits = (K + k_per_split - 1) / k_per_split;
     const int bm = tile == 0 ? 128 : (tile == 1 ? 64 : 32);
     dim3 grid((N + 127) / 128, (M + bm - 1) / bm, splits), block(256);
-#define LAUNCH(T)                                                                                              \
-    do {                                                                                                       \
-        if (tile == 0) gemm_mfma_kernel<T, 128, 128, 2, 2><<<grid, block, 0, stream>>>((const T*)X, (const T*)W, K, k_per_split, ws, e); \
-        else if (tile == 1) gemm_mfma_kernel<T, 128, 64, 2, 2><<<grid, block, 0, stream>>>((const T*)X, (const T*)W, K, k_per_split, ws, e); \
-        else if (tile == 2) gemm_mfma_kernel<T, 128, 32, 4, 1><<<grid, block, 0, stream>>>((const T*)X, (const T*)W, K, k_per_split, ws, e); \
-        else return LI_BAD_ARG;                                                                                \
+#define GO(T, BN, BM, WN, WM, TL) \
+    gemm_mfma_kernel<T, BN, BM, WN, WM, TL><<<grid, block, 0, stream>>>((const T*)X, (const T*)W, K, k_per_split, ws, e)
+#define LAUNCH(T)                                                       \
+    do {                                                                \
+        if (tile == 0) { if (tiled) GO(T, 128, 128, 2, 2, true); else GO(T, 128, 128, 2, 2, false); } \
+        else if (tile == 1) { if (tiled) GO(T, 128, 64, 2, 2, true); else GO(T, 128, 64, 2, 2, false); } \
+        else if (tile == 2) { if (tiled) GO(T, 128, 32, 4, 1, true); else GO(T, 128, 32, 4, 1, false); } \
+        else return LI_BAD_ARG;                                         \
     } while (0)
     if (dt == DT_F16) LAUNCH(f16); else LAUNCH(bf16);
 #undef LAUNCH
+#undef GO
     LI_CHECK_LAUNCH();
     if (splits > 1) {
         const int64_t quads = (int64_t)M * ((N + 3) / 4);
@@ -492,6 +591,51 @@ extern "C" int li_gemv_mfma(const void* X, const void* W, int dt, void* C, int o
         else if (nt == 2) LAUNCH(T, 2, 8);               \
         else if (kw == 4) LAUNCH(T, 1, 4);               \
         else LAUNCH(T, 1, 8);                            \
+    } while (0)
+    if (dt == DT_F16) PICK(f16); else PICK(bf16);
+#undef PICK
+#undef LAUNCH
+    LI_CHECK_LAUNCH();
+    return LI_OK;
+}
+
+// W [N, K] row-major -> tiled order, ceil(N/16)*16 * K elements.
+extern "C" int li_tile_weight(const void* W, void* out, int dt, int N, int K, hipStream_t stream) {
+    if (!W || !out || N <= 0 || K <= 0 || K % 32 != 0) return LI_BAD_ARG;
+    const int64_t total = (int64_t)((N + 15) / 16) * (K / 32) * 64;
+    const unsigned grid = (unsigned)((total + 255) / 256);
+    if (dt == DT_F16) tile_weight_kernel<f16><<<grid, 256, 0, stream>>>((const f16*)W, (f16*)out, N, K, total);
+    else if (dt == DT_BF16) tile_weight_kernel<bf16><<<grid, 256, 0, stream>>>((const bf16*)W, (bf16*)out, N, K, total);
+    else return LI_BAD_ARG;
+    LI_CHECK_LAUNCH();
+    return LI_OK;
+}
+
+extern "C" int li_gemv_tiled(const void* X, const void* Wt, int dt, void* C, int out_dt, int mode,
+                             int M, int N, int K, int nt, int kw, hipStream_t stream) {
+    int rc = check_common(X, Wt, C, M, N, K, mode, out_dt);
+    if (rc) return rc;
+    if (dt != DT_F16 && dt != DT_BF16) return LI_BAD_ARG;
+    if (M > 16) return LI_BAD_ARG;
+    if (K % 32 != 0 || ((uintptr_t)X & 15) || ((uintptr_t)Wt & 15)) return LI_UNSUPPORTED;
+    if (M == 0) return LI_OK;
+    Epilogue e{C, mode, out_dt, M, N};
+    const int n_tiles = (N + 15) / 16;
+    if (nt <= 0) nt = N >= 16384 ? 2 : 1;
+    const int blocks = (n_tiles + nt - 1) / nt;
+    if (kw <= 0) kw = (blocks < 1024 && K >= 2048) ? 8 : 4;
+#define LAUNCH(T, NT, KW) gemv_tiled_kernel<T, NT, KW><<<blocks, 64 * KW, 0, stream>>>((const T*)X, (const T*)Wt, K, e)
+#define PICK(T)                                          \
+    do {                                                 \
+        if (nt == 2 && kw == 4) LAUNCH(T, 2, 4);         \
+        else if (nt == 2 && kw == 8) LAUNCH(T, 2, 8);    \
+        else if (nt == 2 && kw == 2) LAUNCH(T, 2, 2);    \
+        else if (nt == 1 && kw == 4) LAUNCH(T, 1, 4);    \
+        else if (nt == 1 && kw == 8) LAUNCH(T, 1, 8);    \
+        else if (nt == 1 && kw == 16) LAUNCH(T, 1, 16);  \
+        else if (nt == 4 && kw == 4) LAUNCH(T, 4, 4);    \
+        else if (nt == 4 && kw == 2) LAUNCH(T, 4, 2);    \
+        else return LI_BAD_ARG;                          \
     } while (0)
     if (dt == DT_F16) PICK(f16); else PICK(bf16);
 #undef PICK

@@ -90,6 +90,30 @@ def rmsnorm(x: torch.Tensor, w: torch.Tensor, eps: float, out_dtype, rows: torch
     return out
 
 
+class TiledWeight:
+    """A 16-bit matrix [n, k] kept in the order in which the matrix cores take it (csrc/gemm.hip,
+    "Tiled weights"); rows are padded to a multiple of 16.  ``prefix(rows)`` is the matrix of the
+    first rows (a multiple of 16), sharing the storage."""
+
+    def __init__(self, data: torch.Tensor, n: int, k: int):
+        self.data, self.n, self.k = data, n, k
+        self.dtype, self.device, self.shape = data.dtype, data.device, (n, k)
+
+    def prefix(self, rows: int) -> "TiledWeight":
+        _need(rows % 16 == 0 and 0 < rows <= self.n, "a tiled weight is cut at multiples of 16 rows")
+        return TiledWeight(self.data[: rows * self.k], rows, self.k)
+
+
+def can_tile(w: torch.Tensor) -> bool:
+    return w.dim() == 2 and w.dtype in (torch.float16, torch.bfloat16) and w.shape[1] % 32 == 0 and w.is_cuda
+
+
+def prepare_weight(w: torch.Tensor):
+    """The form in which a linear layer keeps its matrix: tiled where the kernels can use that
+    (16-bit, K a multiple of 32), else as it is."""
+    return tile_weight(w) if can_tile(w) else w
+
+
 _ws_cache: dict = {}
 
 
@@ -106,8 +130,10 @@ def linear(x: torch.Tensor, w: torch.Tensor, mode: int = EPI_STORE, out: torch.T
            out_dtype=None, force: str | None = None) -> torch.Tensor:
     """C = X W^T with the epilogue ``mode``: store, add into ``out`` (float32), or SwiGLU over
     interleaved gate/up rows of W (C has N/2 columns).  ``force`` picks a kernel for tests."""
-    _dev(x, w, out)
-    _need(x.dim() == 2 and w.dim() == 2 and x.shape[1] == w.shape[1], f"linear: x {tuple(x.shape)} w {tuple(w.shape)}")
+    tiled = isinstance(w, TiledWeight)
+    wd = w.data if tiled else w
+    _dev(x, wd, out)
+    _need(x.dim() == 2 and len(w.shape) == 2 and x.shape[1] == w.shape[1], f"linear: x {tuple(x.shape)} w {tuple(w.shape)}")
     m, k = x.shape
     n = w.shape[0]
     n_out = n // 2 if mode == EPI_SWIGLU else n
@@ -122,8 +148,14 @@ def linear(x: torch.Tensor, w: torch.Tensor, mode: int = EPI_STORE, out: torch.T
         return out
     lib = core()
     same16 = x.dtype == w.dtype and x.dtype in (torch.float16, torch.bfloat16)
-    fast_ok = same16 and k % 8 == 0 and x.data_ptr() % 16 == 0 and w.data_ptr() % 16 == 0
+    fast_ok = same16 and k % 8 == 0 and x.data_ptr() % 16 == 0 and wd.data_ptr() % 16 == 0
     kind = force or ("fma" if not fast_ok else ("gemv_mfma" if m <= 16 else "mfma"))
+    if tiled:
+        _need(fast_ok and kind != "fma" and kind != "gemv", "a tiled weight needs 16-bit activations of its dtype")
+        if kind == "gemv_mfma":
+            _check(lib.li_gemv_tiled(_ptr(x), _ptr(wd), DT[x.dtype], _ptr(out), DT[out.dtype], mode, m, n, k, 0, 0,
+                                     _stream()), "gemv_tiled")
+            return out
     if kind == "fma":
         _check(lib.li_gemm_fma(_ptr(x), DT[x.dtype], _ptr(w), DT[w.dtype], _ptr(out), DT[out.dtype], mode,
                                m, n, k, _stream()), "gemm_fma")
@@ -146,7 +178,7 @@ def linear(x: torch.Tensor, w: torch.Tensor, mode: int = EPI_STORE, out: torch.T
             _, t_, s_ = kind.split(":")
             tile, splits = int(t_), int(s_)
         ws = _workspace(splits * m * n, x.device) if splits > 1 else None
-        _check(lib.li_gemm_mfma(_ptr(x), _ptr(w), DT[x.dtype], _ptr(out), DT[out.dtype], mode, m, n, k,
+        _check(lib.li_gemm_mfma(_ptr(x), _ptr(wd), int(tiled), DT[x.dtype], _ptr(out), DT[out.dtype], mode, m, n, k,
                                 tile, splits, _ptr(ws), _stream()), "gemm_mfma")
     return out
 
@@ -300,3 +332,23 @@ def sample(logits, temperature: float, seq_slot=None, state=None, forced_r=None,
 def uniform01(key: int, counter: int) -> float:
     """The generator's value for (key, counter), computed on the host by the same function."""
     return float(core().li_uniform01(c_uint64(key & (2 ** 64 - 1)), c_uint64(counter & (2 ** 64 - 1))))
+
+
+def tile_weight(w: torch.Tensor) -> TiledWeight:
+    """A 16-bit matrix [N, K] (K a multiple of 32) in tiled order."""
+    _dev(w)
+    _need(can_tile(w), "tile_weight: 16-bit [N, K] on the GPU with K a multiple of 32")
+    n, k = w.shape
+    out = torch.empty(((n + 15) // 16 * 16 * k,), dtype=w.dtype, device=w.device)
+    _check(core().li_tile_weight(_ptr(w), _ptr(out), DT[w.dtype], n, k, _stream()), "tile_weight")
+    return TiledWeight(out, n, k)
+
+
+def gemv_tiled(x, w: TiledWeight, mode=EPI_STORE, out_dtype=None, nt=0, kw=0):
+    """gemv_tiled with a chosen shape of workgroup (for tuning and tests)."""
+    m, k = x.shape
+    n_out = w.n // 2 if mode == EPI_SWIGLU else w.n
+    out = torch.empty((m, n_out), dtype=out_dtype or x.dtype, device=x.device)
+    _check(core().li_gemv_tiled(_ptr(x), _ptr(w.data), DT[x.dtype], _ptr(out), DT[out.dtype], mode, m, w.n, k,
+                                nt, kw, _stream()), "gemv_tiled")
+    return out

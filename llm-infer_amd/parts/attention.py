@@ -37,8 +37,11 @@ class Attention(Part):
                 "v_proj.weight": ParamSpec((k * hd, d)), "o_proj.weight": ParamSpec((d, h * hd))}
 
     def bind(self, tensors):
-        self.wqkv = torch.cat([tensors["q_proj.weight"], tensors["k_proj.weight"], tensors["v_proj.weight"]], 0)
-        self.wo = tensors["o_proj.weight"]
+        wqkv = torch.cat([tensors["q_proj.weight"], tensors["k_proj.weight"], tensors["v_proj.weight"]], 0)
+        self.wqkv = ops.prepare_weight(wqkv)
+        self.wq = self.wqkv.prefix(self.n_heads * self.head_dim) if isinstance(self.wqkv, ops.TiledWeight) \
+            else self.wqkv[:self.n_heads * self.head_dim]
+        self.wo = ops.prepare_weight(tensors["o_proj.weight"])
 
     def cache_spec(self):
         return KVSpec(self.n_kv_heads, self.head_dim, self.window)
@@ -49,7 +52,7 @@ class Attention(Part):
             qkv = ops.linear(h, self.wqkv, out_dtype=torch.float32)
             q = self.position.rotate_store(qkv, ctx, cache_view, H, K, hd)
         else:                                   # reads another layer's keys and values
-            qkv = ops.linear(h, self.wqkv[:H * hd], out_dtype=torch.float32)
+            qkv = ops.linear(h, self.wq, out_dtype=torch.float32)
             q = self.position.rotate_store(qkv, ctx, None, H, 0, hd)
         kv = cache_view.as_tuple()
         if self.dtype == torch.float32:

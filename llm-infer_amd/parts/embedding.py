@@ -45,10 +45,11 @@ class LMHead(Part):
 
     def bind(self, tensors):
         if not self.tied:
-            self.weight = tensors["weight"]
+            self.weight = ops.prepare_weight(tensors["weight"])
 
     def tie(self, table):
-        self.weight = table
+        # the embedding gathers rows, the head streams the whole matrix: it keeps a tiled copy
+        self.weight = ops.prepare_weight(table)
 
     def forward(self, h):
         return ops.linear(h, self.weight, out_dtype=torch.float32)

@@ -34,8 +34,9 @@ class GatedMLP(Part):
         g, u = tensors["gate_proj.weight"], tensors["up_proj.weight"]
         if g.dtype != u.dtype:
             g, u = g.float(), u.float()
-        self.w_gate_up = torch.stack([g, u], dim=1).reshape(2 * self.intermediate_size, self.hidden_size).contiguous()
-        self.w_down = tensors["down_proj.weight"]
+        gu = torch.stack([g, u], dim=1).reshape(2 * self.intermediate_size, self.hidden_size).contiguous()
+        self.w_gate_up = ops.prepare_weight(gu)
+        self.w_down = ops.prepare_weight(tensors["down_proj.weight"])
 
     def forward(self, h, residual):
         t = ops.linear(h, self.w_gate_up, ops.EPI_SWIGLU, out_dtype=self.dtype)

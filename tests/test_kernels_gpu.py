@@ -105,6 +105,46 @@ def test_linear_all_kernels_and_epilogues(ops, M, N, K, dt):
                 assert torch.allclose(out16.double(), ref, rtol=_tol(dt), atol=_tol(dt))
 
 
+TILED_CASES = [(1, 64, 64), (3, 172, 96), (16, 40, 4096), (9, 16400, 256), (17, 100, 64), (64, 256, 512),
+               (70, 200, 1024), (129, 384, 320), (256, 520, 2048)]
+
+
+@pytest.mark.parametrize("M,N,K", TILED_CASES)
+@pytest.mark.parametrize("dt", F16S)
+def test_linear_tiled_weights(ops, M, N, K, dt):
+    """The same products with W kept in matrix-core order: every kernel that reads it, every epilogue."""
+    g = torch.Generator().manual_seed(M * 1000 + N + K)
+    x = torch.randn(M, K, generator=g).to(dt).to(DEV)
+    w = (torch.randn(N, K, generator=g) / math.sqrt(K)).to(dt).to(DEV)
+    res = torch.randn(M, N, generator=g).to(DEV)
+    wt = ops.tile_weight(w)
+    assert wt.shape == (N, K) and wt.data.numel() == (N + 15) // 16 * 16 * K
+    kinds = [None, "mfma:0:1", "mfma:1:2", "mfma:2:1"] + (["gemv_mfma"] if M <= 16 else [])
+    for kind in kinds:
+        for mode in (0, 1, 2):
+            if mode == 2 and N % 2:
+                continue
+            ref = _linear_ref(x, w, mode, res)
+            if mode == 1:
+                out = res.clone()
+                ops.linear(x, wt, mode, out=out, force=kind)
+            else:
+                out = ops.linear(x, wt, mode, out_dtype=torch.float32, force=kind)
+            err = (out.double() - ref).abs().max().item()
+            assert err < 2e-4 * (1 + ref.abs().max().item()), (kind, mode, err)
+    if M <= 16:
+        for nt, kw in ((1, 4), (1, 8), (1, 16), (2, 2), (2, 4), (2, 8), (4, 2), (4, 4)):
+            out = ops.gemv_tiled(x, wt, out_dtype=torch.float32, nt=nt, kw=kw)
+            assert (out.double() - _linear_ref(x, w, 0)).abs().max().item() < 2e-4 * 4
+    if N % 32 == 0:
+        head = ops.linear(x, wt.prefix(N // 2), out_dtype=torch.float32)
+        assert (head.double() - _linear_ref(x, w[:N // 2], 0)).abs().max().item() < 2e-4 * 4
+    with pytest.raises(ops.KernelError):
+        ops.linear(x, wt, force="fma")
+    with pytest.raises(ops.KernelError):
+        ops.tile_weight(w[:, :K - 8].contiguous())
+
+
 def test_linear_rows_do_not_depend_on_the_batch_in_float32(ops):
     g = torch.Generator().manual_seed(1)
     x = torch.randn(70, 136, generator=g).to(DEV)
