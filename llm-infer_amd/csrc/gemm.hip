@@ -12,13 +12,29 @@
 //              loads, X sits in LDS, v_dot2 accumulates in float32.
 #include "common.h"
 
-enum { EPI_STORE = 0, EPI_ADD = 1, EPI_SWIGLU = 2 };
+enum { EPI_STORE = 0, EPI_ADD = 1, EPI_SWIGLU = 2, EPI_ROPE = 3 };
+
+// What the EPI_ROPE epilogue needs: the columns of the product are the q heads, then the k heads,
+// then the v heads of a token; q and k are rotated by the token's position (adjacent pairs), q goes
+// to q_out [M, H, hd], k and v into the token's cache page.
+struct RopeStore {
+    const float* inv_freq;      // [rotary_dim / 2]
+    const int* pos;             // [M] position of each row
+    const int* tok_slot;        // [M] cache slot of each row
+    const int* page_table;      // [slots, max_pages]
+    void* q_out;
+    void* k_pages;
+    void* v_pages;
+    int64_t page_stride;
+    int rotary_dim, H, K, hd, max_pages, dt;   // dt: DT_* of q_out and the cache
+};
 
 struct Epilogue {
-    void* C;        // output
+    void* C;        // output (unused by EPI_ROPE)
     int mode;       // EPI_*
     int out_dt;     // DT_* of C (EPI_ADD: always float32)
     int M, N;
+    RopeStore rs;
 };
 
 __device__ __forceinline__ void store_one(void* C, int dt, int64_t i, float v) {
@@ -35,6 +51,42 @@ __host__ __device__ __forceinline__ int64_t tiled_offset(int n, int k, int K) {
 // v[0..3] are the results for row m and columns n..n+3 (n a multiple of 4).
 __device__ __forceinline__ void epilogue4(const Epilogue& e, int m, int n, const float* v) {
     if (m >= e.M || n >= e.N) return;
+    if (e.mode == EPI_ROPE) {
+        // include/kernels_cpu.hpp:82-100 and src/model/block.cpp:141-148, on the accumulators
+        const RopeStore& r = e.rs;
+        const int head = n / r.hd, d = n - head * r.hd;       // the 4 columns lie in one head (hd % 16 == 0)
+        const int p = r.pos[m];
+        float o[4] = {v[0], v[1], v[2], v[3]};
+        if (head < r.H + r.K) {
+#pragma unroll
+            for (int j = 0; j < 4; j += 2) {
+                if (d + j < r.rotary_dim) {
+                    float sn, cs;
+                    sincosf((float)p * r.inv_freq[(d + j) >> 1], &sn, &cs);
+                    o[j] = v[j] * cs - v[j + 1] * sn;
+                    o[j + 1] = v[j] * sn + v[j + 1] * cs;
+                }
+            }
+        }
+        if (head < r.H) {
+            const int64_t at = ((int64_t)m * r.H + head) * r.hd + d;
+#pragma unroll
+            for (int j = 0; j < 4; ++j) store_one(r.q_out, r.dt, at + j, o[j]);
+        } else {
+            const int64_t page = r.page_table[(int64_t)r.tok_slot[m] * r.max_pages + p / PAGE];
+            const int tp = p % PAGE;
+            if (head < r.H + r.K) {
+                const int64_t at = page * r.page_stride + (int64_t)(head - r.H) * k_head_elems(r.hd);
+#pragma unroll
+                for (int j = 0; j < 4; ++j) store_one(r.k_pages, r.dt, at + k_offset(tp, d + j, r.hd), o[j]);
+            } else {
+                const int64_t at = page * r.page_stride + (int64_t)(head - r.H - r.K) * v_head_elems(r.hd);
+#pragma unroll
+                for (int j = 0; j < 4; ++j) store_one(r.v_pages, r.dt, at + v_offset(tp, d + j, r.hd), o[j]);
+            }
+        }
+        return;
+    }
     if (e.mode == EPI_SWIGLU) {
         // columns 2j (gate) and 2j+1 (up) give h[m, j] = silu(gate) * up   (src/model/block.cpp:209-213)
         const int64_t row = (int64_t)m * (e.N >> 1);
@@ -478,9 +530,23 @@ __global__ __launch_bounds__(64 * KW) void gemv_tiled_kernel(const T* __restrict
 // ===========================================================================
 // C interface
 // ===========================================================================
+static int make_epilogue(Epilogue& e, void* C, int mode, int out_dt, int M, int N, const RopeStore* rs) {
+    e.C = C; e.mode = mode; e.out_dt = out_dt; e.M = M; e.N = N;
+    e.rs = RopeStore{};
+    if (mode != EPI_ROPE) return LI_OK;
+    if (!rs || !rs->pos || !rs->q_out || rs->hd <= 0 || rs->hd % 16 != 0 || rs->H <= 0 || rs->K < 0) return LI_BAD_ARG;
+    if (N != (rs->H + 2 * rs->K) * rs->hd || rs->rotary_dim < 0 || rs->rotary_dim > rs->hd || (rs->rotary_dim & 1))
+        return LI_BAD_ARG;
+    if (rs->rotary_dim > 0 && !rs->inv_freq) return LI_BAD_ARG;
+    if (rs->K > 0 && (!rs->tok_slot || !rs->page_table || !rs->k_pages || !rs->v_pages)) return LI_BAD_ARG;
+    if (rs->dt < DT_F32 || rs->dt > DT_BF16) return LI_BAD_ARG;
+    e.rs = *rs;
+    return LI_OK;
+}
+
 static int check_common(const void* X, const void* W, const void* C, int M, int N, int K, int mode, int out_dt) {
-    if (!X || !W || !C || M < 0 || N <= 0 || K <= 0) return LI_BAD_ARG;
-    if (mode < EPI_STORE || mode > EPI_SWIGLU) return LI_BAD_ARG;
+    if (!X || !W || (!C && mode != EPI_ROPE) || M < 0 || N <= 0 || K <= 0) return LI_BAD_ARG;
+    if (mode < EPI_STORE || mode > EPI_ROPE) return LI_BAD_ARG;
     if (out_dt < DT_F32 || out_dt > DT_BF16) return LI_BAD_ARG;
     if (mode == EPI_ADD && out_dt != DT_F32) return LI_BAD_ARG;
     if (mode == EPI_SWIGLU && (N & 1)) return LI_BAD_ARG;
@@ -488,11 +554,13 @@ static int check_common(const void* X, const void* W, const void* C, int M, int 
 }
 
 extern "C" int li_gemm_fma(const void* X, int x_dt, const void* W, int w_dt, void* C, int out_dt, int mode,
-                           int M, int N, int K, hipStream_t stream) {
+                           int M, int N, int K, const RopeStore* rs, hipStream_t stream) {
     int rc = check_common(X, W, C, M, N, K, mode, out_dt);
     if (rc) return rc;
     if (M == 0) return LI_OK;
-    Epilogue e{C, mode, out_dt, M, N};
+    Epilogue e;
+    rc = make_epilogue(e, C, mode, out_dt, M, N, rs);
+    if (rc) return rc;
     dim3 grid((N + 63) / 64, (M + 63) / 64), block(256);
 #define CASE(xd, TX, wd, TW)                                                                       \
     if (x_dt == xd && w_dt == wd) {                                                                \
@@ -514,7 +582,7 @@ extern "C" int li_gemm_fma(const void* X, int x_dt, const void* W, int w_dt, voi
 // tile: 0 = 128x128 (W rows x X rows), 1 = 128x64, 2 = 128x32.  splits > 1 needs ws of
 // splits*M*N floats.
 extern "C" int li_gemm_mfma(const void* X, const void* W, int tiled, int dt, void* C, int out_dt, int mode,
-                            int M, int N, int K, int tile, int splits, float* ws, hipStream_t stream) {
+                            int M, int N, int K, int tile, int splits, float* ws, const RopeStore* rs, hipStream_t stream) {
     int rc = check_common(X, W, C, M, N, K, mode, out_dt);
     if (rc) return rc;
     if (dt != DT_F16 && dt != DT_BF16) return LI_BAD_ARG;
@@ -522,7 +590,9 @@ extern "C" int li_gemm_mfma(const void* X, const void* W, int tiled, int dt, voi
     if (tiled && K % 32 != 0) return LI_UNSUPPORTED;
     if (splits < 1 || (splits > 1 && !ws)) return LI_BAD_ARG;
     if (M == 0) return LI_OK;
-    Epilogue e{C, mode, out_dt, M, N};
+    Epilogue e;
+    rc = make_epilogue(e, C, mode, out_dt, M, N, rs);
+    if (rc) return rc;
     int k_per_split = ((K + splits - 1) / splits + 63) / 64 * 64;
     splits = (K + k_per_split - 1) / k_per_split;
     const int bm = tile == 0 ? 128 : (tile == 1 ? 64 : 32);
@@ -549,14 +619,16 @@ extern "C" int li_gemm_mfma(const void* X, const void* W, int tiled, int dt, voi
 }
 
 extern "C" int li_gemv(const void* X, const void* W, int dt, void* C, int out_dt, int mode,
-                       int M, int N, int K, hipStream_t stream) {
+                       int M, int N, int K, const RopeStore* rs, hipStream_t stream) {
     int rc = check_common(X, W, C, M, N, K, mode, out_dt);
     if (rc) return rc;
     if (dt != DT_F16 && dt != DT_BF16) return LI_BAD_ARG;
     if (M > 8) return LI_BAD_ARG;
     if (K % 8 != 0 || ((uintptr_t)X & 15) || ((uintptr_t)W & 15)) return LI_UNSUPPORTED;
     if (M == 0) return LI_OK;
-    Epilogue e{C, mode, out_dt, M, N};
+    Epilogue e;
+    rc = make_epilogue(e, C, mode, out_dt, M, N, rs);
+    if (rc) return rc;
     constexpr int R = 4;
     dim3 grid((N + 4 * R - 1) / (4 * R)), block(256);
 #define LAUNCH(T)                                                                                    \
@@ -573,14 +645,16 @@ extern "C" int li_gemv(const void* X, const void* W, int dt, void* C, int out_dt
 }
 
 extern "C" int li_gemv_mfma(const void* X, const void* W, int dt, void* C, int out_dt, int mode,
-                            int M, int N, int K, hipStream_t stream) {
+                            int M, int N, int K, const RopeStore* rs, hipStream_t stream) {
     int rc = check_common(X, W, C, M, N, K, mode, out_dt);
     if (rc) return rc;
     if (dt != DT_F16 && dt != DT_BF16) return LI_BAD_ARG;
     if (M > 16) return LI_BAD_ARG;
     if (K % 8 != 0 || ((uintptr_t)X & 15) || ((uintptr_t)W & 15)) return LI_UNSUPPORTED;
     if (M == 0) return LI_OK;
-    Epilogue e{C, mode, out_dt, M, N};
+    Epilogue e;
+    rc = make_epilogue(e, C, mode, out_dt, M, N, rs);
+    if (rc) return rc;
     const int nt = N >= 16384 ? 2 : 1;
     const int tiles = (N + 16 * nt - 1) / (16 * nt);
     const int kw = (tiles < 1024 && K >= 2048) ? 8 : 4;
@@ -612,18 +686,20 @@ extern "C" int li_tile_weight(const void* W, void* out, int dt, int N, int K, hi
 }
 
 extern "C" int li_gemv_tiled(const void* X, const void* Wt, int dt, void* C, int out_dt, int mode,
-                             int M, int N, int K, int nt, int kw, hipStream_t stream) {
+                             int M, int N, int K, int nt, int kw, const RopeStore* rs, hipStream_t stream) {
     int rc = check_common(X, Wt, C, M, N, K, mode, out_dt);
     if (rc) return rc;
     if (dt != DT_F16 && dt != DT_BF16) return LI_BAD_ARG;
     if (M > 16) return LI_BAD_ARG;
     if (K % 32 != 0 || ((uintptr_t)X & 15) || ((uintptr_t)Wt & 15)) return LI_UNSUPPORTED;
     if (M == 0) return LI_OK;
-    Epilogue e{C, mode, out_dt, M, N};
+    Epilogue e;
+    rc = make_epilogue(e, C, mode, out_dt, M, N, rs);
+    if (rc) return rc;
     const int n_tiles = (N + 15) / 16;
-    if (nt <= 0) nt = N >= 16384 ? 2 : 1;
+    if (nt <= 0) nt = 1;
     const int blocks = (n_tiles + nt - 1) / nt;
-    if (kw <= 0) kw = (blocks < 1024 && K >= 2048) ? 8 : 4;
+    if (kw <= 0) kw = (K >= 8192 || blocks < 320 || blocks > 4096) ? 8 : 4;   // measured on MI355X
 #define LAUNCH(T, NT, KW) gemv_tiled_kernel<T, NT, KW><<<blocks, 64 * KW, 0, stream>>>((const T*)X, (const T*)Wt, K, e)
 #define PICK(T)                                          \
     do {                                                 \

@@ -13,7 +13,7 @@ from . import build
 
 PAGE = 64
 DT = {torch.float32: 0, torch.float16: 1, torch.bfloat16: 2}
-EPI_STORE, EPI_ADD, EPI_SWIGLU = 0, 1, 2
+EPI_STORE, EPI_ADD, EPI_SWIGLU, EPI_ROPE = 0, 1, 2, 3
 _STATUS = {1: "bad argument", 2: "unsupported size or alignment", 3: "HIP launch error"}
 
 
@@ -90,6 +90,13 @@ def rmsnorm(x: torch.Tensor, w: torch.Tensor, eps: float, out_dtype, rows: torch
     return out
 
 
+class _RopeStore(ctypes.Structure):
+    _fields_ = [("inv_freq", c_void_p), ("pos", c_void_p), ("tok_slot", c_void_p), ("page_table", c_void_p),
+                ("q_out", c_void_p), ("k_pages", c_void_p), ("v_pages", c_void_p), ("page_stride", c_int64),
+                ("rotary_dim", c_int), ("H", c_int), ("K", c_int), ("hd", c_int), ("max_pages", c_int),
+                ("dt", c_int)]
+
+
 class TiledWeight:
     """A 16-bit matrix [n, k] kept in the order in which the matrix cores take it (csrc/gemm.hip,
     "Tiled weights"); rows are padded to a multiple of 16.  ``prefix(rows)`` is the matrix of the
@@ -126,8 +133,8 @@ def _workspace(n_floats: int, device) -> torch.Tensor:
     return ws
 
 
-def linear(x: torch.Tensor, w: torch.Tensor, mode: int = EPI_STORE, out: torch.Tensor | None = None,
-           out_dtype=None, force: str | None = None) -> torch.Tensor:
+def linear(x: torch.Tensor, w, mode: int = EPI_STORE, out: torch.Tensor | None = None,
+           out_dtype=None, force: str | None = None, _rope=None) -> torch.Tensor:
     """C = X W^T with the epilogue ``mode``: store, add into ``out`` (float32), or SwiGLU over
     interleaved gate/up rows of W (C has N/2 columns).  ``force`` picks a kernel for tests."""
     tiled = isinstance(w, TiledWeight)
@@ -139,9 +146,14 @@ def linear(x: torch.Tensor, w: torch.Tensor, mode: int = EPI_STORE, out: torch.T
     n_out = n // 2 if mode == EPI_SWIGLU else n
     if mode == EPI_ADD:
         _need(out is not None and out.dtype == torch.float32, "add epilogue needs a float32 output")
-    if out is None:
+    rs = ctypes.byref(_rope) if _rope is not None else None
+    if mode == EPI_ROPE:
+        _need(_rope is not None, "the rotation epilogue needs its arguments (use linear_rope_store)")
+    elif out is None:
         out = torch.empty((m, n_out), dtype=out_dtype or x.dtype, device=x.device)
-    _need(out.shape == (m, n_out), f"linear: out {tuple(out.shape)}, expected {(m, n_out)}")
+    if mode != EPI_ROPE:
+        _need(out.shape == (m, n_out), f"linear: out {tuple(out.shape)}, expected {(m, n_out)}")
+    out_dt = DT[out.dtype] if out is not None else 0
     if mode == EPI_SWIGLU:
         _need(n % 2 == 0, "SwiGLU epilogue needs an even number of rows of W")
     if m == 0:
@@ -153,19 +165,19 @@ def linear(x: torch.Tensor, w: torch.Tensor, mode: int = EPI_STORE, out: torch.T
     if tiled:
         _need(fast_ok and kind != "fma" and kind != "gemv", "a tiled weight needs 16-bit activations of its dtype")
         if kind == "gemv_mfma":
-            _check(lib.li_gemv_tiled(_ptr(x), _ptr(wd), DT[x.dtype], _ptr(out), DT[out.dtype], mode, m, n, k, 0, 0,
-                                     _stream()), "gemv_tiled")
+            _check(lib.li_gemv_tiled(_ptr(x), _ptr(wd), DT[x.dtype], _ptr(out), out_dt, mode, m, n, k, 0, 0,
+                                     rs, _stream()), "gemv_tiled")
             return out
     if kind == "fma":
-        _check(lib.li_gemm_fma(_ptr(x), DT[x.dtype], _ptr(w), DT[w.dtype], _ptr(out), DT[out.dtype], mode,
-                               m, n, k, _stream()), "gemm_fma")
+        _check(lib.li_gemm_fma(_ptr(x), DT[x.dtype], _ptr(w), DT[w.dtype], _ptr(out), out_dt, mode,
+                               m, n, k, rs, _stream()), "gemm_fma")
     elif kind == "gemv_mfma":
         _need(fast_ok and m <= 16, "gemv_mfma: 16-bit operands, K a multiple of 8, at most 16 rows")
-        _check(lib.li_gemv_mfma(_ptr(x), _ptr(w), DT[x.dtype], _ptr(out), DT[out.dtype], mode, m, n, k, _stream()),
+        _check(lib.li_gemv_mfma(_ptr(x), _ptr(w), DT[x.dtype], _ptr(out), out_dt, mode, m, n, k, rs, _stream()),
                "gemv_mfma")
     elif kind == "gemv":
         _need(fast_ok and m <= 8, "gemv: 16-bit operands, K a multiple of 8, at most 8 rows")
-        _check(lib.li_gemv(_ptr(x), _ptr(w), DT[x.dtype], _ptr(out), DT[out.dtype], mode, m, n, k, _stream()), "gemv")
+        _check(lib.li_gemv(_ptr(x), _ptr(w), DT[x.dtype], _ptr(out), out_dt, mode, m, n, k, rs, _stream()), "gemv")
     else:
         _need(fast_ok, "gemm_mfma: 16-bit operands and K a multiple of 8")
         tile = 0 if m > 64 else (1 if m > 32 else 2)
@@ -178,8 +190,8 @@ def linear(x: torch.Tensor, w: torch.Tensor, mode: int = EPI_STORE, out: torch.T
             _, t_, s_ = kind.split(":")
             tile, splits = int(t_), int(s_)
         ws = _workspace(splits * m * n, x.device) if splits > 1 else None
-        _check(lib.li_gemm_mfma(_ptr(x), _ptr(wd), int(tiled), DT[x.dtype], _ptr(out), DT[out.dtype], mode, m, n, k,
-                                tile, splits, _ptr(ws), _stream()), "gemm_mfma")
+        _check(lib.li_gemm_mfma(_ptr(x), _ptr(wd), int(tiled), DT[x.dtype], _ptr(out), out_dt, mode, m, n, k,
+                                tile, splits, _ptr(ws), rs, _stream()), "gemm_mfma")
     return out
 
 
@@ -214,6 +226,35 @@ def rope_store(qkv, inv_freq, rotary_dim, half_pairing, pos, tok_slot, page_tabl
         _ptr(page_table), page_table.shape[1] if page_table is not None else 0, c_int64(page_stride or 0),
         _ptr(q), _ptr(k_pages),
         _ptr(v_pages), DT[out_dtype], t, n_heads, n_kv_heads, head_dim, _stream()), "rope_store")
+    return q
+
+
+def linear_rope_store(x, w, inv_freq, rotary_dim, pos, tok_slot, page_table, page_stride, k_pages, v_pages,
+                      n_heads, n_kv_heads, head_dim, out_dtype, force=None) -> torch.Tensor:
+    """q, k, v = x W^T with the rotation (adjacent pairs) and the cache write done in the product's
+    epilogue, on the float32 accumulators: the same result as linear (float32) followed by
+    rope_store, without the round trip.  Returns q [T, H, hd]."""
+    _dev(inv_freq, pos, tok_slot, page_table, k_pages, v_pages)
+    t = x.shape[0]
+    _need(w.shape[0] == (n_heads + 2 * n_kv_heads) * head_dim, "linear_rope_store: rows of W are not (H + 2K) hd")
+    _need(head_dim % 16 == 0, "head size must be a multiple of 16")
+    _need(pos.dtype == torch.int32 and pos.numel() >= t, "pos: int32 [T]")
+    if rotary_dim > 0:
+        _need(inv_freq is not None and inv_freq.dtype == torch.float32 and inv_freq.numel() >= rotary_dim // 2,
+              "inv_freq: float32 [rotary_dim / 2]")
+    if n_kv_heads > 0:
+        _need(tok_slot.dtype == torch.int32 and tok_slot.numel() >= t, "tok_slot: int32 [T]")
+        _need(page_table.dtype == torch.int32 and page_table.dim() == 2, "page_table: int32 [slots, pages]")
+        _need(k_pages.dtype == out_dtype and v_pages.dtype == out_dtype, "cache dtype differs from q dtype")
+    q = torch.empty((t, n_heads, head_dim), dtype=out_dtype, device=x.device)
+    rs = _RopeStore(inv_freq.data_ptr() if inv_freq is not None else None, pos.data_ptr(),
+                    tok_slot.data_ptr() if tok_slot is not None else None,
+                    page_table.data_ptr() if page_table is not None else None, q.data_ptr(),
+                    k_pages.data_ptr() if k_pages is not None else None,
+                    v_pages.data_ptr() if v_pages is not None else None, int(page_stride or 0), rotary_dim,
+                    n_heads, n_kv_heads, head_dim, page_table.shape[1] if page_table is not None else 0,
+                    DT[out_dtype])
+    linear(x, w, EPI_ROPE, force=force, _rope=rs)
     return q
 
 
@@ -350,5 +391,5 @@ def gemv_tiled(x, w: TiledWeight, mode=EPI_STORE, out_dtype=None, nt=0, kw=0):
     n_out = w.n // 2 if mode == EPI_SWIGLU else w.n
     out = torch.empty((m, n_out), dtype=out_dtype or x.dtype, device=x.device)
     _check(core().li_gemv_tiled(_ptr(x), _ptr(w.data), DT[x.dtype], _ptr(out), DT[out.dtype], mode, m, w.n, k,
-                                nt, kw, _stream()), "gemv_tiled")
+                                nt, kw, None, _stream()), "gemv_tiled")
     return out

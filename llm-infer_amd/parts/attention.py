@@ -49,11 +49,9 @@ class Attention(Part):
     def forward(self, h, ctx, cache_view, residual, owns_cache=True):
         H, K, hd = self.n_heads, self.n_kv_heads, self.head_dim
         if owns_cache:
-            qkv = ops.linear(h, self.wqkv, out_dtype=torch.float32)
-            q = self.position.rotate_store(qkv, ctx, cache_view, H, K, hd)
+            q = self.position.project_rotate_store(h, self.wqkv, ctx, cache_view, H, K, hd)
         else:                                   # reads another layer's keys and values
-            qkv = ops.linear(h, self.wq, out_dtype=torch.float32)
-            q = self.position.rotate_store(qkv, ctx, None, H, 0, hd)
+            q = self.position.project_rotate_store(h, self.wq, ctx, None, H, 0, hd)
         kv = cache_view.as_tuple()
         if self.dtype == torch.float32:
             a = ops.attention_f32(q, kv, ctx.pos, ctx.tok_slot, H, K, hd, self.scale, self.window)

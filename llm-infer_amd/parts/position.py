@@ -33,6 +33,23 @@ class RotaryPosition:
         return ops.rope_store(qkv, self.inv_freq, self.rotary_dim, self.pairing == "half", ctx.pos, ctx.tok_slot,
                               table, stride, k, v, n_heads, n_kv_heads, head_dim, self.dtype)
 
+    def project_rotate_store(self, h, w, ctx, kv_view, n_heads, n_kv_heads, head_dim):
+        """q, k, v = h W^T, rotated and stored; with adjacent pairing and 16-bit storage the rotation
+        and the cache write happen in the product's epilogue."""
+        return _project(self, h, w, ctx, kv_view, n_heads, n_kv_heads, head_dim, self.inv_freq, self.rotary_dim,
+                        self.pairing == "adjacent")
+
+
+def _project(part, h, w, ctx, kv_view, n_heads, n_kv_heads, head_dim, inv_freq, rotary_dim, fusable):
+    if fusable and part.dtype != torch.float32 and h.dtype == part.dtype:
+        k = v = table = stride = None
+        if n_kv_heads > 0:
+            k, v, table, stride = kv_view.k, kv_view.v, kv_view.page_table, kv_view.page_stride
+        return ops.linear_rope_store(h, w, inv_freq, rotary_dim, ctx.pos, ctx.tok_slot, table, stride, k, v,
+                                     n_heads, n_kv_heads, head_dim, part.dtype)
+    qkv = ops.linear(h, w, out_dtype=torch.float32)
+    return part.rotate_store(qkv, ctx, kv_view, n_heads, n_kv_heads, head_dim)
+
 
 @register_position("none")
 class NoPosition:
@@ -47,3 +64,6 @@ class NoPosition:
             k, v, table, stride = kv_view.k, kv_view.v, kv_view.page_table, kv_view.page_stride
         return ops.rope_store(qkv, None, 0, False, ctx.pos, ctx.tok_slot, table, stride, k, v, n_heads, n_kv_heads,
                               head_dim, self.dtype)
+
+    def project_rotate_store(self, h, w, ctx, kv_view, n_heads, n_kv_heads, head_dim):
+        return _project(self, h, w, ctx, kv_view, n_heads, n_kv_heads, head_dim, None, 0, True)

@@ -339,6 +339,49 @@ def test_rope_store_rotation_and_cache_layout(ops):
     assert torch.allclose(q2.double().cpu(), ref_half, atol=2e-5)
 
 
+@pytest.mark.parametrize("dt", F16S)
+@pytest.mark.parametrize("T,H,K,hd,rot,d", [(1, 4, 2, 16, 16, 64), (9, 3, 1, 32, 16, 96), (70, 5, 5, 48, 24, 160),
+                                           (200, 8, 2, 64, 64, 256), (3, 2, 0, 32, 32, 64)])
+def test_rotation_fused_into_the_projection(ops, dt, T, H, K, hd, rot, d):
+    """The product whose epilogue rotates and stores equals the product followed by rope_store:
+    q bit for bit (same float32 accumulators, same rounding), and the same cache pages."""
+    from llm_infer_amd.cache import Cache, KVSpec
+    g = torch.Generator().manual_seed(T + hd)
+    x = torch.randn(T, d, generator=g).to(dt).to(DEV)
+    w = (torch.randn((H + 2 * K) * hd, d, generator=g) / math.sqrt(d)).to(dt).to(DEV)
+    inv = (1.0 / torch.pow(torch.tensor(500.0), torch.arange(0, rot, 2, dtype=torch.float32) / rot)).to(DEV)
+    pos = (torch.arange(T, dtype=torch.int32) + 60).to(DEV)
+    ts = torch.zeros(T, dtype=torch.int32, device=DEV)
+
+    def fresh():
+        c = Cache([KVSpec(max(K, 1), hd)], 512, 1024, dt, DEV, 2)
+        s_ = c.alloc_slot()
+        c.grow([s_], [60 + T])
+        return c, c.view(0)
+
+    c0, v0 = fresh()
+    qkv = ops.linear(x, w, out_dtype=torch.float32, force="fma")
+    args0 = (v0.page_table, v0.page_stride, v0.k, v0.v) if K else (None, None, None, None)
+    q0 = ops.rope_store(qkv, inv, rot, False, pos, ts, *args0, H, K, hd, dt)
+    kinds = ["fma", None] + (["gemv_mfma"] if T <= 16 else []) + ["mfma:0:1", "mfma:2:2"]
+    for tiled in (False, True):
+        if tiled and d % 32:
+            continue
+        ww = ops.tile_weight(w) if tiled else w
+        for kind in kinds:
+            if tiled and kind == "fma":
+                continue
+            c1, v1 = fresh()
+            args1 = (v1.page_table, v1.page_stride, v1.k, v1.v) if K else (None, None, None, None)
+            q1 = ops.linear_rope_store(x, ww, inv, rot, pos, ts, *args1, H, K, hd, dt, force=kind)
+            tol = 0 if kind == "fma" else 2e-2
+            assert (q1.float() - q0.float()).abs().max().item() <= tol * (1 + q0.float().abs().max().item()), kind
+            if K:
+                a, b = c0.groups[0].storage.float(), c1.groups[0].storage.float()
+                assert (a - b).abs().max().item() <= tol * (1 + a.abs().max().item()), kind
+                assert (b != 0).sum().item() >= 0.9 * T * 2 * K * hd
+
+
 def test_sampling_kernels(ops):
     import plain_llama as P
     g = torch.Generator().manual_seed(0)
