@@ -283,6 +283,169 @@ __global__ __launch_bounds__(256) void gemm_mfma_kernel(const T* __restrict__ X,
         }
 }
 
+// ===========================================================================
+// gemm_big: the prefill product.  BN rows of W x BM rows of X per workgroup of 4
+// waves (2 x 2), each wave a (BN/2) x (BM/2) tile of 32x32 blocks, BK = 64.  Two LDS
+// buffers: the next tile travels global -> registers while the matrix cores work on
+// the current one and is written to the other buffer afterwards, so there is one
+// barrier per tile.  With 256 x 256 tiles a wave issues 16 matrix instructions for
+// 8 LDS fragment reads.  W may be row-major or tiled.
+// ===========================================================================
+template <class T, int BN, int BM, int BK, bool TILED, bool EDGE>
+__global__ __launch_bounds__(256) void gemm_big_kernel(const T* __restrict__ X, const T* __restrict__ W,
+                                                       int K, Epilogue e) {
+    typedef typename Vec<T>::v8 v8;
+    constexpr int LD = BK + 8, CPR = BK / 8;             // chunks of 8 elements per tile row
+    constexpr int TN = BN / 2, TM = BM / 2;
+    constexpr int NB = TN / 32, MB = TM / 32;
+    constexpr int W_CHUNKS = BN * BK / 8 / 256, X_CHUNKS = BM * BK / 8 / 256;
+    constexpr int BUF = (BN + BM) * LD;                  // elements of one buffer
+    constexpr int KSTEPS = BK / 32;
+    extern __shared__ __attribute__((aligned(16))) unsigned char smem_raw[];
+    T* smem = (T*)smem_raw;
+
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int wn = wave & 1, wm = wave >> 1;
+    // consecutive workgroups share the rows of W (blockIdx.x runs over the tiles of X first)
+    const int m0 = blockIdx.x * BM, n0 = blockIdx.y * BN;
+    const int n_limit = TILED ? ((e.N + 15) & ~15) : e.N;
+
+    f32x16 acc[NB][MB];
+#pragma unroll
+    for (int a = 0; a < NB; ++a)
+#pragma unroll
+        for (int b = 0; b < MB; ++b)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) acc[a][b][r] = 0.f;
+
+    // Where each of this thread's 16-byte chunks of a tile comes from and goes to.  Row-major
+    // W: CPR threads a row; tiled W: 64 threads a (16 rows x 32 k) block, as it lies in memory.
+    // Loads are unconditional (addresses clamped into the matrix) and masked afterwards, so that
+    // the loads of two tiles can be in flight at once.
+    const T* wsrc[W_CHUNKS];
+    const T* xsrc[X_CHUNKS];
+    int wdst[W_CHUNKS], xdst[X_CHUNKS], wkc[W_CHUNKS], xkc[X_CHUNKS];
+    bool wok[W_CHUNKS], xok[X_CHUNKS];
+#pragma unroll
+    for (int c = 0; c < W_CHUNKS; ++c) {
+        const int chunk = tid + c * 256;
+        const int row = TILED ? ((chunk / (64 * KSTEPS)) << 4) + (chunk & 15) : chunk / CPR;
+        wkc[c] = TILED ? (((chunk >> 6) % KSTEPS) << 5) + (((chunk >> 4) & 3) << 3) : (chunk % CPR) * 8;
+        wok[c] = n0 + row < n_limit;
+        const int n = min(n0 + row, n_limit - 1);
+        wsrc[c] = TILED ? W + tiled_offset(n, wkc[c], K) : W + (int64_t)n * K + wkc[c];
+        wdst[c] = row * LD + wkc[c];
+    }
+#pragma unroll
+    for (int c = 0; c < X_CHUNKS; ++c) {
+        const int chunk = tid + c * 256, row = chunk / CPR;
+        xkc[c] = (chunk % CPR) * 8;
+        xok[c] = m0 + row < e.M;
+        xsrc[c] = X + (int64_t)min(m0 + row, e.M - 1) * K + xkc[c];
+        xdst[c] = BN * LD + row * LD + xkc[c];
+    }
+    // loads are raw; the mask (rows beyond the matrix, k beyond K) is applied when the tile is
+    // written to LDS, so that nothing waits for a load before then
+    // (EDGE false: M, N and K are whole numbers of tiles and nothing is masked)
+    auto load_tile = [&](int k0, v8 (&rw)[W_CHUNKS], v8 (&rx)[X_CHUNKS]) {
+        const int64_t wstep = TILED ? (int64_t)(k0 >> 5) * 512 : k0;
+#pragma unroll
+        for (int c = 0; c < W_CHUNKS; ++c) {
+            const bool in = !EDGE || k0 + wkc[c] < K;
+            rw[c] = *(const v8*)(wsrc[c] + (in ? wstep : 0));
+        }
+#pragma unroll
+        for (int c = 0; c < X_CHUNKS; ++c) {
+            const bool in = !EDGE || k0 + xkc[c] < K;
+            rx[c] = *(const v8*)(xsrc[c] + (in ? k0 : 0));
+        }
+    };
+    auto store_tile = [&](T* buf, int k0, const v8 (&rw)[W_CHUNKS], const v8 (&rx)[X_CHUNKS]) {
+        const v8 z = {};
+#pragma unroll
+        for (int c = 0; c < W_CHUNKS; ++c)
+            *(v8*)(buf + wdst[c]) = (!EDGE || (wok[c] && k0 + wkc[c] < K)) ? rw[c] : z;
+#pragma unroll
+        for (int c = 0; c < X_CHUNKS; ++c)
+            *(v8*)(buf + xdst[c]) = (!EDGE || (xok[c] && k0 + xkc[c] < K)) ? rx[c] : z;
+    };
+    auto compute = [&](const T* buf) {
+        const T* sW = buf;
+        const T* sX = buf + BN * LD;
+#pragma unroll
+        for (int ks = 0; ks < BK; ks += 16) {
+            v8 a[NB], b[MB];
+            const int kk = ks + 8 * (lane >> 5);
+#pragma unroll
+            for (int i = 0; i < NB; ++i) a[i] = *(const v8*)(sW + (wn * TN + i * 32 + (lane & 31)) * LD + kk);
+#pragma unroll
+            for (int j = 0; j < MB; ++j) b[j] = *(const v8*)(sX + (wm * TM + j * 32 + (lane & 31)) * LD + kk);
+#pragma unroll
+            for (int i = 0; i < NB; ++i)
+#pragma unroll
+                for (int j = 0; j < MB; ++j) acc[i][j] = mfma32(a[i], b[j], acc[i][j]);
+        }
+    };
+
+    // Tile t is computed from LDS buffer t % 2 while tile t + 1 waits in registers and the loads
+    // of tile t + 2 are issued: a load has more than one tile's worth of matrix work to arrive.
+    const int n_tiles = (K + BK - 1) / BK;
+    v8 rw0[W_CHUNKS], rx0[X_CHUNKS], rw1[W_CHUNKS], rx1[X_CHUNKS];
+    T* buf0 = smem;
+    T* buf1 = smem + BUF;
+    // (Loads and stores past the last tile are not branched around: they fetch the last tile again
+    // and write it where nothing reads it, which keeps the count of loads in flight fixed.)
+    const int k_last = (n_tiles - 1) * BK;
+    load_tile(0, rw0, rx0);
+    store_tile(buf0, 0, rw0, rx0);
+    load_tile(min(BK, k_last), rw1, rx1);
+    __syncthreads();
+    int t = 0;
+    for (; t + 1 < n_tiles; t += 2) {
+        // the scheduling barriers keep the loads at the head of each half and the LDS writes at
+        // its tail; left alone the compiler sinks the loads to just before their use
+        load_tile(min((t + 2) * BK, k_last), rw0, rx0);
+        __builtin_amdgcn_sched_barrier(0);
+        compute(buf0);
+        __builtin_amdgcn_sched_barrier(0);
+        store_tile(buf1, (t + 1) * BK, rw1, rx1);
+        __syncthreads();
+        load_tile(min((t + 3) * BK, k_last), rw1, rx1);
+        __builtin_amdgcn_sched_barrier(0);
+        compute(buf1);
+        __builtin_amdgcn_sched_barrier(0);
+        store_tile(buf0, min((t + 2) * BK, k_last), rw0, rx0);
+        __syncthreads();
+    }
+    if (t < n_tiles) compute(buf0);
+    __syncthreads();
+    // Epilogue through LDS: a wave lays each 32x32 block down as [row of X][32 columns] and reads it
+    // back so that 8 lanes write 32 consecutive columns of one row; the loop over the block's
+    // quads is not unrolled, which keeps one copy of the epilogue in the code.
+    constexpr int SLD = 36;                                  // floats per staged row (padded)
+    float* stage = (float*)smem_raw + wave * (32 * SLD);
+#pragma unroll
+    for (int i = 0; i < NB; ++i)
+#pragma unroll
+        for (int j = 0; j < MB; ++j) {
+#pragma unroll
+            for (int g = 0; g < 4; ++g) {
+                f32x4 v = {acc[i][j][4 * g], acc[i][j][4 * g + 1], acc[i][j][4 * g + 2], acc[i][j][4 * g + 3]};
+                *(f32x4*)(stage + (lane & 31) * SLD + 8 * g + 4 * (lane >> 5)) = v;
+            }
+            __builtin_amdgcn_wave_barrier();
+            const int mb = m0 + wm * TM + j * 32, nb = n0 + wn * TN + i * 32;
+#pragma unroll 1
+            for (int q = lane; q < 256; q += 64) {
+                const int r = q >> 3, c = (q & 7) * 4;
+                const f32x4 v = *(const f32x4*)(stage + r * SLD + c);
+                const float vv[4] = {v[0], v[1], v[2], v[3]};
+                epilogue4(e, mb + r, nb + c, vv);
+            }
+            __builtin_amdgcn_wave_barrier();
+        }
+}
+
 // Sum of the split-K partials in ascending split order, then the epilogue.
 __global__ void splitk_reduce_kernel(const float* __restrict__ ws, int splits, Epilogue e) {
     const int64_t quads_per_row = (e.N + 3) >> 2;
@@ -716,6 +879,42 @@ extern "C" int li_gemv_tiled(const void* X, const void* Wt, int dt, void* C, int
     if (dt == DT_F16) PICK(f16); else PICK(bf16);
 #undef PICK
 #undef LAUNCH
+    LI_CHECK_LAUNCH();
+    return LI_OK;
+}
+
+// tile (rows of W x rows of X / depth): 0 = 128x128/64, 1 = 256x128/32
+extern "C" int li_gemm_big(const void* X, const void* W, int tiled, int dt, void* C, int out_dt, int mode,
+                           int M, int N, int K, int tile, const RopeStore* rs, hipStream_t stream) {
+    int rc = check_common(X, W, C, M, N, K, mode, out_dt);
+    if (rc) return rc;
+    if (dt != DT_F16 && dt != DT_BF16) return LI_BAD_ARG;
+    if (K % 8 != 0 || ((uintptr_t)X & 15) || ((uintptr_t)W & 15)) return LI_UNSUPPORTED;
+    if (tiled && K % 32 != 0) return LI_UNSUPPORTED;
+    if (tile < 0 || tile > 1) return LI_BAD_ARG;
+    if (M == 0) return LI_OK;
+    Epilogue e;
+    rc = make_epilogue(e, C, mode, out_dt, M, N, rs);
+    if (rc) return rc;
+    const int bn = tile ? 256 : 128, bm = 128, bk = tile ? 32 : 64;
+    const size_t lds = (size_t)2 * (bn + bm) * (bk + 8) * 2;
+    dim3 grid((M + bm - 1) / bm, (N + bn - 1) / bn), block(256);
+    const bool edge = (M % bm) || (N % bn) || (K % bk);
+#define GO(T, BN, BM, BK, TL)                                                                          \
+    do {                                                                                               \
+        auto kfn = edge ? gemm_big_kernel<T, BN, BM, BK, TL, true> : gemm_big_kernel<T, BN, BM, BK, TL, false>; \
+        if (hipFuncSetAttribute((const void*)kfn, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds) != hipSuccess) \
+            return LI_HIP_ERROR;                                                                       \
+        kfn<<<grid, block, lds, stream>>>((const T*)X, (const T*)W, K, e);                             \
+    } while (0)
+#define LAUNCH(T)                                                                                     \
+    do {                                                                                              \
+        if (tile == 0) { if (tiled) GO(T, 128, 128, 64, true); else GO(T, 128, 128, 64, false); }     \
+        else { if (tiled) GO(T, 256, 128, 32, true); else GO(T, 256, 128, 32, false); }               \
+    } while (0)
+    if (dt == DT_F16) LAUNCH(f16); else LAUNCH(bf16);
+#undef LAUNCH
+#undef GO
     LI_CHECK_LAUNCH();
     return LI_OK;
 }

@@ -161,7 +161,7 @@ def linear(x: torch.Tensor, w, mode: int = EPI_STORE, out: torch.Tensor | None =
     lib = core()
     same16 = x.dtype == w.dtype and x.dtype in (torch.float16, torch.bfloat16)
     fast_ok = same16 and k % 8 == 0 and x.data_ptr() % 16 == 0 and wd.data_ptr() % 16 == 0
-    kind = force or ("fma" if not fast_ok else ("gemv_mfma" if m <= 16 else "mfma"))
+    kind = force or ("fma" if not fast_ok else ("gemv_mfma" if m <= 16 else ("big" if m > 128 else "mfma")))
     if tiled:
         _need(fast_ok and kind != "fma" and kind != "gemv", "a tiled weight needs 16-bit activations of its dtype")
         if kind == "gemv_mfma":
@@ -178,6 +178,11 @@ def linear(x: torch.Tensor, w, mode: int = EPI_STORE, out: torch.Tensor | None =
     elif kind == "gemv":
         _need(fast_ok and m <= 8, "gemv: 16-bit operands, K a multiple of 8, at most 8 rows")
         _check(lib.li_gemv(_ptr(x), _ptr(w), DT[x.dtype], _ptr(out), out_dt, mode, m, n, k, rs, _stream()), "gemv")
+    elif kind.startswith("big"):
+        _need(fast_ok, "gemm_big: 16-bit operands and K a multiple of 8")
+        tile = int(kind.split(":")[1]) if ":" in kind else _big_tile(m, n)
+        _check(lib.li_gemm_big(_ptr(x), _ptr(wd), int(tiled), DT[x.dtype], _ptr(out), out_dt, mode, m, n, k, tile,
+                               rs, _stream()), "gemm_big")
     else:
         _need(fast_ok, "gemm_mfma: 16-bit operands and K a multiple of 8")
         tile = 0 if m > 64 else (1 if m > 32 else 2)
@@ -193,6 +198,12 @@ def linear(x: torch.Tensor, w, mode: int = EPI_STORE, out: torch.Tensor | None =
         _check(lib.li_gemm_mfma(_ptr(x), _ptr(wd), int(tiled), DT[x.dtype], _ptr(out), out_dt, mode, m, n, k,
                                 tile, splits, _ptr(ws), rs, _stream()), "gemm_mfma")
     return out
+
+
+def _big_tile(m: int, n: int) -> int:
+    """The tile of gemm_big for a product of this size (measured on MI355X): the wider tile pays
+    once there are several rounds of workgroups for the chip's 256 CUs."""
+    return 1 if (-(-m // 128)) * (-(-n // 256)) >= 1024 else 0
 
 
 def swiglu(gu: torch.Tensor, out_dtype) -> torch.Tensor:

@@ -64,7 +64,7 @@ def _linear_ref(x, w, mode, res=None):
 
 LIN_CASES = [  # M, N, K
     (1, 64, 64), (2, 16400, 4096), (16, 1000, 2056), (9, 40, 4104), (3, 172, 96), (8, 100, 256), (5, 6, 8), (13, 344, 64), (33, 130, 136),
-    (64, 256, 512), (70, 200, 1024), (129, 384, 320), (200, 136, 72), (256, 512, 2048),
+    (64, 256, 512), (70, 200, 1024), (129, 384, 320), (200, 136, 72), (256, 512, 2048), (384, 256, 192),
 ]
 
 
@@ -81,7 +81,7 @@ def test_linear_all_kernels_and_epilogues(ops, M, N, K, dt):
             kinds.append("gemv")
         if M <= 16:
             kinds.append("gemv_mfma")
-        kinds += ["mfma:0:1", "mfma:1:1", "mfma:2:1", "mfma:2:3", "mfma:0:2", None]
+        kinds += ["mfma:0:1", "mfma:1:1", "mfma:2:1", "mfma:2:3", "mfma:0:2", "big:0", "big:1", None]
     for kind in kinds:
         for mode in (0, 1, 2):
             if mode == 2 and N % 2:
@@ -106,7 +106,7 @@ def test_linear_all_kernels_and_epilogues(ops, M, N, K, dt):
 
 
 TILED_CASES = [(1, 64, 64), (3, 172, 96), (16, 40, 4096), (9, 16400, 256), (17, 100, 64), (64, 256, 512),
-               (70, 200, 1024), (129, 384, 320), (256, 520, 2048)]
+               (70, 200, 1024), (129, 384, 320), (256, 520, 2048), (384, 512, 192), (300, 1000, 96)]
 
 
 @pytest.mark.parametrize("M,N,K", TILED_CASES)
@@ -119,7 +119,7 @@ def test_linear_tiled_weights(ops, M, N, K, dt):
     res = torch.randn(M, N, generator=g).to(DEV)
     wt = ops.tile_weight(w)
     assert wt.shape == (N, K) and wt.data.numel() == (N + 15) // 16 * 16 * K
-    kinds = [None, "mfma:0:1", "mfma:1:2", "mfma:2:1"] + (["gemv_mfma"] if M <= 16 else [])
+    kinds = [None, "mfma:0:1", "mfma:1:2", "mfma:2:1", "big:0", "big:1"] + (["gemv_mfma"] if M <= 16 else [])
     for kind in kinds:
         for mode in (0, 1, 2):
             if mode == 2 and N % 2:
