@@ -78,7 +78,6 @@ struct WaveAttn {
     // maximum and sum; leaves the probabilities in s.  This lane's row sees keys lo..hi.
     __device__ __forceinline__ void scores(const v8 (&kf)[2 * KS], f32x16 (&s)[2], int t0, int lo, int hi,
                                            float scale2) {
-        const int lane = threadIdx.x & 63;
 #pragma unroll
         for (int b = 0; b < 2; ++b) {
 #pragma unroll
@@ -86,6 +85,28 @@ struct WaveAttn {
 #pragma unroll
             for (int ks = 0; ks < KS; ++ks) s[b] = mfma32(kf[b * KS + ks], q[ks], s[b]);
         }
+        softmax_step(s, t0, lo, hi, scale2);
+    }
+
+    // The same with the key fragments fetched where they are used.
+    __device__ __forceinline__ void scores_streamed(const T* kpage, f32x16 (&s)[2], int t0, int lo, int hi,
+                                                    float scale2) {
+        const int lane = threadIdx.x & 63;
+#pragma unroll
+        for (int b = 0; b < 2; ++b) {
+#pragma unroll
+            for (int r = 0; r < 16; ++r) s[b][r] = 0.f;
+#pragma unroll
+            for (int ks = 0; ks < KS; ++ks) {
+                const v8 kf = *(const v8*)(kpage + ((b * KS + ks) * 64 + lane) * 8);
+                s[b] = mfma32(kf, q[ks], s[b]);
+            }
+        }
+        softmax_step(s, t0, lo, hi, scale2);
+    }
+
+    __device__ __forceinline__ void softmax_step(f32x16 (&s)[2], int t0, int lo, int hi, float scale2) {
+        const int lane = threadIdx.x & 63;
         float mx = -INFINITY;
 #pragma unroll
         for (int b = 0; b < 2; ++b)
@@ -133,10 +154,8 @@ struct WaveAttn {
     // register count low enough for several waves per SIMD.
     __device__ __forceinline__ void page(const T* kpage, const T* vpage, int t0, int lo, int hi, float scale2) {
         const int lane = threadIdx.x & 63;
-        v8 kf[2 * KS];
         f32x16 s[2];
-        load_k(kpage, kf);
-        scores(kf, s, t0, lo, hi, scale2);
+        scores_streamed(kpage, s, t0, lo, hi, scale2);
 #pragma unroll
         for (int tj = 0; tj < 4; ++tj) {
             v8 pf;
@@ -154,19 +173,35 @@ struct WaveAttn {
 };
 
 // ---------------------------------------------------------------------------
-// prefill
+// prefill.  A workgroup of 4 waves shares the pages of one KV head through LDS (two
+// buffers: page p+1 travels global -> registers -> LDS while page p is used).  With GW
+// query heads of a KV head packed into a workgroup (GW = 4, 2 or 1, the largest that
+// divides the group), wave w owns head w % GW and the 32-token block w / GW of the
+// workgroup's 128 / GW tokens, so every page is fetched once for up to 4 heads.
 // ---------------------------------------------------------------------------
 template <class T>
-__global__ __launch_bounds__(256) void attn_prefill_kernel(
+__global__ __launch_bounds__(256, HD <= 128 ? 2 : 1) void attn_prefill_kernel(
     const T* __restrict__ q, T* __restrict__ out, CachePtrs c, const int* __restrict__ tile_seq,
     const int* __restrict__ tile_q0, const int* __restrict__ seq_slot, const int* __restrict__ seq_qstart,
-    const int* __restrict__ seq_qlen, const int* __restrict__ seq_ctx, int H, int K, float scale, int window) {
-    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-    const int seq = tile_seq[blockIdx.x];
-    const int h = blockIdx.y, kvh = h / (H / K);
+    const int* __restrict__ seq_qlen, const int* __restrict__ seq_ctx, int H, int K, float scale, int window,
+    int GW) {
+    typedef typename Vec<T>::v8 v8;
+    constexpr int KE = PAGE * HD, VE = PAGE * DB * 32;           // elements of a head's keys / values in a page
+    constexpr int CK = (KE / 8 + 255) / 256, CV = (VE / 8 + 255) / 256;
+    extern __shared__ __attribute__((aligned(16))) unsigned char smem_raw[];
+    T* smem = (T*)smem_raw;
+
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int G = H / K, TT = 32 * (4 / GW);                     // tokens of this workgroup
+    const int tile = blockIdx.x / GW, sub = blockIdx.x % GW;
+    const int seq = tile_seq[tile];
+    const int kvh = blockIdx.y / (G / GW), hc = blockIdx.y % (G / GW);
+    const int h = kvh * G + hc * GW + wave % GW;
     const int qlen = seq_qlen[seq], ctx = seq_ctx[seq];
-    const int first = tile_q0[blockIdx.x] + 32 * wave;          // this wave's first token within the step
-    if (first >= qlen) return;
+    const int q0 = tile_q0[tile] + sub * TT;                     // first token of the workgroup within the step
+    if (q0 >= qlen) return;                                      // the same for all waves
+    const int first = q0 + 32 * (wave / GW);                     // this wave's first token
+    const bool wave_live = first < qlen;
     const int qi = first + (lane & 31);
     const bool live = qi < qlen;
     const int base = ctx - qlen;                                 // tokens cached before this step
@@ -175,15 +210,53 @@ __global__ __launch_bounds__(256) void attn_prefill_kernel(
     WaveAttn<T> a;
     a.init(live ? q + (tok * H + h) * HD : nullptr);
     const int lo = (window > 0 && live) ? max(0, pos - window + 1) : 0;
-    const int last_pos = base + min(first + 31, qlen - 1);
-    const int first_lo = window > 0 ? max(0, base + first - window + 1) : 0;
+    // pages of the workgroup and of this wave
+    const int p_lo = (window > 0 ? max(0, base + q0 - window + 1) : 0) / PAGE;
+    const int p_hi = (base + min(q0 + TT - 1, qlen - 1)) / PAGE;
+    const int wp_lo = (window > 0 ? max(0, base + first - window + 1) : 0) / PAGE;
+    const int wp_hi = wave_live ? (base + min(first + 31, qlen - 1)) / PAGE : -1;
     const int* table = c.page_table + (int64_t)seq_slot[seq] * c.max_pages;
+    const T* kbase = (const T*)c.k + (int64_t)kvh * k_head_elems(HD);
+    const T* vbase = (const T*)c.v + (int64_t)kvh * v_head_elems(HD);
     const float scale2 = scale * LOG2E;
-    for (int p = first_lo / PAGE; p <= last_pos / PAGE; ++p) {
-        const int64_t page = table[p];
-        const T* kp = (const T*)c.k + page * c.page_stride + (int64_t)kvh * k_head_elems(HD);
-        const T* vp = (const T*)c.v + page * c.page_stride + (int64_t)kvh * v_head_elems(HD);
-        a.page(kp, vp, p * PAGE, lo, pos, scale2);
+
+    v8 rk[CK], rv[CV];
+    auto fetch = [&](int p) {
+        const int64_t page = (int64_t)table[p] * c.page_stride;
+#pragma unroll
+        for (int i = 0; i < CK; ++i) {
+            const int ch = tid + i * 256;
+            if (KE / 8 % 256 == 0 || ch < KE / 8) rk[i] = *(const v8*)(kbase + page + ch * 8);
+        }
+#pragma unroll
+        for (int i = 0; i < CV; ++i) {
+            const int ch = tid + i * 256;
+            if (VE / 8 % 256 == 0 || ch < VE / 8) rv[i] = *(const v8*)(vbase + page + ch * 8);
+        }
+    };
+    auto stash = [&](T* buf) {
+#pragma unroll
+        for (int i = 0; i < CK; ++i) {
+            const int ch = tid + i * 256;
+            if (KE / 8 % 256 == 0 || ch < KE / 8) *(v8*)(buf + ch * 8) = rk[i];
+        }
+#pragma unroll
+        for (int i = 0; i < CV; ++i) {
+            const int ch = tid + i * 256;
+            if (VE / 8 % 256 == 0 || ch < VE / 8) *(v8*)(buf + KE + ch * 8) = rv[i];
+        }
+    };
+
+    fetch(p_lo);
+    stash(smem);
+    __syncthreads();
+    for (int p = p_lo; p <= p_hi; ++p) {
+        T* cur = smem + ((p - p_lo) & 1) * (KE + VE);
+        T* nxt = smem + ((p - p_lo + 1) & 1) * (KE + VE);
+        if (p < p_hi) fetch(p + 1);
+        if (p >= wp_lo && p <= wp_hi) a.page(cur, cur + KE, p * PAGE, lo, pos, scale2);
+        if (p < p_hi) stash(nxt);
+        __syncthreads();
     }
     const float inv = 1.f / a.total();
     if (!live) return;
@@ -361,15 +434,22 @@ extern "C" int li_attn_prefill(const void* q, void* out, int dt, const void* k, 
     if (check_heads(H, K)) return LI_BAD_ARG;
     if (n_tiles <= 0) return LI_OK;
     CachePtrs c{k, v, page_stride, page_table, max_pages};
-    dim3 grid(n_tiles, H), block(256);
-    if (dt == DT_F16)
-        attn_prefill_kernel<f16><<<grid, block, 0, stream>>>((const f16*)q, (f16*)out, c, tile_seq, tile_q0, seq_slot,
-                                                             seq_qstart, seq_qlen, seq_ctx, H, K, scale, window);
-    else if (dt == DT_BF16)
-        attn_prefill_kernel<bf16><<<grid, block, 0, stream>>>((const bf16*)q, (bf16*)out, c, tile_seq, tile_q0,
-                                                              seq_slot, seq_qstart, seq_qlen, seq_ctx, H, K, scale,
-                                                              window);
+    const int G = H / K;
+    const int gw = G % 4 == 0 ? 4 : (G % 2 == 0 ? 2 : 1);        // query heads of a KV head per workgroup
+    dim3 grid(n_tiles * gw, K * (G / gw)), block(256);
+    const size_t lds = (size_t)2 * (PAGE * HD + PAGE * DB * 32) * 2;
+#define GO(T)                                                                                                  \
+    do {                                                                                                       \
+        auto kfn = attn_prefill_kernel<T>;                                                                     \
+        if (hipFuncSetAttribute((const void*)kfn, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds) != hipSuccess) \
+            return LI_HIP_ERROR;                                                                               \
+        kfn<<<grid, block, lds, stream>>>((const T*)q, (T*)out, c, tile_seq, tile_q0, seq_slot, seq_qstart,    \
+                                          seq_qlen, seq_ctx, H, K, scale, window, gw);                         \
+    } while (0)
+    if (dt == DT_F16) GO(f16);
+    else if (dt == DT_BF16) GO(bf16);
     else return LI_BAD_ARG;
+#undef GO
     LI_CHECK_LAUNCH();
     return LI_OK;
 }
