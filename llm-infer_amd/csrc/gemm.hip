@@ -8,8 +8,9 @@
 //              It is the true 32-bit path and the fallback for K not a multiple of 8.
 //   gemm_mfma  16-bit operands on the matrix cores (32x32x16), tiles staged through
 //              LDS, optional split over K into a float32 workspace.
-//   gemv       16-bit operands, up to 8 rows of X: W is streamed once with 16-byte
-//              loads, X sits in LDS, v_dot2 accumulates in float32.
+//   gemm_big   the prefill product: larger tiles, two LDS buffers, loads two tiles ahead.
+//   gemv_mfma  up to 16 rows of X (row-major W), gemv_tiled up to 64 rows (tiled W): W is
+//              streamed once from HBM straight into the matrix cores' operand registers.
 #include "common.h"
 
 enum { EPI_STORE = 0, EPI_ADD = 1, EPI_SWIGLU = 2, EPI_ROPE = 3 };
@@ -462,67 +463,6 @@ __global__ void splitk_reduce_kernel(const float* __restrict__ ws, int splits, E
 }
 
 // ===========================================================================
-// gemv: MB <= 8 rows of X against R rows of W per wave.
-// ===========================================================================
-template <class T, int MB, int R>
-__global__ __launch_bounds__(256) void gemv_kernel(const T* __restrict__ X, const T* __restrict__ W,
-                                                   int K, Epilogue e) {
-    typedef typename Vec<T>::v8 v8;
-    typedef typename Vec<T>::v2 v2;
-    constexpr int KC = 2048;                             // elements of K staged at a time
-    __shared__ __attribute__((aligned(16))) T sx[MB * KC];
-    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-    const int n_base = (blockIdx.x * 4 + wave) * R;
-    float acc[R][MB];
-#pragma unroll
-    for (int r = 0; r < R; ++r)
-#pragma unroll
-        for (int m = 0; m < MB; ++m) acc[r][m] = 0.f;
-    const T* wrow[R];
-#pragma unroll
-    for (int r = 0; r < R; ++r) wrow[r] = W + (int64_t)min(n_base + r, e.N - 1) * K;
-
-    for (int kc = 0; kc < K; kc += KC) {
-        const int len = min(KC, K - kc);                 // a multiple of 8
-        __syncthreads();
-        for (int c = tid; c < MB * (KC / 8); c += 256) {
-            const int m = c / (KC / 8), k = (c % (KC / 8)) * 8;
-            v8 z = {};
-            *(v8*)(sx + m * KC + k) = (m < e.M && k < len) ? *(const v8*)(X + (int64_t)m * K + kc + k) : z;
-        }
-        __syncthreads();
-        for (int k = lane * 8; k < len; k += 64 * 8) {
-            v8 w[R];
-#pragma unroll
-            for (int r = 0; r < R; ++r) w[r] = *(const v8*)(wrow[r] + kc + k);
-#pragma unroll
-            for (int m = 0; m < MB; ++m) {
-                const v8 xv = *(const v8*)(sx + m * KC + k);
-#pragma unroll
-                for (int r = 0; r < R; ++r)
-#pragma unroll
-                    for (int p = 0; p < 4; ++p) {
-                        v2 a = {w[r][2 * p], w[r][2 * p + 1]};
-                        v2 b = {xv[2 * p], xv[2 * p + 1]};
-                        acc[r][m] = dot2(a, b, acc[r][m]);
-                    }
-            }
-        }
-    }
-#pragma unroll
-    for (int m = 0; m < MB; ++m) {
-        float v[R];
-#pragma unroll
-        for (int r = 0; r < R; ++r) v[r] = wave_sum(acc[r][m]);
-        if (lane == 0) {
-#pragma unroll
-            for (int r = 0; r < R; r += 4) epilogue4(e, m, n_base + r, v + r);
-        }
-    }
-}
-
-
-// ===========================================================================
 // gemv_mfma: up to 16 rows of X on the matrix cores (16x16x32), W streamed from
 // global memory straight into operand A.  A wave owns NT tiles of 16 rows of W
 // and one slice of K; the KW waves of a workgroup cover K and their partial
@@ -631,12 +571,14 @@ __global__ void tile_weight_kernel(const T* __restrict__ W, T* __restrict__ out,
     *(v8*)(out + i * 8) = n < N ? *(const v8*)(W + (int64_t)n * K + k) : z;
 }
 
-template <class T, int NT, int KW>
+template <class T, int NT, int MT, int KW>
 __global__ __launch_bounds__(64 * KW) void gemv_tiled_kernel(const T* __restrict__ X, const T* __restrict__ Wt,
                                                              int K, Epilogue e) {
+    // NT tiles of 16 rows of W and MT tiles of 16 rows of X per wave; W comes from HBM once, the
+    // rows of X from the caches (they are few)
     typedef typename Vec<T>::v8 v8;
-    constexpr int U = 8;                                  // 32-element steps of K in flight
-    __shared__ float part[KW][NT][64][4];
+    constexpr int U = (NT + MT) <= 2 ? 8 : ((NT + MT) <= 4 ? 4 : 2);   // 32-element steps of K in flight
+    __shared__ float part[KW][NT * MT][64][4];
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int r = lane & 15, g = lane >> 4;
     const int tile0 = blockIdx.x * NT;
@@ -647,47 +589,63 @@ __global__ __launch_bounds__(64 * KW) void gemv_tiled_kernel(const T* __restrict
     const T* wt[NT];
 #pragma unroll
     for (int t = 0; t < NT; ++t) wt[t] = Wt + ((int64_t)min(tile0 + t, n_tiles - 1) * steps * 64 + lane) * 8;
-    const bool have_x = r < e.M;
-    const T* xrow = X + (int64_t)(have_x ? r : 0) * K + 8 * g;
-    f32x4 acc[NT];
+    bool have_x[MT];
+    const T* xrow[MT];
 #pragma unroll
-    for (int t = 0; t < NT; ++t) acc[t] = f32x4{0.f, 0.f, 0.f, 0.f};
+    for (int j = 0; j < MT; ++j) {
+        have_x[j] = 16 * j + r < e.M;
+        xrow[j] = X + (int64_t)(have_x[j] ? 16 * j + r : 0) * K + 8 * g;
+    }
+    f32x4 acc[NT][MT];
+#pragma unroll
+    for (int t = 0; t < NT; ++t)
+#pragma unroll
+        for (int j = 0; j < MT; ++j) acc[t][j] = f32x4{0.f, 0.f, 0.f, 0.f};
     for (int s0 = s_begin; s0 < s_end; s0 += U) {
-        v8 a[U][NT], b[U];
+        v8 a[U][NT], b[U][MT];
 #pragma unroll
         for (int u = 0; u < U; ++u) {
             const bool in = s0 + u < s_end;
             const v8 z = {};
 #pragma unroll
             for (int t = 0; t < NT; ++t) a[u][t] = in ? *(const v8*)(wt[t] + (int64_t)(s0 + u) * 512) : z;
-            b[u] = (in && have_x) ? *(const v8*)(xrow + (s0 + u) * 32) : z;
+#pragma unroll
+            for (int j = 0; j < MT; ++j) b[u][j] = (in && have_x[j]) ? *(const v8*)(xrow[j] + (s0 + u) * 32) : z;
         }
 #pragma unroll
         for (int u = 0; u < U; ++u)
 #pragma unroll
-            for (int t = 0; t < NT; ++t) acc[t] = mfma16(a[u][t], b[u], acc[t]);
+            for (int t = 0; t < NT; ++t)
+#pragma unroll
+                for (int j = 0; j < MT; ++j) acc[t][j] = mfma16(a[u][t], b[u][j], acc[t][j]);
     }
     if (KW > 1) {
 #pragma unroll
         for (int t = 0; t < NT; ++t)
 #pragma unroll
-            for (int q = 0; q < 4; ++q) part[wave][t][lane][q] = acc[t][q];
+            for (int j = 0; j < MT; ++j)
+#pragma unroll
+                for (int q = 0; q < 4; ++q) part[wave][t * MT + j][lane][q] = acc[t][j][q];
         __syncthreads();
         if (wave != 0) return;
 #pragma unroll
         for (int t = 0; t < NT; ++t)
 #pragma unroll
-            for (int q = 0; q < 4; ++q) {
-                float v = part[0][t][lane][q];
-                for (int w = 1; w < KW; ++w) v += part[w][t][lane][q];
-                acc[t][q] = v;
-            }
+            for (int j = 0; j < MT; ++j)
+#pragma unroll
+                for (int q = 0; q < 4; ++q) {
+                    float v = part[0][t * MT + j][lane][q];
+                    for (int w = 1; w < KW; ++w) v += part[w][t * MT + j][lane][q];
+                    acc[t][j][q] = v;
+                }
     }
 #pragma unroll
-    for (int t = 0; t < NT; ++t) {
-        float v[4] = {acc[t][0], acc[t][1], acc[t][2], acc[t][3]};
-        epilogue4(e, r, (tile0 + t) * 16 + 4 * g, v);
-    }
+    for (int t = 0; t < NT; ++t)
+#pragma unroll
+        for (int j = 0; j < MT; ++j) {
+            float v[4] = {acc[t][j][0], acc[t][j][1], acc[t][j][2], acc[t][j][3]};
+            epilogue4(e, 16 * j + r, (tile0 + t) * 16 + 4 * g, v);
+        }
 }
 
 // ===========================================================================
@@ -781,32 +739,6 @@ extern "C" int li_gemm_mfma(const void* X, const void* W, int tiled, int dt, voi
     return LI_OK;
 }
 
-extern "C" int li_gemv(const void* X, const void* W, int dt, void* C, int out_dt, int mode,
-                       int M, int N, int K, const RopeStore* rs, hipStream_t stream) {
-    int rc = check_common(X, W, C, M, N, K, mode, out_dt);
-    if (rc) return rc;
-    if (dt != DT_F16 && dt != DT_BF16) return LI_BAD_ARG;
-    if (M > 8) return LI_BAD_ARG;
-    if (K % 8 != 0 || ((uintptr_t)X & 15) || ((uintptr_t)W & 15)) return LI_UNSUPPORTED;
-    if (M == 0) return LI_OK;
-    Epilogue e;
-    rc = make_epilogue(e, C, mode, out_dt, M, N, rs);
-    if (rc) return rc;
-    constexpr int R = 4;
-    dim3 grid((N + 4 * R - 1) / (4 * R)), block(256);
-#define LAUNCH(T)                                                                                    \
-    do {                                                                                             \
-        if (M == 1) gemv_kernel<T, 1, R><<<grid, block, 0, stream>>>((const T*)X, (const T*)W, K, e); \
-        else if (M == 2) gemv_kernel<T, 2, R><<<grid, block, 0, stream>>>((const T*)X, (const T*)W, K, e); \
-        else if (M <= 4) gemv_kernel<T, 4, R><<<grid, block, 0, stream>>>((const T*)X, (const T*)W, K, e); \
-        else gemv_kernel<T, 8, R><<<grid, block, 0, stream>>>((const T*)X, (const T*)W, K, e);       \
-    } while (0)
-    if (dt == DT_F16) LAUNCH(f16); else LAUNCH(bf16);
-#undef LAUNCH
-    LI_CHECK_LAUNCH();
-    return LI_OK;
-}
-
 extern "C" int li_gemv_mfma(const void* X, const void* W, int dt, void* C, int out_dt, int mode,
                             int M, int N, int K, const RopeStore* rs, hipStream_t stream) {
     int rc = check_common(X, W, C, M, N, K, mode, out_dt);
@@ -853,31 +785,40 @@ extern "C" int li_gemv_tiled(const void* X, const void* Wt, int dt, void* C, int
     int rc = check_common(X, Wt, C, M, N, K, mode, out_dt);
     if (rc) return rc;
     if (dt != DT_F16 && dt != DT_BF16) return LI_BAD_ARG;
-    if (M > 16) return LI_BAD_ARG;
+    if (M > 64) return LI_BAD_ARG;
     if (K % 32 != 0 || ((uintptr_t)X & 15) || ((uintptr_t)Wt & 15)) return LI_UNSUPPORTED;
     if (M == 0) return LI_OK;
     Epilogue e;
     rc = make_epilogue(e, C, mode, out_dt, M, N, rs);
     if (rc) return rc;
     const int n_tiles = (N + 15) / 16;
-    if (nt <= 0) nt = 1;
+    const int mt = (M + 15) / 16;
+    if (nt <= 0) nt = mt >= 2 ? 2 : 1;
+    if (mt >= 3) nt = 2;
     const int blocks = (n_tiles + nt - 1) / nt;
     if (kw <= 0) kw = (K >= 8192 || blocks < 320 || blocks > 4096) ? 8 : 4;   // measured on MI355X
-#define LAUNCH(T, NT, KW) gemv_tiled_kernel<T, NT, KW><<<blocks, 64 * KW, 0, stream>>>((const T*)X, (const T*)Wt, K, e)
-#define PICK(T)                                          \
-    do {                                                 \
-        if (nt == 2 && kw == 4) LAUNCH(T, 2, 4);         \
-        else if (nt == 2 && kw == 8) LAUNCH(T, 2, 8);    \
-        else if (nt == 2 && kw == 2) LAUNCH(T, 2, 2);    \
-        else if (nt == 1 && kw == 4) LAUNCH(T, 1, 4);    \
-        else if (nt == 1 && kw == 8) LAUNCH(T, 1, 8);    \
-        else if (nt == 1 && kw == 16) LAUNCH(T, 1, 16);  \
-        else if (nt == 4 && kw == 4) LAUNCH(T, 4, 4);    \
-        else if (nt == 4 && kw == 2) LAUNCH(T, 4, 2);    \
-        else return LI_BAD_ARG;                          \
+    while (kw * nt * (mt == 3 ? 4 : mt) > 64) kw >>= 1;                       // the partial sums fit 64 KiB of LDS
+    if (kw < 2) return LI_BAD_ARG;
+#define LAUNCH(T, NT, MT, KW) \
+    gemv_tiled_kernel<T, NT, MT, KW><<<blocks, 64 * KW, 0, stream>>>((const T*)X, (const T*)Wt, K, e)
+#define PICK_KW(T, NT, MT)                                \
+    do {                                                  \
+        if (kw == 4) LAUNCH(T, NT, MT, 4);                \
+        else if (kw == 8) LAUNCH(T, NT, MT, 8);           \
+        else return LI_BAD_ARG;                           \
+    } while (0)
+#define PICK(T)                                           \
+    do {                                                  \
+        if (mt == 1 && nt == 1) PICK_KW(T, 1, 1);         \
+        else if (mt == 1 && nt == 2) PICK_KW(T, 2, 1);    \
+        else if (mt == 2 && nt == 1) PICK_KW(T, 1, 2);    \
+        else if (mt == 2 && nt == 2) PICK_KW(T, 2, 2);    \
+        else if (mt <= 4 && nt == 2) PICK_KW(T, 2, 4);    \
+        else return LI_BAD_ARG;                           \
     } while (0)
     if (dt == DT_F16) PICK(f16); else PICK(bf16);
 #undef PICK
+#undef PICK_KW
 #undef LAUNCH
     LI_CHECK_LAUNCH();
     return LI_OK;

@@ -163,8 +163,10 @@ def linear(x: torch.Tensor, w, mode: int = EPI_STORE, out: torch.Tensor | None =
     fast_ok = same16 and k % 8 == 0 and x.data_ptr() % 16 == 0 and wd.data_ptr() % 16 == 0
     kind = force or ("fma" if not fast_ok else ("gemv_mfma" if m <= 16 else ("big" if m > 128 else "mfma")))
     if tiled:
-        _need(fast_ok and kind != "fma" and kind != "gemv", "a tiled weight needs 16-bit activations of its dtype")
-        if kind == "gemv_mfma":
+        _need(fast_ok and kind != "fma", "a tiled weight needs 16-bit activations of its dtype")
+        # up to 64 rows the weight is streamed once past all rows of X; beyond 32 rows that pays
+        # only for matrices small enough that the tiled GEMM cannot fill the chip
+        if kind == "gemv_mfma" or (force is None and (m <= 32 or (m <= 64 and n * k <= (1 << 25)))):
             _check(lib.li_gemv_tiled(_ptr(x), _ptr(wd), DT[x.dtype], _ptr(out), out_dt, mode, m, n, k, 0, 0,
                                      rs, _stream()), "gemv_tiled")
             return out
@@ -175,9 +177,6 @@ def linear(x: torch.Tensor, w, mode: int = EPI_STORE, out: torch.Tensor | None =
         _need(fast_ok and m <= 16, "gemv_mfma: 16-bit operands, K a multiple of 8, at most 16 rows")
         _check(lib.li_gemv_mfma(_ptr(x), _ptr(w), DT[x.dtype], _ptr(out), out_dt, mode, m, n, k, rs, _stream()),
                "gemv_mfma")
-    elif kind == "gemv":
-        _need(fast_ok and m <= 8, "gemv: 16-bit operands, K a multiple of 8, at most 8 rows")
-        _check(lib.li_gemv(_ptr(x), _ptr(w), DT[x.dtype], _ptr(out), out_dt, mode, m, n, k, rs, _stream()), "gemv")
     elif kind.startswith("big"):
         _need(fast_ok, "gemm_big: 16-bit operands and K a multiple of 8")
         tile = int(kind.split(":")[1]) if ":" in kind else _big_tile(m, n)

@@ -77,8 +77,6 @@ def test_linear_all_kernels_and_epilogues(ops, M, N, K, dt):
     res = torch.randn(M, N, generator=g).to(DEV)
     kinds = ["fma"]
     if dt != torch.float32:
-        if M <= 8:
-            kinds.append("gemv")
         if M <= 16:
             kinds.append("gemv_mfma")
         kinds += ["mfma:0:1", "mfma:1:1", "mfma:2:1", "mfma:2:3", "mfma:0:2", "big:0", "big:1", None]
@@ -106,6 +104,7 @@ def test_linear_all_kernels_and_epilogues(ops, M, N, K, dt):
 
 
 TILED_CASES = [(1, 64, 64), (3, 172, 96), (16, 40, 4096), (9, 16400, 256), (17, 100, 64), (64, 256, 512),
+               (33, 4100, 2048), (48, 72, 8192), (50, 6144, 4096),
                (70, 200, 1024), (129, 384, 320), (256, 520, 2048), (384, 512, 192), (300, 1000, 96)]
 
 
@@ -132,8 +131,10 @@ def test_linear_tiled_weights(ops, M, N, K, dt):
                 out = ops.linear(x, wt, mode, out_dtype=torch.float32, force=kind)
             err = (out.double() - ref).abs().max().item()
             assert err < 2e-4 * (1 + ref.abs().max().item()), (kind, mode, err)
-    if M <= 16:
-        for nt, kw in ((1, 4), (1, 8), (1, 16), (2, 2), (2, 4), (2, 8), (4, 2), (4, 4)):
+    if M <= 64:
+        for nt, kw in ((1, 4), (1, 8), (2, 4), (2, 8)):
+            if (M > 32 and nt == 1) or (nt == 2 and kw == 8 and M > 32 and False):
+                continue
             out = ops.gemv_tiled(x, wt, out_dtype=torch.float32, nt=nt, kw=kw)
             assert (out.double() - _linear_ref(x, w, 0)).abs().max().item() < 2e-4 * 4
     if N % 32 == 0:
@@ -166,7 +167,7 @@ def test_linear_refuses_what_it_cannot_do(ops):
     x = torch.randn(4, 12).to(torch.bfloat16).to(DEV)
     w = torch.randn(6, 12).to(torch.bfloat16).to(DEV)
     with pytest.raises(ops.KernelError):
-        ops.linear(x, w, force="gemv")                                # K = 12 is no multiple of 8
+        ops.linear(x, w, force="gemv_mfma")                           # K = 12 is no multiple of 8
     with pytest.raises(ops.KernelError):
         ops.linear(x, w, force="mfma:0:1")
     out = ops.linear(x, w, out_dtype=torch.float32)                  # the general kernel takes it
