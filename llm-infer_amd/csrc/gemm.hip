@@ -294,7 +294,8 @@ __global__ __launch_bounds__(256) void gemm_mfma_kernel(const T* __restrict__ X,
 // ===========================================================================
 template <class T, int BN, int BM, int BK, bool TILED, bool EDGE>
 __global__ __launch_bounds__(256) void gemm_big_kernel(const T* __restrict__ X, const T* __restrict__ W,
-                                                       int K, Epilogue e) {
+                                                       int K, int k_per_split, float* __restrict__ ws,
+                                                       Epilogue e) {
     typedef typename Vec<T>::v8 v8;
     constexpr int LD = BK + 8, CPR = BK / 8;             // chunks of 8 elements per tile row
     constexpr int TN = BN / 2, TM = BM / 2;
@@ -310,6 +311,7 @@ __global__ __launch_bounds__(256) void gemm_big_kernel(const T* __restrict__ X, 
     // consecutive workgroups share the rows of W (blockIdx.x runs over the tiles of X first)
     const int m0 = blockIdx.x * BM, n0 = blockIdx.y * BN;
     const int n_limit = TILED ? ((e.N + 15) & ~15) : e.N;
+    const int kb = blockIdx.z * k_per_split, ke = min(K, kb + k_per_split);   // this workgroup's share of K
 
     f32x16 acc[NB][MB];
 #pragma unroll
@@ -352,12 +354,12 @@ __global__ __launch_bounds__(256) void gemm_big_kernel(const T* __restrict__ X, 
         const int64_t wstep = TILED ? (int64_t)(k0 >> 5) * 512 : k0;
 #pragma unroll
         for (int c = 0; c < W_CHUNKS; ++c) {
-            const bool in = !EDGE || k0 + wkc[c] < K;
+            const bool in = !EDGE || k0 + wkc[c] < ke;
             rw[c] = *(const v8*)(wsrc[c] + (in ? wstep : 0));
         }
 #pragma unroll
         for (int c = 0; c < X_CHUNKS; ++c) {
-            const bool in = !EDGE || k0 + xkc[c] < K;
+            const bool in = !EDGE || k0 + xkc[c] < ke;
             rx[c] = *(const v8*)(xsrc[c] + (in ? k0 : 0));
         }
     };
@@ -365,10 +367,10 @@ __global__ __launch_bounds__(256) void gemm_big_kernel(const T* __restrict__ X, 
         const v8 z = {};
 #pragma unroll
         for (int c = 0; c < W_CHUNKS; ++c)
-            *(v8*)(buf + wdst[c]) = (!EDGE || (wok[c] && k0 + wkc[c] < K)) ? rw[c] : z;
+            *(v8*)(buf + wdst[c]) = (!EDGE || (wok[c] && k0 + wkc[c] < ke)) ? rw[c] : z;
 #pragma unroll
         for (int c = 0; c < X_CHUNKS; ++c)
-            *(v8*)(buf + xdst[c]) = (!EDGE || (xok[c] && k0 + xkc[c] < K)) ? rx[c] : z;
+            *(v8*)(buf + xdst[c]) = (!EDGE || (xok[c] && k0 + xkc[c] < ke)) ? rx[c] : z;
     };
     auto compute = [&](const T* buf) {
         const T* sW = buf;
@@ -390,32 +392,32 @@ __global__ __launch_bounds__(256) void gemm_big_kernel(const T* __restrict__ X, 
 
     // Tile t is computed from LDS buffer t % 2 while tile t + 1 waits in registers and the loads
     // of tile t + 2 are issued: a load has more than one tile's worth of matrix work to arrive.
-    const int n_tiles = (K + BK - 1) / BK;
+    const int n_tiles = (ke - kb + BK - 1) / BK;
     v8 rw0[W_CHUNKS], rx0[X_CHUNKS], rw1[W_CHUNKS], rx1[X_CHUNKS];
     T* buf0 = smem;
     T* buf1 = smem + BUF;
     // (Loads and stores past the last tile are not branched around: they fetch the last tile again
     // and write it where nothing reads it, which keeps the count of loads in flight fixed.)
-    const int k_last = (n_tiles - 1) * BK;
-    load_tile(0, rw0, rx0);
-    store_tile(buf0, 0, rw0, rx0);
-    load_tile(min(BK, k_last), rw1, rx1);
+    const int k_last = kb + (n_tiles - 1) * BK;
+    load_tile(kb, rw0, rx0);
+    store_tile(buf0, kb, rw0, rx0);
+    load_tile(min(kb + BK, k_last), rw1, rx1);
     __syncthreads();
     int t = 0;
     for (; t + 1 < n_tiles; t += 2) {
         // the scheduling barriers keep the loads at the head of each half and the LDS writes at
         // its tail; left alone the compiler sinks the loads to just before their use
-        load_tile(min((t + 2) * BK, k_last), rw0, rx0);
+        load_tile(min(kb + (t + 2) * BK, k_last), rw0, rx0);
         __builtin_amdgcn_sched_barrier(0);
         compute(buf0);
         __builtin_amdgcn_sched_barrier(0);
-        store_tile(buf1, (t + 1) * BK, rw1, rx1);
+        store_tile(buf1, kb + (t + 1) * BK, rw1, rx1);
         __syncthreads();
-        load_tile(min((t + 3) * BK, k_last), rw1, rx1);
+        load_tile(min(kb + (t + 3) * BK, k_last), rw1, rx1);
         __builtin_amdgcn_sched_barrier(0);
         compute(buf1);
         __builtin_amdgcn_sched_barrier(0);
-        store_tile(buf0, min((t + 2) * BK, k_last), rw0, rx0);
+        store_tile(buf0, min(kb + (t + 2) * BK, k_last), rw0, rx0);
         __syncthreads();
     }
     if (t < n_tiles) compute(buf0);
@@ -441,7 +443,12 @@ __global__ __launch_bounds__(256) void gemm_big_kernel(const T* __restrict__ X, 
                 const int r = q >> 3, c = (q & 7) * 4;
                 const f32x4 v = *(const f32x4*)(stage + r * SLD + c);
                 const float vv[4] = {v[0], v[1], v[2], v[3]};
-                epilogue4(e, mb + r, nb + c, vv);
+                if (gridDim.z == 1) epilogue4(e, mb + r, nb + c, vv);
+                else if (mb + r < e.M) {                 // a share of K: the partial sums go to the workspace
+                    float* p = ws + ((int64_t)blockIdx.z * e.M + mb + r) * e.N + nb + c;
+#pragma unroll
+                    for (int j = 0; j < 4; ++j) if (nb + c + j < e.N) p[j] = vv[j];
+                }
             }
             __builtin_amdgcn_wave_barrier();
         }
@@ -826,27 +833,31 @@ extern "C" int li_gemv_tiled(const void* X, const void* Wt, int dt, void* C, int
 
 // tile (rows of W x rows of X / depth): 0 = 128x128/64, 1 = 256x128/32
 extern "C" int li_gemm_big(const void* X, const void* W, int tiled, int dt, void* C, int out_dt, int mode,
-                           int M, int N, int K, int tile, const RopeStore* rs, hipStream_t stream) {
+                           int M, int N, int K, int tile, int splits, float* ws, const RopeStore* rs,
+                           hipStream_t stream) {
     int rc = check_common(X, W, C, M, N, K, mode, out_dt);
     if (rc) return rc;
     if (dt != DT_F16 && dt != DT_BF16) return LI_BAD_ARG;
     if (K % 8 != 0 || ((uintptr_t)X & 15) || ((uintptr_t)W & 15)) return LI_UNSUPPORTED;
     if (tiled && K % 32 != 0) return LI_UNSUPPORTED;
     if (tile < 0 || tile > 1) return LI_BAD_ARG;
+    if (splits < 1 || (splits > 1 && !ws)) return LI_BAD_ARG;
     if (M == 0) return LI_OK;
     Epilogue e;
     rc = make_epilogue(e, C, mode, out_dt, M, N, rs);
     if (rc) return rc;
     const int bn = tile ? 256 : 128, bm = 128, bk = tile ? 32 : 64;
     const size_t lds = (size_t)2 * (bn + bm) * (bk + 8) * 2;
-    dim3 grid((M + bm - 1) / bm, (N + bn - 1) / bn), block(256);
+    int k_per_split = ((K + splits - 1) / splits + bk - 1) / bk * bk;
+    splits = (K + k_per_split - 1) / k_per_split;
+    dim3 grid((M + bm - 1) / bm, (N + bn - 1) / bn, splits), block(256);
     const bool edge = (M % bm) || (N % bn) || (K % bk);
 #define GO(T, BN, BM, BK, TL)                                                                          \
     do {                                                                                               \
         auto kfn = edge ? gemm_big_kernel<T, BN, BM, BK, TL, true> : gemm_big_kernel<T, BN, BM, BK, TL, false>; \
         if (hipFuncSetAttribute((const void*)kfn, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds) != hipSuccess) \
             return LI_HIP_ERROR;                                                                       \
-        kfn<<<grid, block, lds, stream>>>((const T*)X, (const T*)W, K, e);                             \
+        kfn<<<grid, block, lds, stream>>>((const T*)X, (const T*)W, K, k_per_split, ws, e);            \
     } while (0)
 #define LAUNCH(T)                                                                                     \
     do {                                                                                              \
@@ -857,5 +868,10 @@ extern "C" int li_gemm_big(const void* X, const void* W, int tiled, int dt, void
 #undef LAUNCH
 #undef GO
     LI_CHECK_LAUNCH();
+    if (splits > 1) {
+        const int64_t quads = (int64_t)M * ((N + 3) / 4);
+        splitk_reduce_kernel<<<(unsigned)((quads + 255) / 256), 256, 0, stream>>>(ws, splits, e);
+        LI_CHECK_LAUNCH();
+    }
     return LI_OK;
 }

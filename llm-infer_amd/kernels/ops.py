@@ -161,7 +161,7 @@ def linear(x: torch.Tensor, w, mode: int = EPI_STORE, out: torch.Tensor | None =
     lib = core()
     same16 = x.dtype == w.dtype and x.dtype in (torch.float16, torch.bfloat16)
     fast_ok = same16 and k % 8 == 0 and x.data_ptr() % 16 == 0 and wd.data_ptr() % 16 == 0
-    kind = force or ("fma" if not fast_ok else ("gemv_mfma" if m <= 16 else ("big" if m > 128 else "mfma")))
+    kind = force or ("fma" if not fast_ok else ("gemv_mfma" if m <= 16 else ("big" if m > 32 else "mfma")))
     if tiled:
         _need(fast_ok and kind != "fma", "a tiled weight needs 16-bit activations of its dtype")
         # up to 64 rows the weight is streamed once past all rows of X; beyond 32 rows that pays
@@ -179,9 +179,13 @@ def linear(x: torch.Tensor, w, mode: int = EPI_STORE, out: torch.Tensor | None =
                "gemv_mfma")
     elif kind.startswith("big"):
         _need(fast_ok, "gemm_big: 16-bit operands and K a multiple of 8")
-        tile = int(kind.split(":")[1]) if ":" in kind else _big_tile(m, n)
+        parts = kind.split(":")
+        tile = int(parts[1]) if len(parts) > 1 else _big_tile(m, n)
+        groups = -(-m // 128) * -(-n // (256 if tile else 128))
+        splits = int(parts[2]) if len(parts) > 2 else (1 if groups >= 192 else max(1, min(384 // groups, k // 512, 16)))
+        ws = _workspace(splits * m * n, x.device) if splits > 1 else None
         _check(lib.li_gemm_big(_ptr(x), _ptr(wd), int(tiled), DT[x.dtype], _ptr(out), out_dt, mode, m, n, k, tile,
-                               rs, _stream()), "gemm_big")
+                               splits, _ptr(ws), rs, _stream()), "gemm_big")
     else:
         _need(fast_ok, "gemm_mfma: 16-bit operands and K a multiple of 8")
         tile = 0 if m > 64 else (1 if m > 32 else 2)

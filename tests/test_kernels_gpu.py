@@ -79,7 +79,7 @@ def test_linear_all_kernels_and_epilogues(ops, M, N, K, dt):
     if dt != torch.float32:
         if M <= 16:
             kinds.append("gemv_mfma")
-        kinds += ["mfma:0:1", "mfma:1:1", "mfma:2:1", "mfma:2:3", "mfma:0:2", "big:0", "big:1", None]
+        kinds += ["mfma:0:1", "mfma:1:1", "mfma:2:1", "mfma:2:3", "mfma:0:2", "big:0", "big:1", "big:0:3", None]
     for kind in kinds:
         for mode in (0, 1, 2):
             if mode == 2 and N % 2:
@@ -118,7 +118,7 @@ def test_linear_tiled_weights(ops, M, N, K, dt):
     res = torch.randn(M, N, generator=g).to(DEV)
     wt = ops.tile_weight(w)
     assert wt.shape == (N, K) and wt.data.numel() == (N + 15) // 16 * 16 * K
-    kinds = [None, "mfma:0:1", "mfma:1:2", "mfma:2:1", "big:0", "big:1"] + (["gemv_mfma"] if M <= 16 else [])
+    kinds = [None, "mfma:0:1", "mfma:1:2", "mfma:2:1", "big:0", "big:1", "big:0:2", "big:1:5"] + (["gemv_mfma"] if M <= 16 else [])
     for kind in kinds:
         for mode in (0, 1, 2):
             if mode == 2 and N % 2:
