@@ -138,6 +138,28 @@ extern "C" int li_rope_store(const float* qkv, int row_stride, const float* inv_
     return LI_OK;
 }
 
+// cos and sin of pos[t] * inv_freq[j] for the tokens of a step: [T, n_freq, 2] float32.  The angles
+// are the same in every layer, so a step computes them once.
+__global__ void rope_table_kernel(const float* __restrict__ inv_freq, const int* __restrict__ pos,
+                                  float* __restrict__ out, int n_tokens, int n_freq) {
+    const int i = blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= n_tokens * n_freq) return;
+    const int t = i / n_freq, j = i - t * n_freq;
+    float s, c;
+    sincosf((float)pos[t] * inv_freq[j], &s, &c);
+    out[2 * i] = c;
+    out[2 * i + 1] = s;
+}
+
+extern "C" int li_rope_table(const float* inv_freq, const int* pos, float* out, int n_tokens, int n_freq,
+                             hipStream_t stream) {
+    if (n_tokens <= 0 || n_freq <= 0) return LI_OK;
+    const int n = n_tokens * n_freq;
+    rope_table_kernel<<<(n + 255) / 256, 256, 0, stream>>>(inv_freq, pos, out, n_tokens, n_freq);
+    LI_CHECK_LAUNCH();
+    return LI_OK;
+}
+
 // ---------------------------------------------------------------------------
 // Bookkeeping of one decode step, on the device so that a captured step can be
 // replayed: each sequence's new token gets the position lens[slot], the

@@ -20,6 +20,7 @@ enum { EPI_STORE = 0, EPI_ADD = 1, EPI_SWIGLU = 2, EPI_ROPE = 3 };
 // to q_out [M, H, hd], k and v into the token's cache page.
 struct RopeStore {
     const float* inv_freq;      // [rotary_dim / 2]
+    const float* cos_sin;       // [M, rotary_dim / 2, 2] cos and sin of pos * inv_freq, or null
     const int* pos;             // [M] position of each row
     const int* tok_slot;        // [M] cache slot of each row
     const int* page_table;      // [slots, max_pages]
@@ -63,7 +64,10 @@ __device__ __forceinline__ void epilogue4(const Epilogue& e, int m, int n, const
             for (int j = 0; j < 4; j += 2) {
                 if (d + j < r.rotary_dim) {
                     float sn, cs;
-                    sincosf((float)p * r.inv_freq[(d + j) >> 1], &sn, &cs);
+                    if (r.cos_sin) {
+                        const f32x2 t = *(const f32x2*)(r.cos_sin + ((int64_t)m * (r.rotary_dim >> 1) + ((d + j) >> 1)) * 2);
+                        cs = t[0]; sn = t[1];
+                    } else sincosf((float)p * r.inv_freq[(d + j) >> 1], &sn, &cs);
                     o[j] = v[j] * cs - v[j + 1] * sn;
                     o[j + 1] = v[j] * sn + v[j + 1] * cs;
                 }
@@ -665,7 +669,7 @@ static int make_epilogue(Epilogue& e, void* C, int mode, int out_dt, int M, int 
     if (!rs || !rs->pos || !rs->q_out || rs->hd <= 0 || rs->hd % 16 != 0 || rs->H <= 0 || rs->K < 0) return LI_BAD_ARG;
     if (N != (rs->H + 2 * rs->K) * rs->hd || rs->rotary_dim < 0 || rs->rotary_dim > rs->hd || (rs->rotary_dim & 1))
         return LI_BAD_ARG;
-    if (rs->rotary_dim > 0 && !rs->inv_freq) return LI_BAD_ARG;
+    if (rs->rotary_dim > 0 && !rs->inv_freq && !rs->cos_sin) return LI_BAD_ARG;
     if (rs->K > 0 && (!rs->tok_slot || !rs->page_table || !rs->k_pages || !rs->v_pages)) return LI_BAD_ARG;
     if (rs->dt < DT_F32 || rs->dt > DT_BF16) return LI_BAD_ARG;
     e.rs = *rs;

@@ -91,7 +91,7 @@ def rmsnorm(x: torch.Tensor, w: torch.Tensor, eps: float, out_dtype, rows: torch
 
 
 class _RopeStore(ctypes.Structure):
-    _fields_ = [("inv_freq", c_void_p), ("pos", c_void_p), ("tok_slot", c_void_p), ("page_table", c_void_p),
+    _fields_ = [("inv_freq", c_void_p), ("cos_sin", c_void_p), ("pos", c_void_p), ("tok_slot", c_void_p), ("page_table", c_void_p),
                 ("q_out", c_void_p), ("k_pages", c_void_p), ("v_pages", c_void_p), ("page_stride", c_int64),
                 ("rotary_dim", c_int), ("H", c_int), ("K", c_int), ("hd", c_int), ("max_pages", c_int),
                 ("dt", c_int)]
@@ -243,8 +243,19 @@ def rope_store(qkv, inv_freq, rotary_dim, half_pairing, pos, tok_slot, page_tabl
     return q
 
 
+def rope_table(inv_freq: torch.Tensor, pos: torch.Tensor, n_tokens: int) -> torch.Tensor:
+    """cos and sin of pos * inv_freq for the tokens of a step: float32 [T, n_freq, 2]."""
+    _dev(inv_freq, pos)
+    _need(inv_freq.dtype == torch.float32 and pos.dtype == torch.int32 and pos.numel() >= n_tokens,
+          "rope_table: float32 frequencies, int32 positions")
+    out = torch.empty((n_tokens, inv_freq.numel(), 2), dtype=torch.float32, device=inv_freq.device)
+    _check(core().li_rope_table(_ptr(inv_freq), _ptr(pos), _ptr(out), n_tokens, inv_freq.numel(), _stream()),
+           "rope_table")
+    return out
+
+
 def linear_rope_store(x, w, inv_freq, rotary_dim, pos, tok_slot, page_table, page_stride, k_pages, v_pages,
-                      n_heads, n_kv_heads, head_dim, out_dtype, force=None) -> torch.Tensor:
+                      n_heads, n_kv_heads, head_dim, out_dtype, force=None, cos_sin=None) -> torch.Tensor:
     """q, k, v = x W^T with the rotation (adjacent pairs) and the cache write done in the product's
     epilogue, on the float32 accumulators: the same result as linear (float32) followed by
     rope_store, without the round trip.  Returns q [T, H, hd]."""
@@ -261,7 +272,12 @@ def linear_rope_store(x, w, inv_freq, rotary_dim, pos, tok_slot, page_table, pag
         _need(page_table.dtype == torch.int32 and page_table.dim() == 2, "page_table: int32 [slots, pages]")
         _need(k_pages.dtype == out_dtype and v_pages.dtype == out_dtype, "cache dtype differs from q dtype")
     q = torch.empty((t, n_heads, head_dim), dtype=out_dtype, device=x.device)
-    rs = _RopeStore(inv_freq.data_ptr() if inv_freq is not None else None, pos.data_ptr(),
+    if cos_sin is not None:
+        _dev(cos_sin)
+        _need(cos_sin.dtype == torch.float32 and cos_sin.numel() >= t * (rotary_dim // 2) * 2 and
+              cos_sin.shape[1] == rotary_dim // 2, "cos_sin: float32 [T, rotary_dim / 2, 2]")
+    rs = _RopeStore(inv_freq.data_ptr() if inv_freq is not None else None,
+                    cos_sin.data_ptr() if cos_sin is not None else None, pos.data_ptr(),
                     tok_slot.data_ptr() if tok_slot is not None else None,
                     page_table.data_ptr() if page_table is not None else None, q.data_ptr(),
                     k_pages.data_ptr() if k_pages is not None else None,

@@ -19,7 +19,7 @@ class RotaryPosition:
     """
 
     def __init__(self, *, theta: float, rotary_dim: int, head_dim: int, pairing: str = "adjacent", dtype, device):
-        self.rotary_dim, self.head_dim, self.pairing = rotary_dim, head_dim, pairing
+        self.rotary_dim, self.head_dim, self.pairing, self.theta = rotary_dim, head_dim, pairing, float(theta)
         i = torch.arange(0, rotary_dim, 2, dtype=torch.float32)
         # 1 / powf(theta, i / rotary_dim) in float32, as kernels_cpu.hpp:87
         inv = 1.0 / torch.pow(torch.tensor(float(theta), dtype=torch.float32), i / float(rotary_dim))
@@ -37,16 +37,29 @@ class RotaryPosition:
         """q, k, v = h W^T, rotated and stored; with adjacent pairing and 16-bit storage the rotation
         and the cache write happen in the product's epilogue."""
         return _project(self, h, w, ctx, kv_view, n_heads, n_kv_heads, head_dim, self.inv_freq, self.rotary_dim,
-                        self.pairing == "adjacent")
+                        self.pairing == "adjacent", self._table(ctx))
+
+    def _table(self, ctx):
+        """cos and sin of every token's angles, computed once per step and shared by all layers that
+        rotate with the same frequencies."""
+        if self.rotary_dim == 0 or self.pairing != "adjacent" or self.dtype == torch.float32:
+            return None
+        cache = getattr(ctx, "_rope_tables", None)
+        if cache is None:
+            cache = ctx._rope_tables = {}
+        key = (self.theta, self.rotary_dim)
+        if key not in cache:
+            cache[key] = ops.rope_table(self.inv_freq, ctx.pos, ctx.n_tokens)
+        return cache[key]
 
 
-def _project(part, h, w, ctx, kv_view, n_heads, n_kv_heads, head_dim, inv_freq, rotary_dim, fusable):
+def _project(part, h, w, ctx, kv_view, n_heads, n_kv_heads, head_dim, inv_freq, rotary_dim, fusable, table=None):
     if fusable and part.dtype != torch.float32 and h.dtype == part.dtype:
-        k = v = table = stride = None
+        k = v = ptab = stride = None
         if n_kv_heads > 0:
-            k, v, table, stride = kv_view.k, kv_view.v, kv_view.page_table, kv_view.page_stride
-        return ops.linear_rope_store(h, w, inv_freq, rotary_dim, ctx.pos, ctx.tok_slot, table, stride, k, v,
-                                     n_heads, n_kv_heads, head_dim, part.dtype)
+            k, v, ptab, stride = kv_view.k, kv_view.v, kv_view.page_table, kv_view.page_stride
+        return ops.linear_rope_store(h, w, inv_freq, rotary_dim, ctx.pos, ctx.tok_slot, ptab, stride, k, v,
+                                     n_heads, n_kv_heads, head_dim, part.dtype, cos_sin=table)
     qkv = ops.linear(h, w, out_dtype=torch.float32)
     return part.rotate_store(qkv, ctx, kv_view, n_heads, n_kv_heads, head_dim)
 
