@@ -20,17 +20,10 @@ __host__ __device__ __forceinline__ float uniform01(uint64_t key, uint64_t count
 
 extern "C" float li_uniform01(uint64_t key, uint64_t counter) { return uniform01(key, counter); }
 
-__global__ __launch_bounds__(1024) void argmax_kernel(const float* __restrict__ logits, int V,
-                                                      int* __restrict__ out) {
-    __shared__ float sv[16];
-    __shared__ int si[16];
-    const float* row = logits + (int64_t)blockIdx.x * V;
-    float best = -INFINITY;
-    int best_i = 0x7fffffff;
-    for (int i = threadIdx.x; i < V; i += blockDim.x) {
-        const float v = row[i];
-        if (v > best || best_i == 0x7fffffff) { best = v; best_i = i; }      // ascending i: strict > keeps the first
-    }
+// Greedy choice in two stages so that a few rows still use the whole chip: every workgroup finds the
+// first maximum of one chunk of a row, then one workgroup per row picks among the chunks.  Ties go
+// to the lowest index at every stage.
+__device__ __forceinline__ void first_max_reduce(float& best, int& best_i, float* sv, int* si) {
 #pragma unroll
     for (int o = 32; o > 0; o >>= 1) {
         const float ov = __shfl_xor(best, o, WAVE);
@@ -40,11 +33,44 @@ __global__ __launch_bounds__(1024) void argmax_kernel(const float* __restrict__ 
     const int w = threadIdx.x >> 6, nw = (blockDim.x + 63) >> 6;
     if ((threadIdx.x & 63) == 0) { sv[w] = best; si[w] = best_i; }
     __syncthreads();
-    if (threadIdx.x == 0) {
+    if (threadIdx.x == 0)
         for (int i = 1; i < nw; ++i)
             if (sv[i] > best || (sv[i] == best && si[i] < best_i)) { best = sv[i]; best_i = si[i]; }
-        out[blockIdx.x] = best_i == 0x7fffffff ? 0 : best_i;
+}
+
+__global__ __launch_bounds__(256) void argmax_chunks_kernel(const float* __restrict__ logits, int V, int chunk,
+                                                            float* __restrict__ part_v, int* __restrict__ part_i) {
+    __shared__ float sv[4];
+    __shared__ int si[4];
+    const float* row = logits + (int64_t)blockIdx.x * V;
+    const int lo = blockIdx.y * chunk, hi = min(V, lo + chunk);
+    float best = -INFINITY;
+    int best_i = 0x7fffffff;
+    for (int i = lo + threadIdx.x; i < hi; i += blockDim.x) {
+        const float v = row[i];
+        if (v > best || best_i == 0x7fffffff) { best = v; best_i = i; }      // ascending i: strict > keeps the first
     }
+    first_max_reduce(best, best_i, sv, si);
+    if (threadIdx.x == 0) {
+        part_v[blockIdx.x * gridDim.y + blockIdx.y] = best;
+        part_i[blockIdx.x * gridDim.y + blockIdx.y] = best_i;
+    }
+}
+
+__global__ __launch_bounds__(64) void argmax_final_kernel(const float* __restrict__ part_v,
+                                                          const int* __restrict__ part_i, int n_chunks,
+                                                          int* __restrict__ out) {
+    __shared__ float sv[1];
+    __shared__ int si[1];
+    float best = -INFINITY;
+    int best_i = 0x7fffffff;
+    for (int c = threadIdx.x; c < n_chunks; c += blockDim.x) {
+        const float v = part_v[blockIdx.x * n_chunks + c];
+        const int i = part_i[blockIdx.x * n_chunks + c];
+        if (i != 0x7fffffff && (v > best || best_i == 0x7fffffff || (v == best && i < best_i))) { best = v; best_i = i; }
+    }
+    first_max_reduce(best, best_i, sv, si);
+    if (threadIdx.x == 0) out[blockIdx.x] = best_i == 0x7fffffff ? 0 : best_i;
 }
 
 // state: [n_slots, 2] uint64 (key, counter); the counter advances by one per sampled token.
@@ -98,10 +124,18 @@ __global__ __launch_bounds__(1024) void sample_kernel(const float* __restrict__ 
     }
 }
 
-extern "C" int li_argmax(const float* logits, int n_rows, int V, int* out, hipStream_t stream) {
+// part_v, part_i: workspace of n_rows * li_argmax_chunks(V) entries each
+extern "C" int li_argmax_chunks(int V) { return V <= 4096 ? 1 : (V + 4095) / 4096; }
+
+extern "C" int li_argmax(const float* logits, int n_rows, int V, float* part_v, int* part_i, int* out,
+                         hipStream_t stream) {
     if (n_rows <= 0) return LI_OK;
-    if (V <= 0) return LI_BAD_ARG;
-    argmax_kernel<<<n_rows, V >= 4096 ? 1024 : 256, 0, stream>>>(logits, V, out);
+    if (V <= 0 || !part_v || !part_i) return LI_BAD_ARG;
+    const int n_chunks = li_argmax_chunks(V);
+    const int chunk = (V + n_chunks - 1) / n_chunks;
+    argmax_chunks_kernel<<<dim3(n_rows, n_chunks), 256, 0, stream>>>(logits, V, chunk, part_v, part_i);
+    LI_CHECK_LAUNCH();
+    argmax_final_kernel<<<n_rows, 64, 0, stream>>>(part_v, part_i, n_chunks, out);
     LI_CHECK_LAUNCH();
     return LI_OK;
 }
@@ -109,8 +143,7 @@ extern "C" int li_argmax(const float* logits, int n_rows, int V, int* out, hipSt
 extern "C" int li_sample(const float* logits, int n_rows, int V, float temperature, const int* seq_slot,
                          void* state, const float* forced_r, int* out, hipStream_t stream) {
     if (n_rows <= 0) return LI_OK;
-    if (V <= 0) return LI_BAD_ARG;
-    if (temperature <= 0.f) return li_argmax(logits, n_rows, V, out, stream);
+    if (V <= 0 || temperature <= 0.f) return LI_BAD_ARG;             // greedy goes through li_argmax
     if (!forced_r && (!seq_slot || !state)) return LI_BAD_ARG;
     sample_kernel<<<n_rows, V >= 4096 ? 1024 : 256, 0, stream>>>(logits, V, temperature, seq_slot,
                                                                   (unsigned long long*)state, forced_r, out);

@@ -377,7 +377,11 @@ def argmax(logits: torch.Tensor, out: torch.Tensor | None = None) -> torch.Tenso
     if out is None:
         out = torch.empty((logits.shape[0],), dtype=torch.int32, device=logits.device)
     _need(out.dtype == torch.int32 and out.numel() >= logits.shape[0], "out: int32 [B]")
-    _check(core().li_argmax(_ptr(logits), logits.shape[0], logits.shape[1], _ptr(out), _stream()), "argmax")
+    n = logits.shape[0] * core().li_argmax_chunks(logits.shape[1])
+    part_v = torch.empty((n,), dtype=torch.float32, device=logits.device)
+    part_i = torch.empty((n,), dtype=torch.int32, device=logits.device)
+    _check(core().li_argmax(_ptr(logits), logits.shape[0], logits.shape[1], _ptr(part_v), _ptr(part_i), _ptr(out),
+                            _stream()), "argmax")
     return out
 
 
@@ -387,6 +391,8 @@ def sample(logits, temperature: float, seq_slot=None, state=None, forced_r=None,
     _dev(logits, seq_slot, state, forced_r, out)
     _need(logits.dtype == torch.float32 and logits.dim() == 2, "logits: float32 [B, V]")
     b = logits.shape[0]
+    if temperature <= 0:
+        return argmax(logits, out)
     if out is None:
         out = torch.empty((b,), dtype=torch.int32, device=logits.device)
     if temperature > 0 and forced_r is None:

@@ -438,3 +438,83 @@ def test_toy_architecture_with_a_stateful_mixer(lib):
         eng.free_slot(s)
     toks = eng.generate([seqs[1]], max_new_tokens=4, temperature=0.0, use_graph=False)[0]
     assert toks[0] == int(refs[1][-1].argmax())
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_toy_architecture_with_a_window_group(lib, dtype):
+    """Two attention layers with different needs, all keys and a window of 70: two cache groups with
+    pools and page tables of their own; the window group gives pages back while a sequence grows."""
+    from llm_infer_amd.config.spec import LayerSpec, ModelSpec, PartSpec, ScheduleEntry
+    from llm_infer_amd.engine import Engine
+
+    class WindowConfig:
+        def __init__(self, raw):
+            self.raw = raw
+
+        @classmethod
+        def from_dict(cls, raw):
+            return cls(raw)
+
+        def model_spec(self):
+            d, hd = 64, 32
+            norm = PartSpec("rmsnorm", {"size": d, "eps": 1e-5})
+            ffn = PartSpec("gated_mlp", {"hidden_size": d, "intermediate_size": 96})
+            rope = PartSpec("rope", {"theta": 1000.0, "rotary_dim": hd, "head_dim": hd})
+            layers = []
+            for i, window in enumerate((None, 70)):
+                att = PartSpec("attention", {"hidden_size": d, "n_heads": 2, "n_kv_heads": 2, "head_dim": hd,
+                                             "scale": hd ** -0.5, "window": window}, f"l{i}.mix.")
+                layers.append(LayerSpec("pre_norm", att, ffn.with_prefix(f"l{i}.ffn."), norm.with_prefix(f"l{i}.n1."),
+                                        norm.with_prefix(f"l{i}.n2."), rope))
+            return ModelSpec(d, 40, 512, PartSpec("embedding", {"vocab_size": 40, "hidden_size": d}, "emb."),
+                             tuple(layers), (ScheduleEntry(0), ScheduleEntry(1)), norm.with_prefix("final."),
+                             PartSpec("lm_head", {"vocab_size": 40, "hidden_size": d, "tied": True}, "head."))
+
+    lib.register_architecture("WindowToyForCausalLM", WindowConfig)
+    cfg = lib.config_from_dict({"architectures": ["WindowToyForCausalLM"]})
+    eng = Engine.from_random(cfg, seed=2, dtype=dtype, max_tokens=1024, stored_dtype="bfloat16")
+    model, cache = eng.model, eng.cache
+    groups = {g.spec.window: g for g in cache.groups}
+    assert set(groups) == {None, 70}
+
+    emb = model.embedding.weight.double().cpu()
+    fin = model.final_norm.weight.double().cpu()
+
+    def rows(w):                                     # a weight back in plain row order, whatever its layout
+        from llm_infer_amd.kernels import ops
+        if isinstance(w, ops.TiledWeight):
+            eye = torch.eye(w.k, dtype=w.dtype, device=DEV)
+            return ops.linear(eye, w, out_dtype=torch.float32).t().double().cpu()
+        return w.double().cpu()
+
+    def ref_forward(toks):
+        n = len(toks)
+        x = emb[toks]
+        posn = torch.arange(n)
+        for layer, window in zip(model.layers, (None, 70)):
+            att, ffn = layer.mixer, layer.feed_forward
+            wq, wk, wv = rows(att.wqkv).split([64, 64, 64])
+            h = P.rmsnorm(x, layer.mixer_norm.weight.double().cpu(), 1e-5)
+            q = P.rope((h @ wq.t()).view(n, 2, 32), posn, 1000.0, 32)
+            k = P.rope((h @ wk.t()).view(n, 2, 32), posn, 1000.0, 32)
+            v = (h @ wv.t()).view(n, 2, 32)
+            x = x + P.attention(q, k, v, window).reshape(n, 64) @ rows(att.wo).t()
+            gu = rows(ffn.w_gate_up)
+            x = x + P.swiglu(P.rmsnorm(x, layer.feed_forward_norm.weight.double().cpu(), 1e-5), gu[0::2], gu[1::2],
+                             rows(ffn.w_down))
+        return P.rmsnorm(x, fin, 1e-5) @ emb.t()
+
+    toks = torch.randint(0, 40, (300,), generator=torch.Generator().manual_seed(1)).tolist()
+    ref = ref_forward(toks)
+    tol = 1e-5 if dtype == "float32" else 4e-2 * ref.std().item()
+    s = eng.alloc_slot()
+    got = [eng.step([s], [toks[:150]], [list(range(150))])]
+    assert sorted(groups[70].pages_of[s]) == [1, 2] and sorted(groups[None].pages_of[s]) == [0, 1, 2]
+    for p in range(150, 300):
+        got.append(eng.step([s], [[toks[p]]]))
+    assert sorted(groups[70].pages_of[s]) == [3, 4] and sorted(groups[None].pages_of[s]) == [0, 1, 2, 3, 4]
+    got = torch.cat(got).double().cpu()
+    err = (got - ref).abs().max(dim=1).values
+    assert err.max().item() < tol, f"first wrong place: {int((err >= tol).nonzero()[0])}"
+    eng.free_slot(s)
+    assert groups[70].pool.n_free == groups[None].pool.n_free == cache.n_pages - 1
