@@ -235,6 +235,32 @@ def test_reused_slots_and_batch_composition(lib, folders, dtype):
         eng.step(slots, [reqs[0] + reqs[0], reqs[0] + reqs[0], reqs[0] + reqs[0]])
 
 
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_prompt_in_several_chunks(lib, folders, dtype):
+    """A prompt fed in chunks of several tokens (each chunk attends to the cache of the chunks before
+    it and causally to itself), next to a sequence that is decoding: same logits as the whole prompt."""
+    cfg, folder = TINY_A, folders["A"]
+    weights = P.load_weights(folder)
+    eng = lib.load(folder, dtype=dtype, max_tokens=1024)
+    g = torch.Generator().manual_seed(4)
+    a = torch.randint(0, 256, (120,), generator=g).tolist()
+    b = torch.randint(0, 256, (90,), generator=g).tolist()
+    ref_a, ref_b = (P.forward(weights, cfg, t, torch.float64) for t in (a, b))
+    own = (P.forward(weights, cfg, a, torch.float32) if dtype == "float32"
+           else P.forward(weights, cfg, a, torch.float64, torch.bfloat16))
+    tol = 3 * (own.double() - ref_a).abs().max().item() + 1e-6
+    sa, sb = eng.alloc_slot(), eng.alloc_slot()
+    eng.step([sb], [b[:60]])
+    cuts = [0, 5, 64, 65, 100, 120]
+    got = []
+    for i, (lo, hi) in enumerate(zip(cuts, cuts[1:])):
+        out = eng.step([sa, sb], [a[lo:hi], [b[60 + i]]], [list(range(hi - lo)), [0]])
+        got.append(out[:hi - lo])
+        assert (out[hi - lo].double().cpu() - ref_b[60 + i]).abs().max().item() < tol
+    got = torch.cat(got).double().cpu()
+    assert (got - ref_a).abs().max().item() < tol
+
+
 def test_requests_are_checked(lib, folders):
     eng = lib.load(folders["A"], dtype="bfloat16", max_tokens=256)
     s = eng.alloc_slot()
