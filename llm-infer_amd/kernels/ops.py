@@ -122,13 +122,19 @@ def prepare_weight(w: torch.Tensor):
 
 
 _ws_cache: dict = {}
+_ws_retired: list = []
 
 
 def _workspace(n_floats: int, device) -> torch.Tensor:
+    """Scratch for split-K partial sums, one per device and stream.  A workspace that has become
+    too small is kept alive beside its larger successor: a captured graph may still write to it."""
     key = (device, torch.cuda.current_stream().cuda_stream)
     ws = _ws_cache.get(key)
     if ws is None or ws.numel() < n_floats:
-        ws = torch.empty(max(n_floats, 1 << 22), dtype=torch.float32, device=device)
+        if ws is not None:
+            _ws_retired.append(ws)
+        ws = torch.empty(max(n_floats, 1 << 22, 2 * (ws.numel() if ws is not None else 0)),
+                         dtype=torch.float32, device=device)
         _ws_cache[key] = ws
     return ws
 
@@ -164,12 +170,22 @@ def linear(x: torch.Tensor, w, mode: int = EPI_STORE, out: torch.Tensor | None =
     kind = force or ("fma" if not fast_ok else ("gemv_mfma" if m <= 16 else ("big" if m > 32 else "mfma")))
     if tiled:
         _need(fast_ok and kind != "fma", "a tiled weight needs 16-bit activations of its dtype")
-        # up to 64 rows the weight is streamed once past all rows of X; beyond 32 rows that pays
-        # only for matrices small enough that the tiled GEMM cannot fill the chip
-        if kind == "gemv_mfma" or (force is None and (m <= 32 or (m <= 64 and n * k <= (1 << 25)))):
+        # up to 16 rows (32 for a small matrix) every wave fetches the rows of X itself; up to 96
+        # rows they go through LDS once per workgroup; beyond that the tiled GEMM is faster
+        if kind == "gemv_mfma" or (force is None and (m <= 16 or (m <= 32 and n * k <= (1 << 25)))):
             _check(lib.li_gemv_tiled(_ptr(x), _ptr(wd), DT[x.dtype], _ptr(out), out_dt, mode, m, n, k, 0, 0,
                                      rs, _stream()), "gemv_tiled")
             return out
+        if force is None and m <= 96:
+            kind = "stream"
+    if kind.startswith("stream"):
+        _need(tiled and fast_ok and m <= 128, "gemm_stream: a tiled weight and at most 128 rows")
+        parts = kind.split(":")
+        nt, splits = (int(parts[1]), int(parts[2])) if len(parts) > 2 else _stream_shape(n, k)
+        ws = _workspace(splits * m * n, x.device) if splits > 1 else None
+        _check(lib.li_gemm_stream(_ptr(x), _ptr(wd), DT[x.dtype], _ptr(out), out_dt, mode, m, n, k, nt, splits,
+                                  _ptr(ws), rs, _stream()), "gemm_stream")
+        return out
     if kind == "fma":
         _check(lib.li_gemm_fma(_ptr(x), DT[x.dtype], _ptr(w), DT[w.dtype], _ptr(out), out_dt, mode,
                                m, n, k, rs, _stream()), "gemm_fma")
@@ -201,6 +217,22 @@ def linear(x: torch.Tensor, w, mode: int = EPI_STORE, out: torch.Tensor | None =
         _check(lib.li_gemm_mfma(_ptr(x), _ptr(wd), int(tiled), DT[x.dtype], _ptr(out), out_dt, mode, m, n, k,
                                 tile, splits, _ptr(ws), rs, _stream()), "gemm_mfma")
     return out
+
+
+def _stream_shape(n: int, k: int) -> tuple[int, int]:
+    """Tiles of W per wave and splits of K for gemm_stream (measured on MI355X): two tiles per
+    wave halve the traffic of X if that still leaves a workgroup for most of the 256 CUs; K is
+    split down to 1024 elements per workgroup to get there."""
+    def splits_for(groups):
+        want = max(1, 256 // groups)
+        want = 1 << (want.bit_length() - 1)
+        return max(1, min(want, k // 1024, 16))
+    g2 = -(-n // 128)
+    s2 = splits_for(g2)
+    if g2 * s2 >= 192:
+        return 2, s2
+    g1 = -(-n // 64)
+    return 1, splits_for(g1)
 
 
 def _big_tile(m: int, n: int) -> int:

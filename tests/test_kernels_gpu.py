@@ -105,7 +105,7 @@ def test_linear_all_kernels_and_epilogues(ops, M, N, K, dt):
 
 TILED_CASES = [(1, 64, 64), (3, 172, 96), (16, 40, 4096), (9, 16400, 256), (17, 100, 64), (64, 256, 512),
                (33, 4100, 2048), (48, 72, 8192), (50, 6144, 4096),
-               (70, 200, 1024), (129, 384, 320), (256, 520, 2048), (384, 512, 192), (300, 1000, 96)]
+               (70, 200, 1024), (96, 1000, 416), (128, 136, 2048), (129, 384, 320), (256, 520, 2048), (384, 512, 192), (300, 1000, 96)]
 
 
 @pytest.mark.parametrize("M,N,K", TILED_CASES)
@@ -119,6 +119,8 @@ def test_linear_tiled_weights(ops, M, N, K, dt):
     wt = ops.tile_weight(w)
     assert wt.shape == (N, K) and wt.data.numel() == (N + 15) // 16 * 16 * K
     kinds = [None, "mfma:0:1", "mfma:1:2", "mfma:2:1", "big:0", "big:1", "big:0:2", "big:1:5"] + (["gemv_mfma"] if M <= 16 else [])
+    if M <= 128:
+        kinds += ["stream", "stream:1:1", "stream:2:1", "stream:1:3", "stream:2:16"]
     for kind in kinds:
         for mode in (0, 1, 2):
             if mode == 2 and N % 2:
@@ -369,7 +371,7 @@ def test_rotation_fused_into_the_projection(ops, dt, T, H, K, hd, rot, d):
         if tiled and d % 32:
             continue
         ww = ops.tile_weight(w) if tiled else w
-        for kind in kinds:
+        for kind in kinds + (["stream:1:1", "stream:2:2"] if tiled and T <= 128 else []):
             if tiled and kind == "fma":
                 continue
             c1, v1 = fresh()
