@@ -48,15 +48,71 @@ __global__ void rmsnorm_kernel(const float* __restrict__ x, const float* __restr
     for (int i = threadIdx.x; i < d; i += blockDim.x) o[i] = from_f32<TO>(xr[i] / rms * w[i]);
 }
 
+// The same for rows of up to 4 * V * blockDim.x elements (d a multiple of 4, 16-byte aligned
+// pointers): the row and its weights are read once, in 16-byte pieces that stay in registers.
+template <class TO, int V>
+__global__ void rmsnorm_vec_kernel(const float* __restrict__ x, const float* __restrict__ w,
+                                   const int* __restrict__ rows, TO* __restrict__ out, int d, float eps) {
+    struct alignas(4 * sizeof(TO)) Out4 { TO v[4]; };
+    __shared__ float scratch[16];
+    const int r = blockIdx.x, n4 = d >> 2;
+    const f32x4* xr = (const f32x4*)(x + (int64_t)(rows ? rows[r] : r) * d);
+    const f32x4* w4 = (const f32x4*)w;
+    Out4* o = (Out4*)(out + (int64_t)r * d);
+    f32x4 xv[V], wv[V];
+#pragma unroll
+    for (int j = 0; j < V; ++j) {
+        const int i = threadIdx.x + j * blockDim.x;
+        xv[j] = i < n4 ? xr[i] : f32x4{0.f, 0.f, 0.f, 0.f};
+    }
+#pragma unroll
+    for (int j = 0; j < V; ++j) {
+        const int i = threadIdx.x + j * blockDim.x;
+        wv[j] = i < n4 ? w4[i] : f32x4{0.f, 0.f, 0.f, 0.f};
+    }
+    float ss = 0.f;
+#pragma unroll
+    for (int j = 0; j < V; ++j)
+#pragma unroll
+        for (int q = 0; q < 4; ++q) ss += xv[j][q] * xv[j][q];
+    ss = block_sum(ss, scratch);
+    const float rms = sqrtf(ss / (float)d + eps);
+#pragma unroll
+    for (int j = 0; j < V; ++j) {
+        const int i = threadIdx.x + j * blockDim.x;
+        if (i < n4) {
+            Out4 t;
+#pragma unroll
+            for (int q = 0; q < 4; ++q) t.v[q] = from_f32<TO>(xv[j][q] / rms * wv[j][q]);
+            o[i] = t;
+        }
+    }
+}
+
 extern "C" int li_rmsnorm(const float* x, const float* w, const int* rows, void* out, int out_dt,
                           int n_rows, int d, float eps, hipStream_t stream) {
     if (n_rows <= 0) return LI_OK;
     if (d <= 0) return LI_BAD_ARG;
-    dim3 grid(n_rows), block(d >= 2048 ? 512 : (d >= 512 ? 256 : 64));
-    if (out_dt == DT_F32) rmsnorm_kernel<float><<<grid, block, 0, stream>>>(x, w, rows, (float*)out, d, eps);
-    else if (out_dt == DT_F16) rmsnorm_kernel<f16><<<grid, block, 0, stream>>>(x, w, rows, (f16*)out, d, eps);
-    else if (out_dt == DT_BF16) rmsnorm_kernel<bf16><<<grid, block, 0, stream>>>(x, w, rows, (bf16*)out, d, eps);
-    else return LI_BAD_ARG;
+    if (out_dt != DT_F32 && out_dt != DT_F16 && out_dt != DT_BF16) return LI_BAD_ARG;
+    dim3 grid(n_rows);
+    const bool vec = d % 4 == 0 && d <= 8192 && !(((uintptr_t)x | (uintptr_t)w | (uintptr_t)out) & 15);
+    if (vec) {
+        const int n4 = d / 4;
+        const int threads = n4 <= 64 ? 64 : (n4 <= 256 ? 128 : (n4 <= 1024 ? 256 : 512));
+        const bool two = n4 <= 2 * threads;
+#define GO(TO)                                                                                             \
+    do {                                                                                                   \
+        if (two) rmsnorm_vec_kernel<TO, 2><<<grid, threads, 0, stream>>>(x, w, rows, (TO*)out, d, eps);    \
+        else rmsnorm_vec_kernel<TO, 4><<<grid, threads, 0, stream>>>(x, w, rows, (TO*)out, d, eps);        \
+    } while (0)
+        if (out_dt == DT_F32) GO(float); else if (out_dt == DT_F16) GO(f16); else GO(bf16);
+#undef GO
+    } else {
+        dim3 block(d >= 2048 ? 512 : (d >= 512 ? 256 : 64));
+        if (out_dt == DT_F32) rmsnorm_kernel<float><<<grid, block, 0, stream>>>(x, w, rows, (float*)out, d, eps);
+        else if (out_dt == DT_F16) rmsnorm_kernel<f16><<<grid, block, 0, stream>>>(x, w, rows, (f16*)out, d, eps);
+        else rmsnorm_kernel<bf16><<<grid, block, 0, stream>>>(x, w, rows, (bf16*)out, d, eps);
+    }
     LI_CHECK_LAUNCH();
     return LI_OK;
 }

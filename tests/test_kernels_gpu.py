@@ -32,7 +32,7 @@ def test_embed(ops):
         assert torch.equal(out, table[toks.long()].float())
 
 
-@pytest.mark.parametrize("d", [64, 96, 100, 1000, 4096])
+@pytest.mark.parametrize("d", [30, 64, 96, 100, 1000, 1022, 4096, 8192, 10000])
 def test_rmsnorm(ops, d):
     g = torch.Generator().manual_seed(d)
     x = (torch.randn(7, d, generator=g) * 3).to(DEV)
