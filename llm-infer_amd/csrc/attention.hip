@@ -77,7 +77,7 @@ struct WaveAttn {
     // Scores of the page's keys (starting at key t0) against this wave's rows, mask, running
     // maximum and sum; leaves the probabilities in s.  This lane's row sees keys lo..hi.
     __device__ __forceinline__ void scores(const v8 (&kf)[2 * KS], f32x16 (&s)[2], int t0, int lo, int hi,
-                                           float scale2) {
+                                           float scale2, bool masked = true) {
 #pragma unroll
         for (int b = 0; b < 2; ++b) {
 #pragma unroll
@@ -85,12 +85,12 @@ struct WaveAttn {
 #pragma unroll
             for (int ks = 0; ks < KS; ++ks) s[b] = mfma32(kf[b * KS + ks], q[ks], s[b]);
         }
-        softmax_step(s, t0, lo, hi, scale2);
+        softmax_step(s, t0, lo, hi, scale2, masked);
     }
 
     // The same with the key fragments fetched where they are used.
     __device__ __forceinline__ void scores_streamed(const T* kpage, f32x16 (&s)[2], int t0, int lo, int hi,
-                                                    float scale2) {
+                                                    float scale2, bool masked = true) {
         const int lane = threadIdx.x & 63;
 #pragma unroll
         for (int b = 0; b < 2; ++b) {
@@ -102,22 +102,32 @@ struct WaveAttn {
                 s[b] = mfma32(kf, q[ks], s[b]);
             }
         }
-        softmax_step(s, t0, lo, hi, scale2);
+        softmax_step(s, t0, lo, hi, scale2, masked);
     }
 
-    __device__ __forceinline__ void softmax_step(f32x16 (&s)[2], int t0, int lo, int hi, float scale2) {
+    // scale2 > 0.  A page whose keys all lie inside lo..hi for every lane of the wave (the
+    // caller knows: `masked` false) skips the comparisons.
+    __device__ __forceinline__ void softmax_step(f32x16 (&s)[2], int t0, int lo, int hi, float scale2,
+                                                 bool masked = true) {
         const int lane = threadIdx.x & 63;
         float mx = -INFINITY;
+        if (masked) {
 #pragma unroll
-        for (int b = 0; b < 2; ++b)
+            for (int b = 0; b < 2; ++b)
 #pragma unroll
-            for (int r = 0; r < 16; ++r) {
-                const int t = t0 + 32 * b + 8 * (r >> 2) + 4 * (lane >> 5) + (r & 3);
-                const float v = (t >= lo && t <= hi) ? s[b][r] * scale2 : -INFINITY;
-                s[b][r] = v;
-                mx = fmaxf(mx, v);
-            }
-        mx = fmaxf(mx, __shfl_xor(mx, 32, WAVE));
+                for (int r = 0; r < 16; ++r) {
+                    const int t = t0 + 32 * b + 8 * (r >> 2) + 4 * (lane >> 5) + (r & 3);
+                    const float v = (t >= lo && t <= hi) ? s[b][r] : -INFINITY;
+                    s[b][r] = v;
+                    mx = fmaxf(mx, v);
+                }
+        } else {
+#pragma unroll
+            for (int b = 0; b < 2; ++b)
+#pragma unroll
+                for (int r = 0; r < 16; ++r) mx = fmaxf(mx, s[b][r]);
+        }
+        mx = fmaxf(mx, __shfl_xor(mx, 32, WAVE)) * scale2;
         const float m_new = fmaxf(m, mx);
         const float m_safe = (m_new == -INFINITY) ? 0.f : m_new;
         const float alpha = exp2f(m - m_safe);
@@ -126,7 +136,7 @@ struct WaveAttn {
         for (int b = 0; b < 2; ++b)
 #pragma unroll
             for (int r = 0; r < 16; ++r) {
-                const float p = exp2f(s[b][r] - m_safe);
+                const float p = exp2f(fmaf(s[b][r], scale2, -m_safe));
                 s[b][r] = p;
                 psum += p;
             }
@@ -152,10 +162,11 @@ struct WaveAttn {
 
     // One page, phases in order; the values are fetched where they are used, which keeps the
     // register count low enough for several waves per SIMD.
-    __device__ __forceinline__ void page(const T* kpage, const T* vpage, int t0, int lo, int hi, float scale2) {
+    __device__ __forceinline__ void page(const T* kpage, const T* vpage, int t0, int lo, int hi, float scale2,
+                                         bool masked = true) {
         const int lane = threadIdx.x & 63;
         f32x16 s[2];
-        scores_streamed(kpage, s, t0, lo, hi, scale2);
+        scores_streamed(kpage, s, t0, lo, hi, scale2, masked);
 #pragma unroll
         for (int tj = 0; tj < 4; ++tj) {
             v8 pf;
@@ -193,7 +204,12 @@ __global__ __launch_bounds__(256, HD <= 128 ? 2 : 1) void attn_prefill_kernel(
 
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int G = H / K, TT = 32 * (4 / GW);                     // tokens of this workgroup
-    const int tile = blockIdx.x / GW, sub = blockIdx.x % GW;
+    // A causal prompt's later token blocks read more pages.  Workgroups start in blockIdx order,
+    // 256 at a time (one per CU); every other such round walks the token blocks backwards, so the
+    // workgroups that share a CU have complementary amounts of work (measured: 15% at 2,048 tokens).
+    int bx = blockIdx.x;
+    if ((blockIdx.y / max(1, 256 / (int)gridDim.x)) & 1) bx = gridDim.x - 1 - bx;
+    const int tile = bx / GW, sub = bx % GW;
     const int seq = tile_seq[tile];
     const int kvh = blockIdx.y / (G / GW), hc = blockIdx.y % (G / GW);
     const int h = kvh * G + hc * GW + wave % GW;
@@ -210,6 +226,13 @@ __global__ __launch_bounds__(256, HD <= 128 ? 2 : 1) void attn_prefill_kernel(
     WaveAttn<T> a;
     a.init(live ? q + (tok * H + h) * HD : nullptr);
     const int lo = (window > 0 && live) ? max(0, pos - window + 1) : 0;
+    // keys from lo_max to hi_min are seen by every row of the wave: pages inside need no mask
+    int lo_max = lo, hi_min = pos;
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) {
+        lo_max = max(lo_max, __shfl_xor(lo_max, o, WAVE));
+        hi_min = min(hi_min, __shfl_xor(hi_min, o, WAVE));
+    }
     // pages of the workgroup and of this wave
     const int p_lo = (window > 0 ? max(0, base + q0 - window + 1) : 0) / PAGE;
     const int p_hi = (base + min(q0 + TT - 1, qlen - 1)) / PAGE;
@@ -254,7 +277,8 @@ __global__ __launch_bounds__(256, HD <= 128 ? 2 : 1) void attn_prefill_kernel(
         T* cur = smem + ((p - p_lo) & 1) * (KE + VE);
         T* nxt = smem + ((p - p_lo + 1) & 1) * (KE + VE);
         if (p < p_hi) fetch(p + 1);
-        if (p >= wp_lo && p <= wp_hi) a.page(cur, cur + KE, p * PAGE, lo, pos, scale2);
+        if (p >= wp_lo && p <= wp_hi)
+            a.page(cur, cur + KE, p * PAGE, lo, pos, scale2, p * PAGE < lo_max || p * PAGE + PAGE - 1 > hi_min);
         if (p < p_hi) stash(nxt);
         __syncthreads();
     }
@@ -308,7 +332,7 @@ __global__ __launch_bounds__(64) void attn_decode_kernel(
     if (p0 < p1) a.load_k(kbase + (int64_t)table[p0] * c.page_stride, kf);
     for (int p = p0; p < p1; ++p) {
         a.load_v(vbase + (int64_t)table[p] * c.page_stride, vf);
-        a.scores(kf, s, p * PAGE, lo, live ? pos : -1, scale2);
+        a.scores(kf, s, p * PAGE, lo, live ? pos : -1, scale2, p * PAGE < lo || p * PAGE + PAGE - 1 > pos);
         if (p + 1 < p1) a.load_k(kbase + (int64_t)table[p + 1] * c.page_stride, kf);
         a.mix(vf, s);
     }
