@@ -90,7 +90,7 @@ def main() -> int:
     def decode_run(batch, steps, warmup):
         """Fills `batch` sequences to just below the context length with random keys and values,
         then times `steps` decode steps."""
-        start = args.context - steps - warmup - 1
+        start = args.context - steps - warmup - 2            # warm-up enqueues one step more than it returns
         slots = [engine.alloc_slot() for _ in range(batch)]
         cache.grow(slots, [start] * batch)
         for g in cache.groups:
@@ -100,15 +100,17 @@ def main() -> int:
         runner = engine.decode_runner(sampler, use_graph=True)
         gen = torch.Generator().manual_seed(batch)
         toks = torch.randint(0, cfg.vocab_size, (batch,), generator=gen).tolist()
+        # as in the generation loop: the next step is enqueued before this one's tokens are read
         for _ in range(warmup):
-            toks = runner.run(slots, toks)
+            toks = runner.run(slots, toks, may_follow=True)
+        runner.drain()
         torch.cuda.synchronize()
         t = time.perf_counter()
-        for _ in range(steps):
-            toks = runner.run(slots, toks)
+        for i in range(steps):
+            toks = runner.run(slots, toks, may_follow=i + 1 < steps)
         torch.cuda.synchronize()
         dt = time.perf_counter() - t
-        ctx_mid = start + warmup + steps // 2
+        ctx_mid = start + warmup + 1 + steps // 2
         for s in slots:
             engine.free_slot(s)
         return dt, ctx_mid

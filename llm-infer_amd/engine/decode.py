@@ -19,10 +19,13 @@ class PlainDecodeRunner:
     def __init__(self, engine, sampler):
         self.engine, self.sampler = engine, sampler
 
-    def run(self, slots, tokens):
+    def run(self, slots, tokens, may_follow: bool = False):
         logits = self.engine.step(slots, [[t] for t in tokens])
         slot_dev = torch.tensor(slots, dtype=torch.int32, device=self.engine.device)
         return self.sampler.sample(logits, slot_dev, self.engine.cache).tolist()
+
+    def drain(self):
+        pass
 
 
 class _GraphContext:
@@ -59,8 +62,15 @@ class GraphDecodeRunner:
             self.bufs = {k: torch.zeros((n,), dtype=torch.int32, device=dev)
                          for k in ("tokens", "slots", "pos", "ctx", "next")}
             self.bufs["rows"] = torch.arange(n, dtype=torch.int32, device=dev)
+            # where the tokens of the steps in flight arrive on the host
+            self.bufs["host"] = [torch.zeros((n,), dtype=torch.int32, pin_memory=True) for _ in range(3)]
+            self.bufs["done"] = [torch.cuda.Event() for _ in range(3)]
             engine._graph_bufs = self.bufs
         self.current = None            # the slots now in the buffers
+        self._ahead = None             # a step enqueued before its predecessor's tokens were read
+        self._fed = None               # slot -> the token that step was fed on the device
+        self._host, self._done = self.bufs["host"], self.bufs["done"]
+        self._turn = 0
 
     def _splits(self, n, max_ctx):
         spec = None
@@ -82,12 +92,16 @@ class GraphDecodeRunner:
         self.sampler.sample(logits, b["slots"][:n], eng.cache, out=b["next"])
         b["tokens"][:n].copy_(b["next"][:n])
 
-    def run(self, slots, tokens):
+    def _launch(self, slots, tokens):
+        """Enqueues one step for ``slots`` and the copy of its tokens to pinned host memory.
+        ``tokens`` None: the tokens the step before left on the device are fed."""
         eng, cache, b = self.engine, self.engine.cache, self.bufs
         n = len(slots)
         new_lens = [cache.lens[s] + 1 for s in slots]
         cache.grow(slots, new_lens, sync_lens=False)
         if self.current != list(slots):
+            if tokens is None:
+                raise RuntimeError("a new set of sequences needs its tokens")
             b["slots"][:n].copy_(torch.tensor(slots, dtype=torch.int32))
             b["tokens"][:n].copy_(torch.tensor(tokens, dtype=torch.int32))
             self.current = list(slots)
@@ -105,6 +119,46 @@ class GraphDecodeRunner:
                     self._body(n, splits)
                 eng._graphs[key] = entry = g
             entry.replay()
-        out = b["next"][:n].tolist()
-        cache.trim_windows(slots)
+        self._turn = (self._turn + 1) % len(self._host)
+        host, done = self._host[self._turn], self._done[self._turn]
+        host[:n].copy_(b["next"][:n], non_blocking=True)
+        done.record()
+        return list(slots), host, done
+
+    @staticmethod
+    def _collect(step):
+        slots, host, done = step
+        done.synchronize()
+        return host[:len(slots)].tolist()
+
+    def run(self, slots, tokens, may_follow: bool = False):
+        """One token for each of ``slots``.  ``may_follow``: the caller will ask for the same
+        sequences again with the tokens returned here unless one of them ends; then the next
+        step is enqueued before this one's tokens are read, so the device does not wait for
+        the host.  If sequences do end, the step already enqueued still serves those that go
+        on (a sequence's step does not depend on the rest of the batch); what it computed for
+        the others is dropped with their slots."""
+        slots = list(slots)
+        if self._ahead is not None:
+            step, self._ahead = self._ahead, None
+            if list(tokens) != [self._fed[s] for s in slots] or any(s not in step[0] for s in slots):
+                raise RuntimeError("a step was enqueued ahead for other sequences or tokens than those asked for now")
+            if slots == step[0] and may_follow:
+                self._ahead = self._launch(slots, None)
+            every = self._collect(step)
+            out = [every[step[0].index(s)] for s in slots]
+        else:
+            step = self._launch(slots, tokens)
+            if may_follow:
+                self._ahead = self._launch(slots, None)
+            out = self._collect(step)
+        self._fed = dict(zip(slots, out)) if self._ahead is not None else None
+        self.engine.cache.trim_windows(slots)
         return out
+
+    def drain(self):
+        """Waits for a step enqueued ahead and drops its tokens.  Its sequences have moved on by
+        that step all the same: they can be freed, not continued with other tokens."""
+        if self._ahead is not None:
+            self._collect(self._ahead)
+            self._ahead = self._fed = None

@@ -59,6 +59,11 @@ class BatchTracker:
     def live(self):
         return [i for i, f in enumerate(self.finished) if not f]
 
+    def will_go_on(self, live) -> bool:
+        """True if every live request goes on after its next token unless that is a stop token."""
+        return all(len(self.outputs[i]) + 1 < self.max_new and
+                   self.prompt_lens[i] + len(self.outputs[i]) + 1 <= self.max_positions for i in live)
+
     def accept(self, live, sampled):
         go_on = []
         for i, t in zip(live, sampled):
@@ -123,8 +128,9 @@ def generate(engine, prompts, max_new_tokens: int = 256, temperature: float = 1.
                 runner = engine.decode_runner(sampler, use_graph)
                 while live:
                     new = [tracker.outputs[i][-1] for i in live]
-                    sampled = runner.run([slots[i] for i in live], new)
+                    sampled = runner.run([slots[i] for i in live], new, may_follow=tracker.will_go_on(live))
                     live = tracker.accept(live, sampled)
+                runner.drain()
                 torch.cuda.synchronize()
                 stats.decode_s += time.perf_counter() - t0
             for j, r in enumerate(batch):

@@ -167,6 +167,19 @@ def test_the_loop_decisions():
     assert t.live() == [] and t.reason == ["length"]
 
 
+def test_the_loop_knows_beforehand_whether_all_go_on():
+    """will_go_on is what lets a step be enqueued before the tokens of the step before are read:
+    it must say exactly whether tokens that are no stop tokens keep every live request going."""
+    for lens, budget, limit in (([3, 5, 2], 4, 8), ([5], 10, 6), ([1, 1], 1, 100), ([2, 9], 7, 12)):
+        t = BatchTracker(lens, budget, {9}, limit)
+        live = t.live()
+        while live:
+            said = t.will_go_on(live)
+            go = t.accept(live, [1] * len(live))
+            assert said == (go == live)
+            live = go
+
+
 def test_decode_splits_fill_the_chip_and_are_powers_of_two():
     assert decode_splits(1, 8, 32, 8192) == 64
     assert decode_splits(8, 8, 32, 8192) == 16
