@@ -130,22 +130,27 @@ struct WaveAttn {
         mx = fmaxf(mx, __shfl_xor(mx, 32, WAVE)) * scale2;
         const float m_new = fmaxf(m, mx);
         const float m_safe = (m_new == -INFINITY) ? 0.f : m_new;
-        const float alpha = exp2f(m - m_safe);
+        // the hardware's 2^x as it is: results below the smallest normal number become 0, which
+        // is what a probability that small is here
+        const float alpha = __builtin_amdgcn_exp2f(m - m_safe);
         float psum = 0.f;
 #pragma unroll
         for (int b = 0; b < 2; ++b)
 #pragma unroll
             for (int r = 0; r < 16; ++r) {
-                const float p = exp2f(fmaf(s[b][r], scale2, -m_safe));
+                const float p = __builtin_amdgcn_exp2f(fmaf(s[b][r], scale2, -m_safe));
                 s[b][r] = p;
                 psum += p;
             }
         l = l * alpha + psum;
         m = m_new;
+        // once the running maximum has settled no row of the wave needs rescaling
+        if (__builtin_amdgcn_ballot_w64(alpha != 1.f) != 0) {
 #pragma unroll
-        for (int b = 0; b < DB; ++b)
+            for (int b = 0; b < DB; ++b)
 #pragma unroll
-            for (int r = 0; r < 16; ++r) o[b][r] *= alpha;
+                for (int r = 0; r < 16; ++r) o[b][r] *= alpha;
+        }
     }
 
     // o += V^T P^T: the probabilities go from the score accumulators into operand B as they lie.
