@@ -178,6 +178,8 @@ def linear(x: torch.Tensor, w, mode: int = EPI_STORE, out: torch.Tensor | None =
             return out
         if force is None and m <= 96:
             kind = "stream"
+        elif force is None and m * k * 2 < (1 << 32):
+            kind = "dma"
     if kind.startswith("stream"):
         _need(tiled and fast_ok and m <= 128, "gemm_stream: a tiled weight and at most 128 rows")
         parts = kind.split(":")
@@ -185,6 +187,16 @@ def linear(x: torch.Tensor, w, mode: int = EPI_STORE, out: torch.Tensor | None =
         ws = _workspace(splits * m * n, x.device) if splits > 1 else None
         _check(lib.li_gemm_stream(_ptr(x), _ptr(wd), DT[x.dtype], _ptr(out), out_dt, mode, m, n, k, nt, splits,
                                   _ptr(ws), rs, _stream()), "gemm_stream")
+        return out
+    if kind.startswith("dma"):
+        _need(tiled and fast_ok and m * k * 2 < (1 << 32), "gemm_dma: a tiled weight, X below 4 GiB")
+        parts = kind.split(":")
+        tile, splits = _dma_shape(m, n, k)
+        if len(parts) > 1:
+            tile, splits = int(parts[1]), (int(parts[2]) if len(parts) > 2 else 1)
+        ws = _workspace(splits * m * n, x.device) if splits > 1 else None
+        _check(lib.li_gemm_dma(_ptr(x), _ptr(wd), DT[x.dtype], _ptr(out), out_dt, mode, m, n, k, tile, splits,
+                               _ptr(ws), rs, _stream()), "gemm_dma")
         return out
     if kind == "fma":
         _check(lib.li_gemm_fma(_ptr(x), DT[x.dtype], _ptr(w), DT[w.dtype], _ptr(out), out_dt, mode,
@@ -233,6 +245,20 @@ def _stream_shape(n: int, k: int) -> tuple[int, int]:
         return 2, s2
     g1 = -(-n // 64)
     return 1, splits_for(g1)
+
+
+def _dma_shape(m: int, n: int, k: int) -> tuple[int, int]:
+    """Tile (0 = 128x128, 1 = 256x128, 2 = 256x256 rows of W x rows of X) and splits of K for
+    gemm_dma (measured on MI355X): the largest tile that still gives most of the 256 CUs a
+    workgroup; below that the smallest tile with K split."""
+    g2 = -(-m // 256) * -(-n // 256)
+    if g2 >= 192:
+        return 2, 1
+    g1 = -(-m // 128) * -(-n // 256)
+    if g1 >= 192:
+        return 1, 1
+    g0 = -(-m // 128) * -(-n // 128)
+    return 0, (1 if g0 >= 192 else max(1, min(384 // g0, k // 512, 16)))
 
 
 def _big_tile(m: int, n: int) -> int:

@@ -119,6 +119,7 @@ def test_linear_tiled_weights(ops, M, N, K, dt):
     wt = ops.tile_weight(w)
     assert wt.shape == (N, K) and wt.data.numel() == (N + 15) // 16 * 16 * K
     kinds = [None, "mfma:0:1", "mfma:1:2", "mfma:2:1", "big:0", "big:1", "big:0:2", "big:1:5"] + (["gemv_mfma"] if M <= 16 else [])
+    kinds += ["dma", "dma:0", "dma:1", "dma:2", "dma:0:2", "dma:1:5", "dma:2:3"]
     if M <= 128:
         kinds += ["stream", "stream:1:1", "stream:2:1", "stream:1:3", "stream:2:16"]
     for kind in kinds:
@@ -371,7 +372,7 @@ def test_rotation_fused_into_the_projection(ops, dt, T, H, K, hd, rot, d):
         if tiled and d % 32:
             continue
         ww = ops.tile_weight(w) if tiled else w
-        for kind in kinds + (["stream:1:1", "stream:2:2"] if tiled and T <= 128 else []):
+        for kind in kinds + ((["dma:0", "dma:1:2", "dma:2"] + (["stream:1:1", "stream:2:2"] if T <= 128 else [])) if tiled else []):
             if tiled and kind == "fma":
                 continue
             c1, v1 = fresh()
