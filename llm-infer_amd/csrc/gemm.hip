@@ -480,12 +480,12 @@ __global__ __launch_bounds__(256) void gemm_big_kernel(const T* __restrict__ X, 
 // addresses and dropped by the epilogue.  Three LDS buffers: the loads of tile t + 2 are
 // issued while tile t is multiplied; one barrier per tile.
 // ===========================================================================
-template <class T, int BN, int BM, int WAVES>
+template <class T, int BN, int BM, int WAVES, int STAGES>
 __global__ __launch_bounds__(64 * WAVES) void gemm_dma_kernel(const T* __restrict__ X, const T* __restrict__ Wt,
                                                           int K, int k_per_split, float* __restrict__ ws,
                                                           Epilogue e) {
     typedef typename Vec<T>::v8 v8;
-    constexpr int BK = 32, STAGES = 3;
+    constexpr int BK = 32;
     constexpr int TN = BN / 2, TM = BM / (WAVES / 2), NB = TN / 32, MB = TM / 32;   // 2 waves along N
     constexpr int WU = BN / 16, XU = BM / 16, UNITS = WU + XU;       // 1 KiB units of a stage
     constexpr int PER_WAVE = UNITS / WAVES;
@@ -567,18 +567,32 @@ __global__ __launch_bounds__(64 * WAVES) void gemm_dma_kernel(const T* __restric
     // The loop works in half tiles (16 of the 32 elements of K): while the matrix cores work on
     // one half, the fragments of the next are on their way from LDS.  In the middle of tile t every
     // wave has read all of it, so the barrier there both publishes tile t + 1 and frees the buffer
-    // of tile t for the loads of tile t + 3: loads run two tiles ahead with three buffers.
+    // of tile t for the loads of tile t + STAGES: loads run STAGES - 1 tiles ahead.
     // (A bare s_barrier: __syncthreads would also wait for the loads still in flight.)
     // One copy of the body, the buffer a run-time offset: unrolled by the three buffers the
     // register allocator spills.  After the last tile the reads for "the next tile" fetch stale
     // data that nothing uses.
     v8 a0[NB], b0[MB], a1[NB], b1[MB];
-    issue(0, 0);
-    if (n_tiles > 1) issue(1, 1);
-    if (n_tiles > 2) issue(2, 2);
-    if (n_tiles > 2) __builtin_amdgcn_s_waitcnt(0x0F70 | (2 * PER_WAVE));
-    else if (n_tiles > 1) __builtin_amdgcn_s_waitcnt(0x0F70 | PER_WAVE);
-    else __builtin_amdgcn_s_waitcnt(0x0F70);
+    // waits until at most `tiles` of the tiles whose loads were issued last are still in flight
+    auto wait_tiles = [&](int tiles, bool lds_too) {
+        if (lds_too) {
+            if (tiles <= 0) __builtin_amdgcn_s_waitcnt(0x0070);
+            else if (tiles == 1) __builtin_amdgcn_s_waitcnt(0x0070 | PER_WAVE);
+            else if (tiles == 2) __builtin_amdgcn_s_waitcnt(0x0070 | (2 * PER_WAVE));
+            else __builtin_amdgcn_s_waitcnt(0x0070 | (3 * PER_WAVE));
+        } else {
+            if (tiles <= 0) __builtin_amdgcn_s_waitcnt(0x0F70);
+            else if (tiles == 1) __builtin_amdgcn_s_waitcnt(0x0F70 | PER_WAVE);
+            else if (tiles == 2) __builtin_amdgcn_s_waitcnt(0x0F70 | (2 * PER_WAVE));
+            else if (tiles == 3) __builtin_amdgcn_s_waitcnt(0x0F70 | (3 * PER_WAVE));
+            else __builtin_amdgcn_s_waitcnt(0x0F70 | (3 * PER_WAVE));
+        }
+    };
+    static_assert(STAGES >= 3 && STAGES <= 5 && (STAGES - 2) * PER_WAVE <= 15, "stages");
+#pragma unroll
+    for (int i = 0; i < STAGES; ++i)
+        if (i < n_tiles) issue(i, i);
+    wait_tiles(min(min(STAGES, n_tiles) - 1, 3), false);
     __builtin_amdgcn_s_barrier();
     read_frags(0, 0, a0, b0);
     int cur = 0;
@@ -589,11 +603,11 @@ __global__ __launch_bounds__(64 * WAVES) void gemm_dma_kernel(const T* __restric
         __builtin_amdgcn_sched_barrier(0);
         multiply(a0, b0);
         __builtin_amdgcn_sched_barrier(0);
-        // tile t + 1 has landed (tile t + 2 may be in flight); this wave's reads of tile t are done
-        if (t + 2 < n_tiles) __builtin_amdgcn_s_waitcnt(0x0070 | PER_WAVE);
-        else __builtin_amdgcn_s_waitcnt(0x0070);
+        // tile t + 1 has landed (up to STAGES - 2 later ones may be in flight); this wave's reads
+        // of tile t are done
+        wait_tiles(min(STAGES - 2, n_tiles - 2 - t), true);
         __builtin_amdgcn_s_barrier();
-        if (t + 3 < n_tiles) issue(t + 3, cur);
+        if (t + STAGES < n_tiles) issue(t + STAGES, cur);
         read_frags(nxt, 0, a0, b0);
         __builtin_amdgcn_sched_barrier(0);
         multiply(a1, b1);
@@ -1220,7 +1234,7 @@ extern "C" int li_gemm_stream(const void* X, const void* Wt, int dt, void* C, in
     return LI_OK;
 }
 
-// tile: 0 = 128 x 128, 1 = 256 x 128, 2 = 256 x 256 with 8 waves (rows of W x rows of X), BK = 32; W tiled
+// tile: 0 = 128 x 128, 1 = 256 x 128, 2 = 256 x 256 with 8 waves (rows of W x rows of X); BK = 32; W tiled
 extern "C" int li_gemm_dma(const void* X, const void* Wt, int dt, void* C, int out_dt, int mode,
                            int M, int N, int K, int tile, int splits, float* ws, const RopeStore* rs,
                            hipStream_t stream) {
@@ -1235,19 +1249,24 @@ extern "C" int li_gemm_dma(const void* X, const void* Wt, int dt, void* C, int o
     Epilogue e;
     rc = make_epilogue(e, C, mode, out_dt, M, N, rs);
     if (rc) return rc;
-    const int bn = tile ? 256 : 128, bm = tile >= 2 ? 256 : 128, bk = 32;
+    const int bn = tile ? 256 : 128, bm = tile == 2 ? 256 : 128, bk = 32;
     const size_t lds = (size_t)3 * (bn + bm) / 16 * 1024;
     int k_per_split = ((K + splits - 1) / splits + bk - 1) / bk * bk;
     splits = (K + k_per_split - 1) / k_per_split;
     dim3 grid((M + bm - 1) / bm, (N + bn - 1) / bn, splits), block(tile == 2 ? 512 : 256);
-#define GO(T, BN, BM, WV)                                                                                \
+#define GO(T, BN, BM, WV, ST)                                                                                \
     do {                                                                                               \
-        auto kfn = gemm_dma_kernel<T, BN, BM, WV>;                                                     \
+        auto kfn = gemm_dma_kernel<T, BN, BM, WV, ST>;                                                 \
         if (hipFuncSetAttribute((const void*)kfn, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds) != hipSuccess) \
             return LI_HIP_ERROR;                                                                       \
         kfn<<<grid, block, lds, stream>>>((const T*)X, (const T*)Wt, K, k_per_split, ws, e);           \
     } while (0)
-#define LAUNCH(T) do { if (tile == 0) GO(T, 128, 128, 4); else if (tile == 1) GO(T, 256, 128, 4); else GO(T, 256, 256, 8); } while (0)
+#define LAUNCH(T)                                    \
+    do {                                             \
+        if (tile == 0) GO(T, 128, 128, 4, 3);        \
+        else if (tile == 1) GO(T, 256, 128, 4, 3);   \
+        else GO(T, 256, 256, 8, 3);                  \
+    } while (0)
     if (dt == DT_F16) LAUNCH(f16); else LAUNCH(bf16);
 #undef LAUNCH
 #undef GO
