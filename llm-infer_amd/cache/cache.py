@@ -85,7 +85,7 @@ class KVGroup:
             return 0
         return max(0, length - self.spec.window + 1) // PAGE
 
-    def reserve(self, slot: int, old_len: int, new_len: int, dirty: set, fresh: list) -> None:
+    def reserve(self, slot: int, old_len: int, new_len: int, dirty: set, fresh: list, filled: bool = False) -> None:
         have = self.pages_of[slot]
         lo = self.first_needed_page(old_len) if self.spec.window is not None else 0
         want = range(lo, (new_len + PAGE - 1) // PAGE)
@@ -96,7 +96,10 @@ class KVGroup:
         for p, page in zip(need, got):
             have[p] = page
             self.table_host[slot, p] = page
-        fresh.extend(got)
+            # a page that the caller fills from its first to its last token needs no clearing: only
+            # what stays unwritten could reach a product as 0 x garbage
+            if not (filled and old_len <= p * PAGE and new_len >= (p + 1) * PAGE):
+                fresh.append(page)
         dirty.add(slot)
 
     def release_outside_window(self, slot: int, length: int, dirty: set) -> None:
@@ -200,9 +203,11 @@ class Cache:
                 g.release(slot)
         self.lens[slot] = 0
 
-    def grow(self, slots, new_lens, sync_lens: bool = True) -> None:
+    def grow(self, slots, new_lens, sync_lens: bool = True, filled: bool = False) -> None:
         """Make room for each slot to reach its new length, then record the lengths.  All page
-        tables and fresh pages are updated with one small copy and one fill per group."""
+        tables and fresh pages are updated with one small copy and one fill per group.
+        ``filled``: the caller writes every position between the old and the new length before
+        anything reads the cache (a step does), so pages that lie wholly in between are not cleared."""
         for slot, n in zip(slots, new_lens):
             if n > self.max_positions:
                 raise CacheError(f"a sequence of {n} tokens exceeds the model's {self.max_positions} positions")
@@ -214,7 +219,7 @@ class Cache:
             dirty, fresh = set(), []
             try:
                 for slot, n in zip(slots, new_lens):
-                    g.reserve(slot, self.lens[slot], n, dirty, fresh)
+                    g.reserve(slot, self.lens[slot], n, dirty, fresh, filled)
             finally:
                 g.flush(dirty, fresh)
         for slot, n in zip(slots, new_lens):

@@ -107,5 +107,6 @@ class Engine:
             if any(not 0 <= i < len(t) for i in w):
                 raise ValueError(f"step: wanted place outside the {len(t)} tokens of slot {s}")
         before = [self.cache.lens[s] for s in slots]
-        self.cache.grow(slots, [b + len(t) for b, t in zip(before, tokens)])
+        # every mixer writes all of the step's tokens into its cache before anything reads it
+        self.cache.grow(slots, [b + len(t) for b, t in zip(before, tokens)], filled=True)
         return StepContext(self.device, slots, tokens, before, want)
