@@ -288,6 +288,27 @@ __global__ __launch_bounds__(256) void gemm_mfma_kernel(const T* __restrict__ X,
         }
 }
 
+// Which tile a workgroup works on.  Workgroups go to the 8 XCDs in turn (workgroup L to XCD
+// L % 8) and every XCD has an L2 of its own, so the tiles are numbered such that an XCD works on
+// one contiguous run of them; within the run, groups of GM tiles of X go through all tiles of W
+// before the next group starts.  The workgroups that are resident on an XCD together (32 or 64)
+// then cover a near-square block of tiles and share its rows of X and W through that L2; with
+// the tiles of X simply fastest they would share one tile of W and stream all of X past it.
+__device__ __forceinline__ void tile_of_workgroup(int GM, int& bx, int& by, int& bz) {
+    const int gx = gridDim.x, gy = gridDim.y;
+    const int total = gx * gy * gridDim.z;
+    const int L = blockIdx.x + gx * (blockIdx.y + gy * blockIdx.z);
+    const int xcd = L & 7, per = total >> 3, rem = total & 7;
+    const int id = xcd * per + min(xcd, rem) + (L >> 3);
+    bz = id / (gx * gy);
+    const int in_split = id - bz * gx * gy;
+    const int group = in_split / (GM * gy), first = group * GM;
+    const int size = min(gx - first, GM);
+    const int in_group = in_split - group * GM * gy;
+    bx = first + in_group % size;
+    by = in_group / size;
+}
+
 // ===========================================================================
 // gemm_big: the prefill product.  BN rows of W x BM rows of X per workgroup of 4
 // waves (2 x 2), each wave a (BN/2) x (BM/2) tile of 32x32 blocks, BK = 64.  Two LDS
@@ -312,16 +333,8 @@ __global__ __launch_bounds__(256) void gemm_big_kernel(const T* __restrict__ X, 
 
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int wn = wave & 1, wm = wave >> 1;
-    // Workgroups go to the 8 XCDs in turn (workgroup L to XCD L % 8) and every XCD has an L2 of its
-    // own.  The tiles are numbered so that an XCD works on one contiguous run of them, the tiles of
-    // X fastest: the workgroups that are resident on an XCD together then share their rows of W
-    // (and a few tiles of X) through its L2 instead of fetching them into all eight.
-    const int gx = gridDim.x, gy = gridDim.y;
-    const int total = gx * gy * gridDim.z;
-    const int L = blockIdx.x + gx * (blockIdx.y + gy * blockIdx.z);
-    const int xcd = L & 7, per = total >> 3, rem = total & 7;
-    const int id = xcd * per + min(xcd, rem) + (L >> 3);
-    const int bx = id % gx, by = (id / gx) % gy, bz = id / (gx * gy);
+    int bx, by, bz;
+    tile_of_workgroup(8, bx, by, bz);
     const int m0 = bx * BM, n0 = by * BN;
     const int n_limit = TILED ? ((e.N + 15) & ~15) : e.N;
     const int kb = bz * k_per_split, ke = min(K, kb + k_per_split);   // this workgroup's share of K
@@ -496,13 +509,8 @@ __global__ __launch_bounds__(64 * WAVES) void gemm_dma_kernel(const T* __restric
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);       // uniform: what depends on it stays scalar
     const int wn = wave & 1, wm = wave >> 1;
-    // tiles numbered so that an XCD (workgroup L goes to XCD L % 8) works on a contiguous run
-    const int gx = gridDim.x, gy = gridDim.y;
-    const int total = gx * gy * gridDim.z;
-    const int L = blockIdx.x + gx * (blockIdx.y + gy * blockIdx.z);
-    const int xcd = L & 7, per = total >> 3, rem = total & 7;
-    const int id = xcd * per + min(xcd, rem) + (L >> 3);
-    const int bx = id % gx, by = (id / gx) % gy, bz = id / (gx * gy);
+    int bx, by, bz;
+    tile_of_workgroup(BM == 256 ? 4 : 8, bx, by, bz);
     const int m0 = bx * BM, n0 = by * BN;
     const int kb = bz * k_per_split, ke = min(K, kb + k_per_split);
     const int n_tiles = (ke - kb) / BK;
