@@ -78,7 +78,9 @@ class Engine:
 
     def decode_runner(self, sampler, use_graph: bool = True):
         from .decode import GraphDecodeRunner, PlainDecodeRunner
-        return GraphDecodeRunner(self, sampler) if use_graph else PlainDecodeRunner(self, sampler)
+        if use_graph and self.model.recordable():
+            return GraphDecodeRunner(self, sampler)
+        return PlainDecodeRunner(self, sampler)
 
     def generate(self, prompts, **kw):
         from .generate import generate

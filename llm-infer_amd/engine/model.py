@@ -41,6 +41,16 @@ class DecoderModel(Part):
     def children(self):
         return [self.embedding, *self.layers, self.final_norm, self.head]
 
+    def recordable(self) -> bool:
+        """True if every part's forward pass can be recorded into a graph."""
+        stack = list(self.children())
+        while stack:
+            part = stack.pop()
+            if not getattr(part, "recordable", True):
+                return False
+            stack += list(part.children()) if hasattr(part, "children") else []
+        return True
+
     def params(self) -> dict:
         """Full tensor name -> ParamSpec of everything the model needs."""
         return {name: spec for name, (_, _, spec) in getattr(self, "_table", {}).items()}

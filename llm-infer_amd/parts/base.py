@@ -12,6 +12,9 @@ from __future__ import annotations
 
 class Part:
     prefix: str = ""
+    # False for a part whose forward pass waits for the device (a data-dependent shape, a copy to
+    # the host): such a step cannot be recorded, and decoding then runs it eagerly.
+    recordable: bool = True
 
     def params(self) -> dict:
         """local tensor name -> ParamSpec"""

@@ -544,3 +544,155 @@ def test_toy_architecture_with_a_window_group(lib, dtype):
     assert err.max().item() < tol, f"first wrong place: {int((err >= tol).nonzero()[0])}"
     eng.free_slot(s)
     assert groups[70].pool.n_free == groups[None].pool.n_free == cache.n_pages - 1
+
+
+# ---------------------------------------------------------------------------
+# a toy feed-forward with routing and a toy position encoding, both defined here
+# ---------------------------------------------------------------------------
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_toy_routed_feed_forward_and_another_position_encoding(lib, dtype):
+    """A feed-forward that sends every token to one of three experts (router logits and weights in
+    float32) and a rotation whose angles are those of position / 4: registered from the test, built
+    by the registry from a config, run by the engine whole, cut and in a ragged batch.  Nothing in
+    the framework's files names either."""
+    from llm_infer_amd.config.spec import LayerSpec, ModelSpec, PartSpec, ScheduleEntry
+    from llm_infer_amd.engine import Engine
+    from llm_infer_amd.kernels import ops
+    from llm_infer_amd.parts.base import Part
+    from llm_infer_amd.parts.position import RotaryPosition
+    from llm_infer_amd.weights.loader import ParamSpec
+
+    @lib.register_feed_forward("toy_top1")
+    class Top1Experts(Part):
+        recordable = False            # the rows of an expert are counted on the host
+
+        def __init__(self, *, hidden_size, expert_size, n_experts, prefix, dtype, device):
+            self.d, self.f, self.e, self.prefix, self.dtype = hidden_size, expert_size, n_experts, prefix, dtype
+
+        def params(self):
+            p = {"router.weight": ParamSpec((self.e, self.d))}
+            for i in range(self.e):
+                p[f"experts.{i}.up.weight"] = ParamSpec((self.f, self.d))
+                p[f"experts.{i}.down.weight"] = ParamSpec((self.d, self.f))
+            return p
+
+        def bind(self, tensors):
+            self.router = tensors["router.weight"].float()
+            self.up = [tensors[f"experts.{i}.up.weight"] for i in range(self.e)]
+            self.down = [tensors[f"experts.{i}.down.weight"] for i in range(self.e)]
+
+        def forward(self, h, residual):
+            logits = ops.linear(h.float(), self.router, out_dtype=torch.float32)       # float32 router
+            weight, pick = torch.softmax(logits, dim=-1).max(dim=-1)
+            for i in range(self.e):
+                rows = (pick == i).nonzero().flatten()
+                if rows.numel() == 0:
+                    continue
+                a = torch.relu(ops.linear(h[rows].contiguous(), self.up[i], out_dtype=torch.float32))
+                y = ops.linear(a.to(self.dtype), self.down[i], out_dtype=torch.float32)
+                residual.index_add_(0, rows, y * weight[rows, None])
+
+    @lib.register_position("toy_slow_rope")
+    class SlowRotary(RotaryPosition):
+        """The rotation of position / slowdown: only the table of frequencies differs."""
+
+        def __init__(self, *, slowdown, **kw):
+            super().__init__(**kw)
+            self.inv_freq = self.inv_freq / float(slowdown)
+            self.theta = (self.theta, float(slowdown))          # the per-step table is keyed by it
+
+    class RoutedConfig:
+        def __init__(self, raw):
+            self.raw = raw
+
+        @classmethod
+        def from_dict(cls, raw):
+            return cls(raw)
+
+        def model_spec(self):
+            r = self.raw
+            d, hd = r["width"], r["head"]
+            norm = PartSpec("rmsnorm", {"size": d, "eps": r["eps"]})
+            layers = []
+            for i in range(2):
+                mix = PartSpec("attention", {"hidden_size": d, "n_heads": 3, "n_kv_heads": 3, "head_dim": hd,
+                                             "scale": hd ** -0.5}, f"l{i}.mix.")
+                ffn = PartSpec("toy_top1", {"hidden_size": d, "expert_size": r["expert"], "n_experts": 3}, f"l{i}.moe.")
+                pos = PartSpec("toy_slow_rope", {"theta": 50.0, "rotary_dim": hd, "head_dim": hd, "slowdown": 4.0})
+                layers.append(LayerSpec("pre_norm", mix, ffn, norm.with_prefix(f"l{i}.n1."),
+                                        norm.with_prefix(f"l{i}.n2."), pos))
+            return ModelSpec(d, r["vocab"], r["positions"],
+                             PartSpec("embedding", {"vocab_size": r["vocab"], "hidden_size": d}, "emb."),
+                             tuple(layers), (ScheduleEntry(0), ScheduleEntry(1)), norm.with_prefix("final."),
+                             PartSpec("lm_head", {"vocab_size": r["vocab"], "hidden_size": d, "tied": False}, "head."))
+
+    lib.register_architecture("RoutedToyForCausalLM", RoutedConfig)
+    raw = {"architectures": ["RoutedToyForCausalLM"], "width": 64, "head": 16, "expert": 40, "eps": 1e-6,
+           "vocab": 70, "positions": 256}
+    eng = Engine.from_random(lib.config_from_dict(raw), seed=4, dtype=dtype, max_tokens=512)
+    # the same weights (values that bfloat16 holds) as plain float32 tensors, for the reference
+    model = Engine.from_random(lib.config_from_dict(raw), seed=4, dtype="float32", max_tokens=64).model
+
+    # random routers are indifferent; scaled up they decide, so that a wrong choice would show
+    for m_ in (eng.model, model):
+        for layer in m_.layers:
+            layer.feed_forward.router *= 30.0
+
+    def dbl(t):
+        return t.double().cpu()
+
+    def ref_forward(toks):
+        """float64, whole sequence; the expert of a token is taken from the engine's own choice only
+        where the two best router logits are closer than rounding could decide."""
+        n = len(toks)
+        x = dbl(model.embedding.weight)[toks]
+        posn = torch.arange(n, dtype=torch.float64) / 4.0
+        for layer in model.layers:
+            att, moe = layer.mixer, layer.feed_forward
+            h = P.rmsnorm(x, dbl(layer.mixer_norm.weight), 1e-6)
+            wq, wk, wv = dbl(att.wqkv).split([48, 48, 48])
+            q = P.rope((h @ wq.t()).view(n, 3, 16), posn, 50.0, 16)
+            k = P.rope((h @ wk.t()).view(n, 3, 16), posn, 50.0, 16)
+            x = x + P.attention(q, k, (h @ wv.t()).view(n, 3, 16)).reshape(n, 48) @ dbl(att.wo).t()
+            h = P.rmsnorm(x, dbl(layer.feed_forward_norm.weight), 1e-6)
+            prob = torch.softmax(h @ moe.router.double().cpu().t(), dim=-1)
+            weight, pick = prob.max(dim=-1)
+            top2 = prob.topk(2, dim=-1).values
+            sure = (top2[:, 0] - top2[:, 1]) > 0.05
+            y = torch.zeros_like(x)
+            for t in range(n):
+                e = int(pick[t])
+                y[t] = weight[t] * (torch.relu(h[t] @ dbl(moe.up[e]).t()) @ dbl(moe.down[e]).t())
+            x = x + y
+        return P.rmsnorm(x, dbl(model.final_norm.weight), 1e-6) @ dbl(model.head.weight).t(), sure
+
+    g = torch.Generator().manual_seed(11)
+    seqs = [torch.randint(0, 70, (n,), generator=g).tolist() for n in (40, 7, 90)]
+    tol = 3e-5 if dtype == "float32" else 3e-2
+    slots = [eng.alloc_slot() for _ in seqs]
+    whole = eng.step(slots, seqs, [list(range(len(t))) for t in seqs]).double().cpu()
+    for s in slots:
+        eng.free_slot(s)
+    off = 0
+    for toks in seqs:
+        ref, sure = ref_forward(toks)
+        # a token whose router was too close to call may differ from there on: compare up to it
+        upto = len(toks) if bool(sure.all()) else int((~sure).nonzero()[0])
+        scale = ref.abs().max().item()
+        assert upto >= min(5, len(toks))
+        assert (whole[off:off + upto] - ref[:upto]).abs().max().item() < tol * (1 + scale)
+        off += len(toks)
+    # cut: a first part, then one token at a time, against the engine's own whole run
+    slots = [eng.alloc_slot() for _ in seqs]
+    heads = [len(t) - 4 for t in seqs]
+    eng.step(slots, [t[:h] for t, h in zip(seqs, heads)])
+    starts = [0, len(seqs[0]), len(seqs[0]) + len(seqs[1])]
+    for kk in range(4):
+        out = eng.step(slots, [[t[h + kk]] for t, h in zip(seqs, heads)]).double().cpu()
+        for i, (h, st) in enumerate(zip(heads, starts)):
+            assert (out[i] - whole[st + h + kk]).abs().max().item() < tol * (1 + whole.abs().max().item())
+    for s in slots:
+        eng.free_slot(s)
+    a = eng.generate([seqs[1], seqs[0]], max_new_tokens=6, temperature=0.0, use_graph=True)
+    b = eng.generate([seqs[1], seqs[0]], max_new_tokens=6, temperature=0.0, use_graph=False)
+    assert a == b and all(len(o) == 6 for o in a)
