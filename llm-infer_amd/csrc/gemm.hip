@@ -291,8 +291,7 @@ __global__ __launch_bounds__(256) void gemm_mfma_kernel(const T* __restrict__ X,
 // Which tile a workgroup works on.  Workgroups go to the 8 XCDs in turn (workgroup L to XCD
 // L % 8) and every XCD has an L2 of its own, so the tiles are numbered such that an XCD works on
 // one contiguous run of them; within the run, groups of GM tiles of X go through all tiles of W
-// before the next group starts (one group if there are at most 2 GM tiles of X).  The workgroups
-// that are resident on an XCD together (32 or 64)
+// before the next group starts.  The workgroups that are resident on an XCD together (32 or 64)
 // then cover a near-square block of tiles and share its rows of X and W through that L2; with
 // the tiles of X simply fastest they would share one tile of W and stream all of X past it.
 __device__ __forceinline__ void tile_of_workgroup(int GM, int& bx, int& by, int& bz) {
@@ -303,7 +302,6 @@ __device__ __forceinline__ void tile_of_workgroup(int GM, int& bx, int& by, int&
     const int id = xcd * per + min(xcd, rem) + (L >> 3);
     bz = id / (gx * gy);
     const int in_split = id - bz * gx * gy;
-    if (gx <= 2 * GM) GM = gx;                  // few tiles of X: all of them in one group (measured)
     const int group = in_split / (GM * gy), first = group * GM;
     const int size = min(gx - first, GM);
     const int in_group = in_split - group * GM * gy;
