@@ -565,11 +565,13 @@ __global__ __launch_bounds__(64 * WAVES) void gemm_dma_kernel(const T* __restric
 #pragma unroll
         for (int i = 0; i < NB; ++i) a[i] = *(const v8*)(sW + buf * STAGE + i * 2048 + ks * 512);
     };
-    auto multiply = [&](const v8 (&a)[NB], const v8 (&b)[MB]) {
+    auto multiply = [&](const v8 (&a)[NB], const v8 (&b)[MB], int lo, int hi) {
 #pragma unroll
         for (int i = 0; i < NB; ++i)
+            if (i >= lo && i < hi) {
 #pragma unroll
-            for (int j = 0; j < MB; ++j) acc[i][j] = mfma32(a[i], b[j], acc[i][j]);
+                for (int j = 0; j < MB; ++j) acc[i][j] = mfma32(a[i], b[j], acc[i][j]);
+            }
     };
 
     // The loop works in half tiles (16 of the 32 elements of K): while the matrix cores work on
@@ -607,18 +609,25 @@ __global__ __launch_bounds__(64 * WAVES) void gemm_dma_kernel(const T* __restric
 #pragma unroll 1
     for (int t = 0; t < n_tiles; ++t) {
         const int nxt = cur == STAGES - 1 ? 0 : cur + 1;
+        // the second half's fragments are requested between the matrix instructions of the first
+        // half: requested before them, the wait the compiler places for the first half's fragments
+        // (it merges the loop's entry and back edge pessimistically) would cover these reads too
+        multiply(a0, b0, 0, NB / 2);
+        __builtin_amdgcn_sched_barrier(0);
         read_frags(cur, 1, a1, b1);
         __builtin_amdgcn_sched_barrier(0);
-        multiply(a0, b0);
+        multiply(a0, b0, NB / 2, NB);
         __builtin_amdgcn_sched_barrier(0);
         // tile t + 1 has landed (up to STAGES - 2 later ones may be in flight); this wave's reads
         // of tile t are done
         wait_tiles(min(STAGES - 2, n_tiles - 2 - t), true);
         __builtin_amdgcn_s_barrier();
         if (t + STAGES < n_tiles) issue(t + STAGES, cur);
+        multiply(a1, b1, 0, NB / 2);
+        __builtin_amdgcn_sched_barrier(0);
         read_frags(nxt, 0, a0, b0);
         __builtin_amdgcn_sched_barrier(0);
-        multiply(a1, b1);
+        multiply(a1, b1, NB / 2, NB);
         __builtin_amdgcn_sched_barrier(0);
         cur = nxt;
     }
