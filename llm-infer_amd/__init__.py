@@ -14,7 +14,8 @@ register_architecture("LlamaForCausalLM", LlamaConfig)
 
 
 def load(folder: str, dtype: str = "bfloat16", max_tokens: int = 8192, n_slots=None):
-    """Open a model folder (config.json + model.safetensors) on the GPU."""
+    """Open a model on the GPU: a folder with config.json and model.safetensors, or a GGUF file
+    with unquantized tensors (the reference's own format) or the folder that holds one."""
     from .engine import Engine
     return Engine.from_folder(folder, dtype=dtype, max_tokens=max_tokens, n_slots=n_slots)
 

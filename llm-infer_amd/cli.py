@@ -5,8 +5,9 @@
 
 Options the reference has keep their names and meanings: -i, -f, -n (tokens to generate,
 256), -t (temperature, 1.0; <= 0 is greedy), --seed, -T (context length override), -d (device;
-here only "hip": there is no CPU path), -h.  Differences: the model is a folder with
-config.json and model.safetensors; prompts may be given as token ids (one --tokens or one
+here only "hip": there is no CPU path), -h.  The model is a folder with config.json and
+model.safetensors, or, as for the reference, a GGUF file (F32/F16/BF16 tensors; its metadata
+is the configuration and holds the vocabulary).  Differences: prompts may be given as token ids (one --tokens or one
 line of --tokens-file for each request of a batch); seed 0 is a fixed seed, not a random one.
 """
 from __future__ import annotations
@@ -15,13 +16,13 @@ import json
 import sys
 import time
 
-USAGE = """Usage: infer <model_dir> [options]
+USAGE = """Usage: infer <model_dir | model.gguf> [options]
 Example: infer model_dir -i "Hello, world!"
 
 Options:
   -h                    Display this help message
   -d <device>           Device to use: hip (default: hip)
-  -i <string>           Input prompt (needs tokenizer.json in the model folder)
+  -i <string>           Input prompt (needs tokenizer.json in the folder or a GGUF vocabulary)
   -f <file>             Input prompt from file
   --tokens <ids>        Input prompt as comma separated token ids (repeat for a batch)
   --tokens-file <file>  One prompt a line, token ids separated by commas or blanks
@@ -103,8 +104,8 @@ def run(cfg) -> int:
         raw["max_position_embeddings"] = cfg["context"]
         raw["eos_token_id"] = list(config.eos_token_ids) or None
         config = llm_infer_amd.config_from_dict(raw)
-    tok = Tokenizer.from_folder(cfg["model"], config.bos_token_id,
-                                config.eos_token_ids[0] if config.eos_token_ids else None)
+    tok = Tokenizer.from_model(cfg["model"], config.bos_token_id,
+                               config.eos_token_ids[0] if config.eos_token_ids else None)
     if cfg["prompt_file"]:
         try:
             with open(cfg["prompt_file"], encoding="utf-8") as f:
@@ -113,7 +114,8 @@ def run(cfg) -> int:
             raise RuntimeError(f"Failed to open prompt file: {cfg['prompt_file']}")
     if cfg["prompt"] is not None:
         if tok is None:
-            raise RuntimeError("the model folder has no tokenizer.json: give the prompt as token ids (--tokens)")
+            raise RuntimeError("the model has no tokenizer (tokenizer.json in the folder, or tokenizer.ggml.tokens "
+                               "in a GGUF file): give the prompt as token ids (--tokens)")
         prompts = [tok.encode(cfg["prompt"], True)]
     elif cfg["tokens_file"]:
         with open(cfg["tokens_file"]) as f:

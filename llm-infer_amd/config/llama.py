@@ -79,6 +79,79 @@ class LlamaConfig:
         cfg.validate()
         return cfg
 
+    # GGUF: the reference's own model files (src/gguf.cpp:86-168 reads these keys, u32 or u64)
+    gguf_architecture = "llama"
+    _GGUF_REQUIRED = ("context_length", "embedding_length", "block_count", "feed_forward_length",
+                      "rope.dimension_count", "attention.head_count", "attention.layer_norm_rms_epsilon")
+
+    @classmethod
+    def from_gguf(cls, metadata: dict, tensor_shapes: dict) -> "LlamaConfig":
+        """``metadata``: the file's key/value pairs; ``tensor_shapes``: GGUF tensor name -> shape."""
+        md = {k[len("llama."):]: v for k, v in metadata.items() if k.startswith("llama.")}
+        missing = ["llama." + k for k in cls._GGUF_REQUIRED if k not in md]
+        if missing:
+            raise ConfigError("the GGUF file lacks required metadata: " + ", ".join(missing))
+        hidden, n_heads = int(md["embedding_length"]), int(md["attention.head_count"])
+        if n_heads <= 0 or (hidden % n_heads != 0 and "attention.key_length" not in md):
+            raise ConfigError("llama.embedding_length must be divisible by llama.attention.head_count")
+        head_dim = int(md.get("attention.key_length") or hidden // n_heads)
+        emb = tensor_shapes.get("token_embd.weight")
+        # the reference falls back to a tokenizer key of another type (src/gguf.cpp:162-167); the
+        # rows of the embedding table say it without doubt
+        vocab = int(md.get("vocab_size") or (emb[0] if emb else 0) or len(metadata.get("tokenizer.ggml.tokens", ())))
+        if "expert_count" in md and int(md["expert_count"]) > 0:
+            raise ConfigError("this GGUF file holds a model with experts; only the dense decoder is built")
+        eos = metadata.get("tokenizer.ggml.eos_token_id")
+        bos = metadata.get("tokenizer.ggml.bos_token_id")
+        cfg = cls(
+            num_hidden_layers=int(md["block_count"]), hidden_size=hidden,
+            intermediate_size=int(md["feed_forward_length"]), num_attention_heads=n_heads,
+            num_key_value_heads=int(md.get("attention.head_count_kv") or n_heads), head_dim=head_dim,
+            vocab_size=vocab, max_position_embeddings=int(md["context_length"]),
+            rope_theta=float(md.get("rope.freq_base", 10000.0)), rotary_dim=int(md["rope.dimension_count"]),
+            rms_norm_eps=float(md["attention.layer_norm_rms_epsilon"]), hidden_act="silu",
+            tie_word_embeddings="output.weight" not in tensor_shapes, torch_dtype=None,
+            bos_token_id=None if bos is None else int(bos),
+            eos_token_ids=() if eos is None else (int(eos),), rope_pairing="adjacent")
+        cfg.validate()
+        return cfg
+
+    def gguf_metadata(self) -> dict:
+        """The metadata that reads back as this configuration."""
+        md = {"general.architecture": "llama", "general.quantization_version": 2,
+              "llama.context_length": self.max_position_embeddings, "llama.embedding_length": self.hidden_size,
+              "llama.block_count": self.num_hidden_layers, "llama.feed_forward_length": self.intermediate_size,
+              "llama.rope.dimension_count": self.rotary_dim, "llama.attention.head_count": self.num_attention_heads,
+              "llama.attention.head_count_kv": self.num_key_value_heads,
+              "llama.attention.layer_norm_rms_epsilon": float(self.rms_norm_eps),
+              "llama.rope.freq_base": float(self.rope_theta), "llama.vocab_size": self.vocab_size}
+        if self.head_dim * self.num_attention_heads != self.hidden_size:
+            md["llama.attention.key_length"] = self.head_dim
+        if self.bos_token_id is not None:
+            md["tokenizer.ggml.bos_token_id"] = int(self.bos_token_id)
+        if self.eos_token_ids:
+            md["tokenizer.ggml.eos_token_id"] = int(self.eos_token_ids[0])
+        return md
+
+    @staticmethod
+    def gguf_tensor_name(name: str) -> str:
+        """This library's tensor name (the config.json world's) -> the GGUF name the reference binds
+        (src/model/model.cpp:25-38, src/model/block.cpp:18-62)."""
+        fixed = {"model.embed_tokens.weight": "token_embd.weight", "model.norm.weight": "output_norm.weight",
+                 "lm_head.weight": "output.weight"}
+        if name in fixed:
+            return fixed[name]
+        parts = {"input_layernorm": "attn_norm", "post_attention_layernorm": "ffn_norm",
+                 "self_attn.q_proj": "attn_q", "self_attn.k_proj": "attn_k", "self_attn.v_proj": "attn_v",
+                 "self_attn.o_proj": "attn_output", "mlp.gate_proj": "ffn_gate", "mlp.up_proj": "ffn_up",
+                 "mlp.down_proj": "ffn_down"}
+        head = "model.layers."
+        if name.startswith(head) and name.endswith(".weight"):
+            layer, _, rest = name[len(head):-len(".weight")].partition(".")
+            if rest in parts and layer.isdigit():
+                return f"blk.{layer}.{parts[rest]}.weight"
+        return name
+
     @classmethod
     def from_folder(cls, folder: str) -> "LlamaConfig":
         with open(os.path.join(folder, "config.json")) as f:

@@ -47,7 +47,7 @@ class Engine:
         _require_gpu()
         config = config_from_folder(folder)
         model = DecoderModel(config.model_spec(), as_dtype(dtype), device)
-        load_into(model, folder)
+        load_into(model, folder, config)
         return cls(config, model, max_tokens, n_slots)
 
     @classmethod

@@ -67,9 +67,42 @@ def config_from_dict(raw: dict):
     return ARCHITECTURES[name].from_dict(raw)
 
 
+def find_gguf(path: str):
+    """The GGUF file that ``path`` names: the file itself, or the only ``*.gguf`` of a folder."""
+    if os.path.isfile(path) and path.endswith(".gguf"):
+        return path
+    if os.path.isdir(path):
+        found = sorted(f for f in os.listdir(path) if f.endswith(".gguf"))
+        if len(found) == 1:
+            return os.path.join(path, found[0])
+        if len(found) > 1:
+            raise ConfigError(f"{path} holds several GGUF files ({', '.join(found)}): name one")
+    return None
+
+
 def config_from_folder(folder: str):
+    """The configuration of a model folder (config.json), or of a GGUF file or the folder that
+    holds one (the reference's own model format: its metadata is the configuration)."""
     path = os.path.join(folder, "config.json")
-    if not os.path.isfile(path):
+    if os.path.isfile(path):
+        with open(path) as f:
+            return config_from_dict(json.load(f))
+    gguf = find_gguf(folder)
+    if gguf is None:
         raise ConfigError(f"no config.json in {folder}")
-    with open(path) as f:
-        return config_from_dict(json.load(f))
+    from .weights.gguf_io import GGUFFile
+    f = GGUFFile(gguf)
+    arch = f.metadata.get("general.architecture")
+    if arch is None:
+        raise ConfigError("Missing required metadata: general.architecture")      # src/gguf.cpp:219-223
+    for cls in ARCHITECTURES.values():
+        if getattr(cls, "gguf_architecture", None) == arch and hasattr(cls, "from_gguf"):
+            shapes = {}
+            for n in f.names():
+                try:
+                    shapes[n] = f.info(n)[1]
+                except ValueError:
+                    shapes[n] = None                # a tensor type that is not read: the loader will say so
+            return cls.from_gguf(f.metadata, shapes)
+    known = sorted({getattr(c, "gguf_architecture", None) for c in ARCHITECTURES.values()} - {None})
+    raise ConfigError(f"unknown GGUF architecture {arch!r}; known: " + ", ".join(known))

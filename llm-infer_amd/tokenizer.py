@@ -41,6 +41,30 @@ class Tokenizer:
             vocab[t["content"]] = t["id"]
         return cls(vocab, bos_id, eos_id)
 
+    @classmethod
+    def from_gguf(cls, metadata: dict, bos_id=None, eos_id=None):
+        """The vocabulary a GGUF file carries (``tokenizer.ggml.tokens``, src/tokenizer.cpp:13-60)."""
+        tokens = metadata.get("tokenizer.ggml.tokens")
+        if tokens is None:
+            return None
+        if bos_id is None and "tokenizer.ggml.bos_token_id" in metadata:
+            bos_id = int(metadata["tokenizer.ggml.bos_token_id"])
+        if eos_id is None and "tokenizer.ggml.eos_token_id" in metadata:
+            eos_id = int(metadata["tokenizer.ggml.eos_token_id"])
+        return cls({str(t): i for i, t in enumerate(tokens)}, bos_id, eos_id)
+
+    @classmethod
+    def from_model(cls, path: str, bos_id=None, eos_id=None):
+        """tokenizer.json of a model folder, else the vocabulary inside its GGUF file."""
+        tok = cls.from_folder(path, bos_id, eos_id) if os.path.isdir(path) else None
+        if tok is None:
+            from .registry import find_gguf
+            gguf = find_gguf(path)
+            if gguf is not None:
+                from .weights.gguf_io import GGUFFile
+                tok = cls.from_gguf(GGUFFile(gguf).metadata, bos_id, eos_id)
+        return tok
+
     def encode(self, text: str, add_bos: bool = True) -> list:
         data = text.encode("utf-8")
         out = [self.bos_id] if add_bos and self.bos_id is not None else []

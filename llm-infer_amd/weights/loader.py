@@ -66,7 +66,37 @@ class Checkpoint:
         return self._where[name].tensor(name)
 
 
-def read_checkpoint(folder: str) -> Checkpoint:
+class GGUFCheckpoint:
+    """The tensors of a GGUF file under the names this library uses: ``rename`` maps a name of
+    the model's table to the name in the file (the configuration class knows it)."""
+
+    def __init__(self, path: str, needed, rename):
+        from .gguf_io import GGUFFile
+        self.file = GGUFFile(path)
+        self._to_file = {n: rename(n) for n in needed}
+        back = {v: k for k, v in self._to_file.items()}
+        self._names = [back.get(n, n) for n in self.file.names()]
+        self._to_file.update({n: n for n in self._names if n not in self._to_file})
+
+    def names(self) -> list:
+        return list(self._names)
+
+    def info(self, name: str):
+        return self.file.info(self._to_file[name])
+
+    def tensor(self, name: str) -> torch.Tensor:
+        return self.file.tensor(self._to_file[name])
+
+
+def read_checkpoint(folder: str, needed=(), config=None):
+    """A folder with safetensors, or a GGUF file (or the folder that holds one)."""
+    from ..registry import find_gguf
+    has_st = os.path.isdir(folder) and (os.path.isfile(os.path.join(folder, "model.safetensors")) or
+                                        os.path.isfile(os.path.join(folder, "model.safetensors.index.json")))
+    gguf = None if has_st else find_gguf(folder)
+    if gguf is not None:
+        rename = getattr(config, "gguf_tensor_name", None) or (lambda n: n)
+        return GGUFCheckpoint(gguf, needed, rename)
     return Checkpoint(folder)
 
 
@@ -112,10 +142,15 @@ def place_tensor(t: torch.Tensor, kind: str, compute: torch.dtype, device) -> to
     return t.to(device=device, dtype=kept_dtype(t.dtype, kind, compute)).contiguous()
 
 
-def load_into(model, folder: str) -> None:
+def load_into(model, folder: str, config=None) -> None:
     """Check the folder's tensors against ``model.params()`` and hand each part its tensors."""
-    ckpt = read_checkpoint(folder)
     needed = model.params()
-    check_tensors(needed, ckpt, model.ignorable_names())
+    ckpt = read_checkpoint(folder, needed, config)
+    ignorable = list(model.ignorable_names())
+    if isinstance(ckpt, GGUFCheckpoint):
+        # exported beside the weights by other tools; the reference binds tensors by name and never
+        # looks at it (frequency factors of a rotation scaling that neither it nor this library applies)
+        ignorable.append("rope_freqs.weight")
+    check_tensors(needed, ckpt, ignorable)
     model.bind({name: place_tensor(ckpt.tensor(name), spec.kind, model.dtype, model.device)
                 for name, spec in needed.items()})

@@ -61,3 +61,18 @@ def write_random_model(folder: str, config, seed: int, dtype: str = "bfloat16") 
         json.dump(raw, f, indent=1)
     write_safetensors(os.path.join(folder, "model.safetensors"),
                       random_tensors(model.params(), seed, matrix_dtype), {"format": "pt", "seed": seed})
+
+
+def write_random_gguf(path: str, config, seed: int, dtype: str = "float16", vocabulary=None) -> None:
+    """The same random model as one GGUF file (matrices float16 by default, norms float32), under
+    the tensor names and metadata keys the reference reads; ``vocabulary``: optional list of token
+    strings for ``tokenizer.ggml.tokens``."""
+    from ..engine.model import DecoderModel
+    from .gguf_io import write_gguf
+    matrix_dtype = {"bfloat16": torch.bfloat16, "float16": torch.float16, "float32": torch.float32}[dtype]
+    model = DecoderModel(config.model_spec(), dtype=torch.float32, device="cpu", allocate=False)
+    md = config.gguf_metadata()
+    if vocabulary is not None:
+        md["tokenizer.ggml.tokens"] = list(vocabulary)
+    tensors = random_tensors(model.params(), seed, matrix_dtype)
+    write_gguf(path, md, {config.gguf_tensor_name(n): t for n, t in tensors.items()})

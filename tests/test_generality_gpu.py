@@ -332,6 +332,32 @@ def test_command_line_generates_greedily(folders):
     assert bad.returncode == 1 and "Error:" in bad.stderr
 
 
+def test_a_gguf_file_runs_like_the_folder(lib, folders, tmp_path):
+    """The reference's own model format: the same weights as one GGUF file (its tensor names, its
+    metadata keys, a vocabulary inside) give the same logits as the folder, through the library
+    and through the command line with a text prompt."""
+    from llm_infer_amd.weights import write_gguf
+    cfg = lib.config_from_dict(TINY_B)
+    weights = P.load_weights(folders["B"])
+    path = str(tmp_path / "tiny.gguf")
+    vocab = [f"<{i}>" for i in range(cfg.vocab_size)]
+    vocab[65:91] = [chr(c) for c in range(65, 91)]                       # "A".."Z" are tokens 65..90
+    md = dict(cfg.gguf_metadata(), **{"tokenizer.ggml.tokens": vocab})
+    write_gguf(path, md, {cfg.gguf_tensor_name(n): (t.float() if t.dim() == 1 else t) for n, t in weights.items()})
+    prompt = [72, 69, 76, 76, 79]                                         # "HELLO"
+    a = lib.load(folders["B"], dtype="float32", max_tokens=256)
+    b = lib.load(path, dtype="float32", max_tokens=256)
+    la = a.step([a.alloc_slot()], [prompt], [list(range(5))])
+    lb = b.step([b.alloc_slot()], [prompt], [list(range(5))])
+    assert torch.equal(la, lb)
+    res = subprocess.run([sys.executable, os.path.join(ROOT, "bin", "infer"), path, "-i", "HELLO", "-n", "6",
+                          "-t", "0", "--dtype", "float32"], capture_output=True, text=True, timeout=300)
+    assert res.returncode == 0, res.stderr
+    got = [json.loads(line.split("tokens: ", 1)[1]) for line in res.stdout.splitlines() if " tokens: [" in line]
+    assert got == [P.generate_greedy(weights, TINY_B, prompt, 6)]
+    assert "Prompt tokens: 5" in res.stdout
+
+
 # ---------------------------------------------------------------------------
 # a toy architecture, defined here
 # ---------------------------------------------------------------------------
