@@ -1126,7 +1126,7 @@ extern "C" int li_gemv_tiled(const void* X, const void* Wt, int dt, void* C, int
     if (rc) return rc;
     const int n_tiles = (N + 15) / 16;
     const int mt = (M + 15) / 16;
-    if (nt <= 0) nt = mt >= 2 ? 2 : 1;
+    if (nt <= 0) nt = (mt >= 2 || (M > 12 && N >= 16384)) ? 2 : 1;           // measured on MI355X
     if (mt >= 3) nt = 2;
     const int blocks = (n_tiles + nt - 1) / nt;
     if (kw <= 0) kw = (K >= 8192 || blocks < 320 || blocks > 4096) ? 8 : 4;   // measured on MI355X
