@@ -31,8 +31,10 @@ Options:
   -T <int>              Context length override (default: model max)
   --seed <int>          Random seed (default: 0)
   --dtype <name>        bfloat16 (default), float16 or float32
-  --random-weights      Ignore model.safetensors: random weights from --seed-weights
+  --slots <int>         Most sequences that run as one batch (default: all requests given)
+  --random-weights      Ignore the model's tensors: random weights from --seed-weights
   --seed-weights <int>  Seed of the random weights (default: 0)
+  --config <json>       With --random-weights: the configuration file (the model argument is not opened)
   --no-graph            Launch every decode step kernel by kernel"""
 
 
@@ -43,7 +45,7 @@ def parse_ids(text: str) -> list:
 def parse_args(argv):
     cfg = dict(model=None, device="hip", prompt=None, prompt_file=None, tokens=[], tokens_file=None,
                max_tokens=256, temperature=1.0, seed=0, context=None, dtype="bfloat16", random=False,
-               seed_weights=0, graph=True, help=False)
+               seed_weights=0, graph=True, help=False, slots=None, config=None)
     if any(a in ("-h", "--help") for a in argv):
         cfg["help"] = True
         return cfg
@@ -52,7 +54,8 @@ def parse_args(argv):
     cfg["model"] = argv[0]
     takes = {"-d": ("device", str), "-i": ("prompt", str), "-f": ("prompt_file", str), "-n": ("max_tokens", int),
              "-t": ("temperature", float), "-T": ("context", int), "--seed": ("seed", int),
-             "--dtype": ("dtype", str), "--tokens-file": ("tokens_file", str), "--seed-weights": ("seed_weights", int)}
+             "--dtype": ("dtype", str), "--tokens-file": ("tokens_file", str), "--seed-weights": ("seed_weights", int),
+             "--slots": ("slots", int), "--config": ("config", str)}
     i = 1
     while i < len(argv):
         a = argv[i]
@@ -98,14 +101,23 @@ def run(cfg) -> int:
     from llm_infer_amd.engine import Engine
     from llm_infer_amd.tokenizer import Tokenizer
     print(f"Loading model: {cfg['model']}")
-    config = llm_infer_amd.config_from_folder(cfg["model"])
+    if cfg["config"]:
+        if not cfg["random"]:
+            raise RuntimeError("--config goes with --random-weights")
+        try:
+            with open(cfg["config"]) as f:
+                config = llm_infer_amd.config_from_dict(json.load(f))
+        except OSError:
+            raise RuntimeError(f"Failed to open configuration file: {cfg['config']}")
+    else:
+        config = llm_infer_amd.config_from_folder(cfg["model"])
     if cfg["context"]:
         raw = config.to_dict()
         raw["max_position_embeddings"] = cfg["context"]
         raw["eos_token_id"] = list(config.eos_token_ids) or None
         config = llm_infer_amd.config_from_dict(raw)
-    tok = Tokenizer.from_model(cfg["model"], config.bos_token_id,
-                               config.eos_token_ids[0] if config.eos_token_ids else None)
+    tok = None if cfg["config"] else Tokenizer.from_model(
+        cfg["model"], config.bos_token_id, config.eos_token_ids[0] if config.eos_token_ids else None)
     if cfg["prompt_file"]:
         try:
             with open(cfg["prompt_file"], encoding="utf-8") as f:
@@ -122,11 +134,17 @@ def run(cfg) -> int:
             prompts = [parse_ids(line) for line in f if line.strip()]
     else:
         prompts = cfg["tokens"]
-    need = sum(-(-min(len(p) + cfg["max_tokens"], config.max_position_embeddings) // 64) * 64 for p in prompts)
+    if cfg["slots"] is not None and cfg["slots"] <= 0:
+        raise RuntimeError("--slots must be positive")
+    n_slots = min(cfg["slots"] or len(prompts), len(prompts)) or 1
+    each = sorted((-(-min(len(p) + cfg["max_tokens"], config.max_position_embeddings) // 64) * 64 for p in prompts),
+                  reverse=True)
+    need = sum(each[:n_slots])                       # the largest batch that can be live at once
     if cfg["random"]:
-        engine = Engine.from_random(config, seed=cfg["seed_weights"], dtype=cfg["dtype"], max_tokens=need)
+        engine = Engine.from_random(config, seed=cfg["seed_weights"], dtype=cfg["dtype"], max_tokens=need,
+                                    n_slots=n_slots)
     else:
-        engine = Engine.from_folder(cfg["model"], dtype=cfg["dtype"], max_tokens=need)
+        engine = Engine.from_folder(cfg["model"], dtype=cfg["dtype"], max_tokens=need, n_slots=n_slots)
         engine.config = config
         if cfg["context"]:
             engine.max_positions = min(engine.max_positions, cfg["context"])

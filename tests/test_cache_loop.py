@@ -197,6 +197,9 @@ def test_command_line_follows_the_reference():
     assert parse_args(["m"]) is None and parse_args([]) is None
     assert parse_args(["m", "-i", "a", "-f", "b"]) is None and parse_args(["m", "-i", "a", "--bogus"]) is None
     assert parse_args(["m", "-i", "a", "-d", "cuda"]) is None and parse_args(["-h"])["help"]
+    c = parse_args(["-", "--tokens", "1", "--random-weights", "--config", "c.json", "--slots", "2", "--dtype", "float16"])
+    assert (c["random"], c["config"], c["slots"], c["dtype"]) == (True, "c.json", 2, "float16")
+    assert parse_args(["m", "--tokens", "1", "--slots", "two"]) is None
 
 
 def test_tokenizer_longest_match_and_bytes():

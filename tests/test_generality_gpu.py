@@ -330,6 +330,18 @@ def test_command_line_generates_greedily(folders):
     bad = subprocess.run([sys.executable, os.path.join(ROOT, "bin", "infer"), folder + "_nope", "--tokens", "1"],
                          capture_output=True, text=True, timeout=300)
     assert bad.returncode == 1 and "Error:" in bad.stderr
+    # two slots for three requests (two batches, the slots used again), random weights from a
+    # configuration file alone: the same tokens as the library gives for that seed
+    cmd = [sys.executable, os.path.join(ROOT, "bin", "infer"), "-", "--random-weights", "--seed-weights", "5",
+           "--config", os.path.join(folder, "config.json"), "--slots", "2", "-n", "6", "-t", "0", "--dtype", "float32"]
+    for p in prompts:
+        cmd += ["--tokens", ",".join(map(str, p))]
+    res = subprocess.run(cmd, capture_output=True, text=True, timeout=300)
+    assert res.returncode == 0, res.stderr
+    got = [json.loads(line.split("tokens: ", 1)[1]) for line in res.stdout.splitlines() if " tokens: [" in line]
+    import llm_infer_amd
+    eng = llm_infer_amd.random_model(llm_infer_amd.config_from_folder(folder), seed=5, dtype="float32", max_tokens=512)
+    assert got == eng.generate(prompts, max_new_tokens=6, temperature=0.0)
 
 
 def test_a_gguf_file_runs_like_the_folder(lib, folders, tmp_path):
