@@ -1,0 +1,165 @@
+// Shared by the matrix-product sources: the epilogues, the tiled-weight layout and the split-K
+// reduction.  (Included by gemm.hip and gemm_prefill.hip; every kernel here is static or inline.)
+#pragma once
+#include "common.h"
+
+enum { EPI_STORE = 0, EPI_ADD = 1, EPI_SWIGLU = 2, EPI_ROPE = 3 };
+
+// What the EPI_ROPE epilogue needs: the columns of the product are the q heads, then the k heads,
+// then the v heads of a token; q and k are rotated by the token's position (adjacent pairs), q goes
+// to q_out [M, H, hd], k and v into the token's cache page.
+struct RopeStore {
+    const float* inv_freq;      // [rotary_dim / 2]
+    const float* cos_sin;       // [M, rotary_dim / 2, 2] cos and sin of pos * inv_freq, or null
+    const int* pos;             // [M] position of each row
+    const int* tok_slot;        // [M] cache slot of each row
+    const int* page_table;      // [slots, max_pages]
+    void* q_out;
+    void* k_pages;
+    void* v_pages;
+    int64_t page_stride;
+    int rotary_dim, H, K, hd, max_pages, dt;   // dt: DT_* of q_out and the cache
+};
+
+struct Epilogue {
+    void* C;        // output (unused by EPI_ROPE)
+    int mode;       // EPI_*
+    int out_dt;     // DT_* of C (EPI_ADD: always float32)
+    int M, N;
+    RopeStore rs;
+};
+
+__device__ __forceinline__ void store_one(void* C, int dt, int64_t i, float v) {
+    if (dt == DT_F32) ((float*)C)[i] = v;
+    else if (dt == DT_F16) ((f16*)C)[i] = (f16)v;
+    else ((bf16*)C)[i] = (bf16)v;
+}
+
+// Offset of W[n, k] in the tiled order of a weight matrix (see "Tiled weights" in gemm.hip).
+__host__ __device__ __forceinline__ int64_t tiled_offset(int n, int k, int K) {
+    return ((((int64_t)(n >> 4) * (K >> 5) + (k >> 5)) * 64) + (((k & 31) >> 3) << 4) + (n & 15)) * 8 + (k & 7);
+}
+
+// v[0..3] are the results for row m and columns n..n+3 (n a multiple of 4).
+__device__ __forceinline__ void epilogue4(const Epilogue& e, int m, int n, const float* v) {
+    if (m >= e.M || n >= e.N) return;
+    if (e.mode == EPI_ROPE) {
+        // include/kernels_cpu.hpp:82-100 and src/model/block.cpp:141-148, on the accumulators
+        const RopeStore& r = e.rs;
+        const int head = n / r.hd, d = n - head * r.hd;       // the 4 columns lie in one head (hd % 16 == 0)
+        const int p = r.pos[m];
+        float o[4] = {v[0], v[1], v[2], v[3]};
+        if (head < r.H + r.K) {
+#pragma unroll
+            for (int j = 0; j < 4; j += 2) {
+                if (d + j < r.rotary_dim) {
+                    float sn, cs;
+                    if (r.cos_sin) {
+                        const f32x2 t = *(const f32x2*)(r.cos_sin + ((int64_t)m * (r.rotary_dim >> 1) + ((d + j) >> 1)) * 2);
+                        cs = t[0]; sn = t[1];
+                    } else sincosf((float)p * r.inv_freq[(d + j) >> 1], &sn, &cs);
+                    o[j] = v[j] * cs - v[j + 1] * sn;
+                    o[j + 1] = v[j] * sn + v[j + 1] * cs;
+                }
+            }
+        }
+        if (head < r.H) {
+            const int64_t at = ((int64_t)m * r.H + head) * r.hd + d;
+#pragma unroll
+            for (int j = 0; j < 4; ++j) store_one(r.q_out, r.dt, at + j, o[j]);
+        } else {
+            const int64_t page = r.page_table[(int64_t)r.tok_slot[m] * r.max_pages + p / PAGE];
+            const int tp = p % PAGE;
+            if (head < r.H + r.K) {
+                const int64_t at = page * r.page_stride + (int64_t)(head - r.H) * k_head_elems(r.hd);
+#pragma unroll
+                for (int j = 0; j < 4; ++j) store_one(r.k_pages, r.dt, at + k_offset(tp, d + j, r.hd), o[j]);
+            } else {
+                const int64_t at = page * r.page_stride + (int64_t)(head - r.H - r.K) * v_head_elems(r.hd);
+#pragma unroll
+                for (int j = 0; j < 4; ++j) store_one(r.v_pages, r.dt, at + v_offset(tp, d + j, r.hd), o[j]);
+            }
+        }
+        return;
+    }
+    if (e.mode == EPI_SWIGLU) {
+        // columns 2j (gate) and 2j+1 (up) give h[m, j] = silu(gate) * up   (src/model/block.cpp:209-213)
+        const int64_t row = (int64_t)m * (e.N >> 1);
+#pragma unroll
+        for (int j = 0; j < 4; j += 2) {
+            if (n + j + 1 < e.N) {
+                const float g = v[j], u = v[j + 1];
+                store_one(e.C, e.out_dt, row + ((n + j) >> 1), g / (1.f + expf(-g)) * u);
+            }
+        }
+        return;
+    }
+    const int64_t base = (int64_t)m * e.N + n;
+    const bool full = (n + 3 < e.N) && ((e.N & 3) == 0);
+    if (e.mode == EPI_ADD) {
+        float* c = (float*)e.C + base;
+        if (full) {
+            f32x4 o = *(f32x4*)c;
+            o[0] += v[0]; o[1] += v[1]; o[2] += v[2]; o[3] += v[3];
+            *(f32x4*)c = o;
+        } else {
+#pragma unroll
+            for (int j = 0; j < 4; ++j) if (n + j < e.N) c[j] += v[j];
+        }
+        return;
+    }
+    if (full && e.out_dt == DT_F32) {
+        f32x4 o = {v[0], v[1], v[2], v[3]};
+        *(f32x4*)((float*)e.C + base) = o;
+    } else if (full && e.out_dt == DT_F16) {
+        f16x4 o = {(f16)v[0], (f16)v[1], (f16)v[2], (f16)v[3]};
+        *(f16x4*)((f16*)e.C + base) = o;
+    } else if (full && e.out_dt == DT_BF16) {
+        bf16x4 o = {(bf16)v[0], (bf16)v[1], (bf16)v[2], (bf16)v[3]};
+        *(bf16x4*)((bf16*)e.C + base) = o;
+    } else {
+#pragma unroll
+        for (int j = 0; j < 4; ++j) if (n + j < e.N) store_one(e.C, e.out_dt, base + j, v[j]);
+    }
+}
+
+
+// Sum of the split-K partials in ascending split order, then the epilogue.
+static __global__ void splitk_reduce_kernel(const float* __restrict__ ws, int splits, Epilogue e) {
+    const int64_t quads_per_row = (e.N + 3) >> 2;
+    const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= quads_per_row * e.M) return;
+    const int m = (int)(i / quads_per_row), n = (int)(i % quads_per_row) * 4;
+    float v[4] = {0.f, 0.f, 0.f, 0.f};
+    for (int s = 0; s < splits; ++s) {
+        const float* p = ws + ((int64_t)s * e.M + m) * e.N + n;
+#pragma unroll
+        for (int q = 0; q < 4; ++q) if (n + q < e.N) v[q] += p[q];
+    }
+    epilogue4(e, m, n, v);
+}
+
+
+static int make_epilogue(Epilogue& e, void* C, int mode, int out_dt, int M, int N, const RopeStore* rs) {
+    e.C = C; e.mode = mode; e.out_dt = out_dt; e.M = M; e.N = N;
+    e.rs = RopeStore{};
+    if (mode != EPI_ROPE) return LI_OK;
+    if (!rs || !rs->pos || !rs->q_out || rs->hd <= 0 || rs->hd % 16 != 0 || rs->H <= 0 || rs->K < 0) return LI_BAD_ARG;
+    if (N != (rs->H + 2 * rs->K) * rs->hd || rs->rotary_dim < 0 || rs->rotary_dim > rs->hd || (rs->rotary_dim & 1))
+        return LI_BAD_ARG;
+    if (rs->rotary_dim > 0 && !rs->inv_freq && !rs->cos_sin) return LI_BAD_ARG;
+    if (rs->K > 0 && (!rs->tok_slot || !rs->page_table || !rs->k_pages || !rs->v_pages)) return LI_BAD_ARG;
+    if (rs->dt < DT_F32 || rs->dt > DT_BF16) return LI_BAD_ARG;
+    e.rs = *rs;
+    return LI_OK;
+}
+
+static int check_common(const void* X, const void* W, const void* C, int M, int N, int K, int mode, int out_dt) {
+    if (!X || !W || (!C && mode != EPI_ROPE) || M < 0 || N <= 0 || K <= 0) return LI_BAD_ARG;
+    if (mode < EPI_STORE || mode > EPI_ROPE) return LI_BAD_ARG;
+    if (out_dt < DT_F32 || out_dt > DT_BF16) return LI_BAD_ARG;
+    if (mode == EPI_ADD && out_dt != DT_F32) return LI_BAD_ARG;
+    if (mode == EPI_SWIGLU && (N & 1)) return LI_BAD_ARG;
+    return LI_OK;
+}
+

@@ -1,0 +1,470 @@
+// The prefill products: more than 96 rows of X (gemm_dma against a tiled weight, gemm_big against
+// a row-major one).  Epilogues, layouts and the split-K reduction are in gemm_common.h.
+#include "gemm_common.h"
+
+// Which tile a workgroup works on.  Workgroups go to the 8 XCDs in turn (workgroup L to XCD
+// L % 8) and every XCD has an L2 of its own, so the tiles are numbered such that an XCD works on
+// one contiguous run of them; within the run, groups of GM tiles of X go through all tiles of W
+// before the next group starts.  The workgroups that are resident on an XCD together (32 or 64)
+// then cover a near-square block of tiles and share its rows of X and W through that L2; with
+// the tiles of X simply fastest they would share one tile of W and stream all of X past it.
+__device__ __forceinline__ void tile_of_workgroup(int GM, int& bx, int& by, int& bz) {
+    const int gx = gridDim.x, gy = gridDim.y;
+    const int total = gx * gy * gridDim.z;
+    const int L = blockIdx.x + gx * (blockIdx.y + gy * blockIdx.z);
+    const int xcd = L & 7, per = total >> 3, rem = total & 7;
+    const int id = xcd * per + min(xcd, rem) + (L >> 3);
+    bz = id / (gx * gy);
+    const int in_split = id - bz * gx * gy;
+    const int group = in_split / (GM * gy), first = group * GM;
+    const int size = min(gx - first, GM);
+    const int in_group = in_split - group * GM * gy;
+    bx = first + in_group % size;
+    by = in_group / size;
+}
+
+// ===========================================================================
+// gemm_big: the prefill product.  BN rows of W x BM rows of X per workgroup of 4
+// waves (2 x 2), each wave a (BN/2) x (BM/2) tile of 32x32 blocks, BK = 64.  Two LDS
+// buffers: the next tile travels global -> registers while the matrix cores work on
+// the current one and is written to the other buffer afterwards, so there is one
+// barrier per tile.  With 256 x 256 tiles a wave issues 16 matrix instructions for
+// 8 LDS fragment reads.  W may be row-major or tiled.
+// ===========================================================================
+template <class T, int BN, int BM, int BK, bool TILED, bool EDGE>
+__global__ __launch_bounds__(256) void gemm_big_kernel(const T* __restrict__ X, const T* __restrict__ W,
+                                                       int K, int k_per_split, float* __restrict__ ws,
+                                                       Epilogue e) {
+    typedef typename Vec<T>::v8 v8;
+    constexpr int LD = BK + 8, CPR = BK / 8;             // chunks of 8 elements per tile row
+    constexpr int TN = BN / 2, TM = BM / 2;
+    constexpr int NB = TN / 32, MB = TM / 32;
+    constexpr int W_CHUNKS = BN * BK / 8 / 256, X_CHUNKS = BM * BK / 8 / 256;
+    constexpr int BUF = (BN + BM) * LD;                  // elements of one buffer
+    constexpr int KSTEPS = BK / 32;
+    extern __shared__ __attribute__((aligned(16))) unsigned char smem_raw[];
+    T* smem = (T*)smem_raw;
+
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int wn = wave & 1, wm = wave >> 1;
+    int bx, by, bz;
+    tile_of_workgroup(8, bx, by, bz);
+    const int m0 = bx * BM, n0 = by * BN;
+    const int n_limit = TILED ? ((e.N + 15) & ~15) : e.N;
+    const int kb = bz * k_per_split, ke = min(K, kb + k_per_split);   // this workgroup's share of K
+
+    f32x16 acc[NB][MB];
+#pragma unroll
+    for (int a = 0; a < NB; ++a)
+#pragma unroll
+        for (int b = 0; b < MB; ++b)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) acc[a][b][r] = 0.f;
+
+    // Where each of this thread's 16-byte chunks of a tile comes from and goes to.  Row-major
+    // W: CPR threads a row; tiled W: 64 threads a (16 rows x 32 k) block, as it lies in memory.
+    // Loads are unconditional (addresses clamped into the matrix) and masked afterwards, so that
+    // the loads of two tiles can be in flight at once.
+    const T* wsrc[W_CHUNKS];
+    const T* xsrc[X_CHUNKS];
+    int wdst[W_CHUNKS], xdst[X_CHUNKS], wkc[W_CHUNKS], xkc[X_CHUNKS];
+    bool wok[W_CHUNKS], xok[X_CHUNKS];
+#pragma unroll
+    for (int c = 0; c < W_CHUNKS; ++c) {
+        const int chunk = tid + c * 256;
+        const int row = TILED ? ((chunk / (64 * KSTEPS)) << 4) + (chunk & 15) : chunk / CPR;
+        wkc[c] = TILED ? (((chunk >> 6) % KSTEPS) << 5) + (((chunk >> 4) & 3) << 3) : (chunk % CPR) * 8;
+        wok[c] = n0 + row < n_limit;
+        const int n = min(n0 + row, n_limit - 1);
+        wsrc[c] = TILED ? W + tiled_offset(n, wkc[c], K) : W + (int64_t)n * K + wkc[c];
+        wdst[c] = row * LD + wkc[c];
+    }
+#pragma unroll
+    for (int c = 0; c < X_CHUNKS; ++c) {
+        const int chunk = tid + c * 256, row = chunk / CPR;
+        xkc[c] = (chunk % CPR) * 8;
+        xok[c] = m0 + row < e.M;
+        xsrc[c] = X + (int64_t)min(m0 + row, e.M - 1) * K + xkc[c];
+        xdst[c] = BN * LD + row * LD + xkc[c];
+    }
+    // loads are raw; the mask (rows beyond the matrix, k beyond K) is applied when the tile is
+    // written to LDS, so that nothing waits for a load before then
+    // (EDGE false: M, N and K are whole numbers of tiles and nothing is masked)
+    auto load_tile = [&](int k0, v8 (&rw)[W_CHUNKS], v8 (&rx)[X_CHUNKS]) {
+        const int64_t wstep = TILED ? (int64_t)(k0 >> 5) * 512 : k0;
+#pragma unroll
+        for (int c = 0; c < W_CHUNKS; ++c) {
+            const bool in = !EDGE || k0 + wkc[c] < ke;
+            rw[c] = *(const v8*)(wsrc[c] + (in ? wstep : 0));
+        }
+#pragma unroll
+        for (int c = 0; c < X_CHUNKS; ++c) {
+            const bool in = !EDGE || k0 + xkc[c] < ke;
+            rx[c] = *(const v8*)(xsrc[c] + (in ? k0 : 0));
+        }
+    };
+    auto store_tile = [&](T* buf, int k0, const v8 (&rw)[W_CHUNKS], const v8 (&rx)[X_CHUNKS]) {
+        const v8 z = {};
+#pragma unroll
+        for (int c = 0; c < W_CHUNKS; ++c)
+            *(v8*)(buf + wdst[c]) = (!EDGE || (wok[c] && k0 + wkc[c] < ke)) ? rw[c] : z;
+#pragma unroll
+        for (int c = 0; c < X_CHUNKS; ++c)
+            *(v8*)(buf + xdst[c]) = (!EDGE || (xok[c] && k0 + xkc[c] < ke)) ? rx[c] : z;
+    };
+    auto compute = [&](const T* buf) {
+        const T* sW = buf;
+        const T* sX = buf + BN * LD;
+#pragma unroll
+        for (int ks = 0; ks < BK; ks += 16) {
+            v8 a[NB], b[MB];
+            const int kk = ks + 8 * (lane >> 5);
+#pragma unroll
+            for (int i = 0; i < NB; ++i) a[i] = *(const v8*)(sW + (wn * TN + i * 32 + (lane & 31)) * LD + kk);
+#pragma unroll
+            for (int j = 0; j < MB; ++j) b[j] = *(const v8*)(sX + (wm * TM + j * 32 + (lane & 31)) * LD + kk);
+#pragma unroll
+            for (int i = 0; i < NB; ++i)
+#pragma unroll
+                for (int j = 0; j < MB; ++j) acc[i][j] = mfma32(a[i], b[j], acc[i][j]);
+        }
+    };
+
+    // Tile t is computed from LDS buffer t % 2 while tile t + 1 waits in registers and the loads
+    // of tile t + 2 are issued: a load has more than one tile's worth of matrix work to arrive.
+    const int n_tiles = (ke - kb + BK - 1) / BK;
+    v8 rw0[W_CHUNKS], rx0[X_CHUNKS], rw1[W_CHUNKS], rx1[X_CHUNKS];
+    T* buf0 = smem;
+    T* buf1 = smem + BUF;
+    // (Loads and stores past the last tile are not branched around: they fetch the last tile again
+    // and write it where nothing reads it, which keeps the count of loads in flight fixed.)
+    const int k_last = kb + (n_tiles - 1) * BK;
+    load_tile(kb, rw0, rx0);
+    store_tile(buf0, kb, rw0, rx0);
+    load_tile(min(kb + BK, k_last), rw1, rx1);
+    __syncthreads();
+    int t = 0;
+    for (; t + 1 < n_tiles; t += 2) {
+        // the scheduling barriers keep the loads at the head of each half and the LDS writes at
+        // its tail; left alone the compiler sinks the loads to just before their use
+        load_tile(min(kb + (t + 2) * BK, k_last), rw0, rx0);
+        __builtin_amdgcn_sched_barrier(0);
+        compute(buf0);
+        __builtin_amdgcn_sched_barrier(0);
+        store_tile(buf1, kb + (t + 1) * BK, rw1, rx1);
+        __syncthreads();
+        load_tile(min(kb + (t + 3) * BK, k_last), rw1, rx1);
+        __builtin_amdgcn_sched_barrier(0);
+        compute(buf1);
+        __builtin_amdgcn_sched_barrier(0);
+        store_tile(buf0, min(kb + (t + 2) * BK, k_last), rw0, rx0);
+        __syncthreads();
+    }
+    if (t < n_tiles) compute(buf0);
+    __syncthreads();
+    // Epilogue through LDS: a wave lays each 32x32 block down as [row of X][32 columns] and reads it
+    // back so that 8 lanes write 32 consecutive columns of one row; the loop over the block's
+    // quads is not unrolled, which keeps one copy of the epilogue in the code.
+    constexpr int SLD = 36;                                  // floats per staged row (padded)
+    float* stage = (float*)smem_raw + wave * (32 * SLD);
+#pragma unroll
+    for (int i = 0; i < NB; ++i)
+#pragma unroll
+        for (int j = 0; j < MB; ++j) {
+#pragma unroll
+            for (int g = 0; g < 4; ++g) {
+                f32x4 v = {acc[i][j][4 * g], acc[i][j][4 * g + 1], acc[i][j][4 * g + 2], acc[i][j][4 * g + 3]};
+                *(f32x4*)(stage + (lane & 31) * SLD + 8 * g + 4 * (lane >> 5)) = v;
+            }
+            __builtin_amdgcn_wave_barrier();
+            const int mb = m0 + wm * TM + j * 32, nb = n0 + wn * TN + i * 32;
+#pragma unroll 1
+            for (int q = lane; q < 256; q += 64) {
+                const int r = q >> 3, c = (q & 7) * 4;
+                const f32x4 v = *(const f32x4*)(stage + r * SLD + c);
+                const float vv[4] = {v[0], v[1], v[2], v[3]};
+                if (gridDim.z == 1) epilogue4(e, mb + r, nb + c, vv);
+                else if (mb + r < e.M) {                 // a share of K: the partial sums go to the workspace
+                    float* p = ws + ((int64_t)bz * e.M + mb + r) * e.N + nb + c;
+#pragma unroll
+                    for (int j = 0; j < 4; ++j) if (nb + c + j < e.N) p[j] = vv[j];
+                }
+            }
+            __builtin_amdgcn_wave_barrier();
+        }
+}
+
+// ===========================================================================
+// gemm_dma: the prefill product against a tiled W, with both operands going from global
+// memory straight into LDS (global_load_lds, 16 bytes a lane): no staging registers, no
+// LDS store instructions.  A load instruction of a wave fills 1 KiB of LDS in lane order,
+// so a tile lies in LDS as units of 16 rows x 32 elements of K in the order of the tiled
+// weight, [lane = 16*((k%32)/8) + row%16][k%8]: a unit of W is copied as it lies in
+// memory, a unit of X is gathered by the lanes (16 rows, 64 contiguous bytes each).  A
+// fragment of the 32x32x16 instruction is read from two such units, 16 lanes a contiguous
+// 256 bytes, which is free of bank conflicts without padding.  BK = 32 (K of a tiled weight
+// is a multiple of 32, so no tile is cut in K); rows beyond M or N are read from clamped
+// addresses and dropped by the epilogue.  Three LDS buffers: the loads of tile t + 2 are
+// issued while tile t is multiplied; one barrier per tile.
+// ===========================================================================
+template <class T, int BN, int BM, int WAVES, int STAGES>
+__global__ __launch_bounds__(64 * WAVES) void gemm_dma_kernel(const T* __restrict__ X, const T* __restrict__ Wt,
+                                                          int K, int k_per_split, float* __restrict__ ws,
+                                                          Epilogue e) {
+    typedef typename Vec<T>::v8 v8;
+    constexpr int BK = 32;
+    constexpr int TN = BN / 2, TM = BM / (WAVES / 2), NB = TN / 32, MB = TM / 32;   // 2 waves along N
+    constexpr int WU = BN / 16, XU = BM / 16, UNITS = WU + XU;       // 1 KiB units of a stage
+    constexpr int PER_WAVE = UNITS / WAVES;
+    constexpr int STAGE = UNITS * 1024;                              // bytes
+    static_assert(UNITS % WAVES == 0, "units of a stage are dealt to the waves");
+    extern __shared__ __attribute__((aligned(16))) unsigned char smem_raw[];
+
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);       // uniform: what depends on it stays scalar
+    const int wn = wave & 1, wm = wave >> 1;
+    int bx, by, bz;
+    tile_of_workgroup(BM == 256 ? 4 : 8, bx, by, bz);
+    const int m0 = bx * BM, n0 = by * BN;
+    const int kb = bz * k_per_split, ke = min(K, kb + k_per_split);
+    const int n_tiles = (ke - kb) / BK;
+    const int w_blocks = (e.N + 15) >> 4, steps = K >> 5;
+
+    // Where the 16 bytes of this lane come from, for each of the wave's units: a base address that
+    // is the same for the whole wave and moves on by `step` bytes per tile of K, plus a 32-bit
+    // offset of the lane (the host checks that X has fewer than 4 GiB).
+    const unsigned char* base[PER_WAVE];
+    uint32_t lane_off[PER_WAVE];
+    int step[PER_WAVE];
+#pragma unroll
+    for (int i = 0; i < PER_WAVE; ++i) {
+        const int u = wave * PER_WAVE + i;
+        if (u < WU) {
+            const int blk = min(n0 / 16 + u, w_blocks - 1);
+            base[i] = (const unsigned char*)(Wt + ((int64_t)blk * steps + (kb >> 5)) * 512);
+            lane_off[i] = lane * 16;
+            step[i] = 1024;
+        } else {
+            const int row = min(m0 + 16 * (u - WU) + (lane & 15), e.M - 1);
+            base[i] = (const unsigned char*)(X + kb);
+            lane_off[i] = ((uint32_t)row * (uint32_t)K + 8 * (lane >> 4)) * 2;
+            step[i] = BK * 2;
+        }
+    }
+    auto issue = [&](int t, int buf) {
+#pragma unroll
+        for (int i = 0; i < PER_WAVE; ++i) {
+            const int u = wave * PER_WAVE + i;
+            __builtin_amdgcn_global_load_lds(
+                (const __attribute__((address_space(1))) void*)(base[i] + (int64_t)t * step[i] + lane_off[i]),
+                (__attribute__((address_space(3))) void*)(smem_raw + buf * STAGE + u * 1024), 16, 0, 0);
+        }
+    };
+
+    f32x16 acc[NB][MB];
+#pragma unroll
+    for (int a = 0; a < NB; ++a)
+#pragma unroll
+        for (int b = 0; b < MB; ++b)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) acc[a][b][r] = 0.f;
+
+    // byte offset of this lane's piece of a fragment within its pair of units, for k-step 0
+    const int frag = ((lane & 31) >> 4) * 1024 + (16 * (lane >> 5) + (lane & 15)) * 16;
+    const unsigned char* sW = smem_raw + (wn * TN / 16) * 1024 + frag;
+    const unsigned char* sX = smem_raw + (WU + wm * TM / 16) * 1024 + frag;
+    auto read_frags = [&](int buf, int ks, v8 (&a)[NB], v8 (&b)[MB]) {
+#pragma unroll
+        for (int j = 0; j < MB; ++j) b[j] = *(const v8*)(sX + buf * STAGE + j * 2048 + ks * 512);
+#pragma unroll
+        for (int i = 0; i < NB; ++i) a[i] = *(const v8*)(sW + buf * STAGE + i * 2048 + ks * 512);
+    };
+    auto multiply = [&](const v8 (&a)[NB], const v8 (&b)[MB], int lo, int hi) {
+#pragma unroll
+        for (int i = 0; i < NB; ++i)
+            if (i >= lo && i < hi) {
+#pragma unroll
+                for (int j = 0; j < MB; ++j) acc[i][j] = mfma32(a[i], b[j], acc[i][j]);
+            }
+    };
+
+    // The loop works in half tiles (16 of the 32 elements of K): while the matrix cores work on
+    // one half, the fragments of the next are on their way from LDS.  In the middle of tile t every
+    // wave has read all of it, so the barrier there both publishes tile t + 1 and frees the buffer
+    // of tile t for the loads of tile t + STAGES: loads run STAGES - 1 tiles ahead.
+    // (A bare s_barrier: __syncthreads would also wait for the loads still in flight.)
+    // One copy of the body, the buffer a run-time offset: unrolled by the three buffers the
+    // register allocator spills.  After the last tile the reads for "the next tile" fetch stale
+    // data that nothing uses.
+    v8 a0[NB], b0[MB], a1[NB], b1[MB];
+    // waits until at most `tiles` of the tiles whose loads were issued last are still in flight
+    auto wait_tiles = [&](int tiles, bool lds_too) {
+        if (lds_too) {
+            if (tiles <= 0) __builtin_amdgcn_s_waitcnt(0x0070);
+            else if (tiles == 1) __builtin_amdgcn_s_waitcnt(0x0070 | PER_WAVE);
+            else if (tiles == 2) __builtin_amdgcn_s_waitcnt(0x0070 | (2 * PER_WAVE));
+            else __builtin_amdgcn_s_waitcnt(0x0070 | (3 * PER_WAVE));
+        } else {
+            if (tiles <= 0) __builtin_amdgcn_s_waitcnt(0x0F70);
+            else if (tiles == 1) __builtin_amdgcn_s_waitcnt(0x0F70 | PER_WAVE);
+            else if (tiles == 2) __builtin_amdgcn_s_waitcnt(0x0F70 | (2 * PER_WAVE));
+            else if (tiles == 3) __builtin_amdgcn_s_waitcnt(0x0F70 | (3 * PER_WAVE));
+            else __builtin_amdgcn_s_waitcnt(0x0F70 | (3 * PER_WAVE));
+        }
+    };
+    static_assert(STAGES >= 3 && STAGES <= 5 && (STAGES - 2) * PER_WAVE <= 15, "stages");
+#pragma unroll
+    for (int i = 0; i < STAGES; ++i)
+        if (i < n_tiles) issue(i, i);
+    wait_tiles(min(min(STAGES, n_tiles) - 1, 3), false);
+    __builtin_amdgcn_s_barrier();
+    read_frags(0, 0, a0, b0);
+    int cur = 0;
+#pragma unroll 1
+    for (int t = 0; t < n_tiles; ++t) {
+        const int nxt = cur == STAGES - 1 ? 0 : cur + 1;
+        // the second half's fragments are requested between the matrix instructions of the first
+        // half: requested before them, the wait the compiler places for the first half's fragments
+        // (it merges the loop's entry and back edge pessimistically) would cover these reads too
+        multiply(a0, b0, 0, NB / 2);
+        __builtin_amdgcn_sched_barrier(0);
+        read_frags(cur, 1, a1, b1);
+        __builtin_amdgcn_sched_barrier(0);
+        multiply(a0, b0, NB / 2, NB);
+        __builtin_amdgcn_sched_barrier(0);
+        // tile t + 1 has landed (up to STAGES - 2 later ones may be in flight); this wave's reads
+        // of tile t are done
+        wait_tiles(min(STAGES - 2, n_tiles - 2 - t), true);
+        __builtin_amdgcn_s_barrier();
+        if (t + STAGES < n_tiles) issue(t + STAGES, cur);
+        multiply(a1, b1, 0, NB / 2);
+        __builtin_amdgcn_sched_barrier(0);
+        read_frags(nxt, 0, a0, b0);
+        __builtin_amdgcn_sched_barrier(0);
+        multiply(a1, b1, NB / 2, NB);
+        __builtin_amdgcn_sched_barrier(0);
+        cur = nxt;
+    }
+    __syncthreads();
+    constexpr int SLD = 36;
+    float* stage = (float*)smem_raw + wave * (32 * SLD);
+#pragma unroll
+    for (int i = 0; i < NB; ++i)
+#pragma unroll
+        for (int j = 0; j < MB; ++j) {
+#pragma unroll
+            for (int g = 0; g < 4; ++g) {
+                f32x4 v = {acc[i][j][4 * g], acc[i][j][4 * g + 1], acc[i][j][4 * g + 2], acc[i][j][4 * g + 3]};
+                *(f32x4*)(stage + (lane & 31) * SLD + 8 * g + 4 * (lane >> 5)) = v;
+            }
+            __builtin_amdgcn_wave_barrier();
+            const int mb = m0 + wm * TM + j * 32, nb = n0 + wn * TN + i * 32;
+#pragma unroll 1
+            for (int q = lane; q < 256; q += 64) {
+                const int r = q >> 3, c = (q & 7) * 4;
+                const f32x4 v = *(const f32x4*)(stage + r * SLD + c);
+                const float vv[4] = {v[0], v[1], v[2], v[3]};
+                if (gridDim.z == 1) epilogue4(e, mb + r, nb + c, vv);
+                else if (mb + r < e.M) {
+                    float* p = ws + ((int64_t)bz * e.M + mb + r) * e.N + nb + c;
+#pragma unroll
+                    for (int jj = 0; jj < 4; ++jj) if (nb + c + jj < e.N) p[jj] = vv[jj];
+                }
+            }
+            __builtin_amdgcn_wave_barrier();
+        }
+}
+
+// ===========================================================================
+// C interface
+// ===========================================================================
+// tile (rows of W x rows of X / depth): 0 = 128x128/64, 1 = 256x128/32
+extern "C" int li_gemm_big(const void* X, const void* W, int tiled, int dt, void* C, int out_dt, int mode,
+                           int M, int N, int K, int tile, int splits, float* ws, const RopeStore* rs,
+                           hipStream_t stream) {
+    int rc = check_common(X, W, C, M, N, K, mode, out_dt);
+    if (rc) return rc;
+    if (dt != DT_F16 && dt != DT_BF16) return LI_BAD_ARG;
+    if (K % 8 != 0 || ((uintptr_t)X & 15) || ((uintptr_t)W & 15)) return LI_UNSUPPORTED;
+    if (tiled && K % 32 != 0) return LI_UNSUPPORTED;
+    if (tile < 0 || tile > 1) return LI_BAD_ARG;
+    if (splits < 1 || (splits > 1 && !ws)) return LI_BAD_ARG;
+    if (M == 0) return LI_OK;
+    Epilogue e;
+    rc = make_epilogue(e, C, mode, out_dt, M, N, rs);
+    if (rc) return rc;
+    const int bn = tile ? 256 : 128, bm = 128, bk = tile ? 32 : 64;
+    const size_t lds = (size_t)2 * (bn + bm) * (bk + 8) * 2;
+    int k_per_split = ((K + splits - 1) / splits + bk - 1) / bk * bk;
+    splits = (K + k_per_split - 1) / k_per_split;
+    dim3 grid((M + bm - 1) / bm, (N + bn - 1) / bn, splits), block(256);
+    const bool edge = (M % bm) || (N % bn) || (K % bk);
+#define GO(T, BN, BM, BK, TL)                                                                          \
+    do {                                                                                               \
+        auto kfn = edge ? gemm_big_kernel<T, BN, BM, BK, TL, true> : gemm_big_kernel<T, BN, BM, BK, TL, false>; \
+        if (hipFuncSetAttribute((const void*)kfn, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds) != hipSuccess) \
+            return LI_HIP_ERROR;                                                                       \
+        kfn<<<grid, block, lds, stream>>>((const T*)X, (const T*)W, K, k_per_split, ws, e);            \
+    } while (0)
+#define LAUNCH(T)                                                                                     \
+    do {                                                                                              \
+        if (tile == 0) { if (tiled) GO(T, 128, 128, 64, true); else GO(T, 128, 128, 64, false); }     \
+        else { if (tiled) GO(T, 256, 128, 32, true); else GO(T, 256, 128, 32, false); }               \
+    } while (0)
+    if (dt == DT_F16) LAUNCH(f16); else LAUNCH(bf16);
+#undef LAUNCH
+#undef GO
+    LI_CHECK_LAUNCH();
+    if (splits > 1) {
+        const int64_t quads = (int64_t)M * ((N + 3) / 4);
+        splitk_reduce_kernel<<<(unsigned)((quads + 255) / 256), 256, 0, stream>>>(ws, splits, e);
+        LI_CHECK_LAUNCH();
+    }
+    return LI_OK;
+}
+
+// tile: 0 = 128 x 128, 1 = 256 x 128, 2 = 256 x 256 with 8 waves (rows of W x rows of X); BK = 32; W tiled
+extern "C" int li_gemm_dma(const void* X, const void* Wt, int dt, void* C, int out_dt, int mode,
+                           int M, int N, int K, int tile, int splits, float* ws, const RopeStore* rs,
+                           hipStream_t stream) {
+    int rc = check_common(X, Wt, C, M, N, K, mode, out_dt);
+    if (rc) return rc;
+    if (dt != DT_F16 && dt != DT_BF16) return LI_BAD_ARG;
+    if (K % 32 != 0 || ((uintptr_t)X & 15) || ((uintptr_t)Wt & 15)) return LI_UNSUPPORTED;
+    if (tile < 0 || tile > 2) return LI_BAD_ARG;
+    if ((int64_t)M * K * 2 >= ((int64_t)1 << 32)) return LI_UNSUPPORTED;     // 32-bit offsets into X
+    if (splits < 1 || (splits > 1 && !ws)) return LI_BAD_ARG;
+    if (M == 0) return LI_OK;
+    Epilogue e;
+    rc = make_epilogue(e, C, mode, out_dt, M, N, rs);
+    if (rc) return rc;
+    const int bn = tile ? 256 : 128, bm = tile == 2 ? 256 : 128, bk = 32;
+    const size_t lds = (size_t)3 * (bn + bm) / 16 * 1024;
+    int k_per_split = ((K + splits - 1) / splits + bk - 1) / bk * bk;
+    splits = (K + k_per_split - 1) / k_per_split;
+    dim3 grid((M + bm - 1) / bm, (N + bn - 1) / bn, splits), block(tile == 2 ? 512 : 256);
+#define GO(T, BN, BM, WV, ST)                                                                                \
+    do {                                                                                               \
+        auto kfn = gemm_dma_kernel<T, BN, BM, WV, ST>;                                                 \
+        if (hipFuncSetAttribute((const void*)kfn, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds) != hipSuccess) \
+            return LI_HIP_ERROR;                                                                       \
+        kfn<<<grid, block, lds, stream>>>((const T*)X, (const T*)Wt, K, k_per_split, ws, e);           \
+    } while (0)
+#define LAUNCH(T)                                    \
+    do {                                             \
+        if (tile == 0) GO(T, 128, 128, 4, 3);        \
+        else if (tile == 1) GO(T, 256, 128, 4, 3);   \
+        else GO(T, 256, 256, 8, 3);                  \
+    } while (0)
+    if (dt == DT_F16) LAUNCH(f16); else LAUNCH(bf16);
+#undef LAUNCH
+#undef GO
+    LI_CHECK_LAUNCH();
+    if (splits > 1) {
+        const int64_t quads = (int64_t)M * ((N + 3) / 4);
+        splitk_reduce_kernel<<<(unsigned)((quads + 255) / 256), 256, 0, stream>>>(ws, splits, e);
+        LI_CHECK_LAUNCH();
+    }
+    return LI_OK;
+}
+

@@ -22,9 +22,9 @@ from concurrent.futures import ThreadPoolExecutor
 
 CSRC = os.path.join(os.path.dirname(os.path.dirname(os.path.abspath(__file__))), "csrc")
 ARCH = "gfx950"
-CORE_SOURCES = ("elementwise.hip", "gemm.hip", "sampling.hip")
+CORE_SOURCES = ("elementwise.hip", "gemm.hip", "gemm_prefill.hip", "sampling.hip")
 ATTN_SOURCE = "attention.hip"
-HEADERS = ("common.h",)
+HEADERS = ("common.h", "gemm_common.h")
 FLAGS = ["--offload-arch=" + ARCH, "-O3", "-std=c++17", "-fPIC",
          "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops", "-Wno-unused-command-line-argument"]
 
