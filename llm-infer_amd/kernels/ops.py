@@ -25,7 +25,14 @@ def _ptr(t):
     return c_void_p(t.data_ptr()) if t is not None else c_void_p(0)
 
 
+_raw_stream = getattr(torch._C, "_cuda_getCurrentRawStream", None)
+
+
 def _stream():
+    """The current HIP stream of the current device (looked up for every launch: a graph is
+    recorded on a stream of its own)."""
+    if _raw_stream is not None:
+        return c_void_p(_raw_stream(torch.cuda.current_device()))
     return c_void_p(torch.cuda.current_stream().cuda_stream)
 
 
@@ -128,7 +135,7 @@ _ws_retired: list = []
 def _workspace(n_floats: int, device) -> torch.Tensor:
     """Scratch for split-K partial sums, one per device and stream.  A workspace that has become
     too small is kept alive beside its larger successor: a captured graph may still write to it."""
-    key = (device, torch.cuda.current_stream().cuda_stream)
+    key = (device, _stream().value)
     ws = _ws_cache.get(key)
     if ws is None or ws.numel() < n_floats:
         if ws is not None:
