@@ -734,3 +734,131 @@ def test_toy_routed_feed_forward_and_another_position_encoding(lib, dtype):
     a = eng.generate([seqs[1], seqs[0]], max_new_tokens=6, temperature=0.0, use_graph=True)
     b = eng.generate([seqs[1], seqs[0]], max_new_tokens=6, temperature=0.0, use_graph=False)
     assert a == b and all(len(o) == 6 for o in a)
+
+
+# ---------------------------------------------------------------------------
+# a toy norm and a toy arrangement of a block, both defined here
+# ---------------------------------------------------------------------------
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_toy_norm_and_parallel_block(lib, dtype):
+    """A norm with mean and bias (LayerNorm) and a block whose mixer and feed-forward both read the
+    same normed input (parallel residual): registered from here, chosen by a configuration, run
+    whole, cut and through generation, against a float64 reference of the same toy model."""
+    from llm_infer_amd.config.spec import LayerSpec, ModelSpec, PartSpec, ScheduleEntry
+    from llm_infer_amd.engine import Engine
+    from llm_infer_amd.parts.base import Part
+    from llm_infer_amd.weights.loader import ParamSpec
+
+    @lib.register_norm("toy_layernorm")
+    class LayerNorm(Part):
+        def __init__(self, *, size, eps, prefix, dtype, device):
+            self.size, self.eps, self.prefix, self.dtype = size, eps, prefix, dtype
+
+        def params(self):
+            return {"weight": ParamSpec((self.size,), "vector", "ones"), "bias": ParamSpec((self.size,), "vector")}
+
+        def bind(self, tensors):
+            self.weight, self.bias = tensors["weight"], tensors["bias"]
+
+        def forward(self, x, rows=None):
+            if rows is not None:
+                x = x[rows.long()]
+            y = torch.nn.functional.layer_norm(x, (self.size,), self.weight, self.bias, self.eps)   # float32
+            return y.to(self.dtype)
+
+    @lib.register_block("toy_parallel")
+    class ParallelBlock(Part):
+        """x += mixer(n(x)) + feed_forward(n(x)) with one norm; the second norm of the spec is unused."""
+
+        def __init__(self, mixer_norm, mixer, feed_forward_norm, feed_forward):
+            self.norm, self.mixer, self.feed_forward = mixer_norm, mixer, feed_forward
+
+        def children(self):
+            return [self.norm, self.mixer, self.feed_forward]
+
+        def forward(self, x, ctx, cache_view, owns_cache=True):
+            h = self.norm.forward(x)
+            self.mixer.forward(h, ctx, cache_view, x, owns_cache)
+            self.feed_forward.forward(h, x)
+
+    class ParallelConfig:
+        def __init__(self, raw):
+            self.raw = raw
+
+        @classmethod
+        def from_dict(cls, raw):
+            return cls(raw)
+
+        def model_spec(self):
+            r = self.raw
+            d, hd = r["width"], r["head"]
+            layers = []
+            for i in range(r["layers"]):
+                norm = PartSpec("toy_layernorm", {"size": d, "eps": r["eps"]}, f"h.{i}.ln.")
+                mix = PartSpec("attention", {"hidden_size": d, "n_heads": 4, "n_kv_heads": 2, "head_dim": hd,
+                                             "scale": hd ** -0.5}, f"h.{i}.attn.")
+                ffn = PartSpec("gated_mlp", {"hidden_size": d, "intermediate_size": r["ffn"]}, f"h.{i}.mlp.")
+                pos = PartSpec("rope", {"theta": 777.0, "rotary_dim": hd // 2, "head_dim": hd})
+                layers.append(LayerSpec("toy_parallel", mix, ffn, norm, norm, pos))
+            return ModelSpec(d, r["vocab"], r["positions"],
+                             PartSpec("embedding", {"vocab_size": r["vocab"], "hidden_size": d}, "wte."),
+                             tuple(layers), tuple(ScheduleEntry(i) for i in range(r["layers"])),
+                             PartSpec("toy_layernorm", {"size": d, "eps": r["eps"]}, "ln_f."),
+                             PartSpec("lm_head", {"vocab_size": r["vocab"], "hidden_size": d, "tied": True}, "head."))
+
+    lib.register_architecture("ParallelToyForCausalLM", ParallelConfig)
+    raw = {"architectures": ["ParallelToyForCausalLM"], "width": 96, "head": 32, "ffn": 120, "eps": 1e-5,
+           "vocab": 90, "positions": 512, "layers": 2}
+    eng = Engine.from_random(lib.config_from_dict(raw), seed=8, dtype=dtype, max_tokens=1024)
+    model = Engine.from_random(lib.config_from_dict(raw), seed=8, dtype="float32", max_tokens=64).model
+    for m_ in (eng.model, model):                       # biases that matter
+        for part in [b.norm for b in m_.layers] + [m_.final_norm]:
+            part.bias += 0.1 * torch.arange(96, device=part.bias.device, dtype=torch.float32).cos()
+
+    def dbl(t):
+        return t.double().cpu()
+
+    def layernorm(x, part):
+        mu = x.mean(-1, keepdim=True)
+        var = ((x - mu) ** 2).mean(-1, keepdim=True)
+        return (x - mu) / torch.sqrt(var + 1e-5) * dbl(part.weight) + dbl(part.bias)
+
+    def ref_forward(toks):
+        n = len(toks)
+        x = dbl(model.embedding.weight)[toks]
+        posn = torch.arange(n)
+        for layer in model.layers:
+            att, ffn = layer.mixer, layer.feed_forward
+            h = layernorm(x, layer.norm)
+            wq, wk, wv = dbl(att.wqkv).split([128, 64, 64])
+            q = P.rope((h @ wq.t()).view(n, 4, 32), posn, 777.0, 16)
+            k = P.rope((h @ wk.t()).view(n, 2, 32), posn, 777.0, 16)
+            a = P.attention(q, k, (h @ wv.t()).view(n, 2, 32)).reshape(n, 128) @ dbl(att.wo).t()
+            gu = dbl(ffn.w_gate_up)
+            x = x + a + P.swiglu(h, gu[0::2], gu[1::2], dbl(ffn.w_down))
+        return layernorm(x, model.final_norm) @ dbl(model.embedding.weight).t()
+
+    g = torch.Generator().manual_seed(2)
+    seqs = [torch.randint(0, 90, (n,), generator=g).tolist() for n in (150, 3, 66)]
+    refs = [ref_forward(t) for t in seqs]
+    tol = 3e-5 if dtype == "float32" else 4e-2
+    scale = 1 + max(r.abs().max().item() for r in refs)
+    slots = [eng.alloc_slot() for _ in seqs]
+    whole = eng.step(slots, seqs, [list(range(len(t))) for t in seqs]).double().cpu()
+    assert (whole - torch.cat(refs)).abs().max().item() < tol * scale
+    for s in slots:
+        eng.free_slot(s)
+    slots = [eng.alloc_slot() for _ in seqs]
+    heads = [len(t) - 2 for t in seqs]
+    eng.step(slots, [t[:h] for t, h in zip(seqs, heads)])
+    for kk in range(2):
+        out = eng.step(slots, [[t[h + kk]] for t, h in zip(seqs, heads)]).double().cpu()
+        for i, (r, h) in enumerate(zip(refs, heads)):
+            assert (out[i] - r[h + kk]).abs().max().item() < tol * scale
+    for s in slots:
+        eng.free_slot(s)
+    a = eng.generate(seqs, max_new_tokens=5, temperature=0.0, use_graph=True)
+    b = eng.generate(seqs, max_new_tokens=5, temperature=0.0, use_graph=False)
+    assert a == b
+    if dtype == "float32":
+        assert a[1][0] == int(refs[1][-1].argmax())
