@@ -149,3 +149,33 @@ def test_a_gguf_file_that_does_not_fit(tmp_path):
     msg = str(e.value)
     assert "model.layers.1.mlp.up_proj.weight" in msg and "extra.weight" in msg and "rope_freqs" not in msg
     assert "model.layers.0.self_attn.q_proj.weight: expected [64, 64], got [64, 56]" in msg
+
+
+def test_model_info_tells_what_a_folder_or_a_file_holds(tmp_path):
+    """The tool of the reference's tools/gguf_info.cpp and tools/hf_info.cpp: configuration, tensors,
+    tokenizer; exit status 1 and the loader's one error if the tensors do not fit."""
+    import io
+
+    from llm_infer_amd.info import describe, main
+    from safetensors.torch import load_file, save_file
+    cfg = llm_infer_amd.config_from_dict(dict(TINY_B, bos_token_id=1, eos_token_id=2))
+    folder, path = str(tmp_path / "m"), str(tmp_path / "m.gguf")
+    write_random_model(folder, cfg, 0)
+    vocab = ["<unk>", "<s>", "</s>"] + [f"t{i}" for i in range(cfg.vocab_size - 4)] + ["<|eot_id|>"]
+    write_random_gguf(path, cfg, 0, vocabulary=vocab)
+    for where, fmt in ((folder, "config.json + safetensors"), (path, "GGUF")):
+        out = io.StringIO()
+        assert describe(where, 3, out) == 0
+        text = out.getvalue()
+        assert fmt in text and f"hidden_size: {cfg.hidden_size}" in text and "The tensors fit the model." in text
+        assert f"Tensor count: {len(read_checkpoint(where, config=cfg).names())}" in text and "more" in text
+    out = io.StringIO()
+    describe(path, 0, out)
+    assert f"Tokenizer vocab size: {cfg.vocab_size}" in out.getvalue() and "BOS token ID: 1" in out.getvalue()
+    assert f"EOT token ID: {cfg.vocab_size - 1}" in out.getvalue()
+    tensors = load_file(os.path.join(folder, "model.safetensors"))
+    del tensors["model.norm.weight"]
+    save_file(tensors, os.path.join(folder, "model.safetensors"))
+    out = io.StringIO()
+    assert describe(folder, 0, out) == 1 and "missing tensors (1): model.norm.weight" in out.getvalue()
+    assert main([]) == 1 and main(["-h"]) == 0 and main([str(tmp_path / "nothing")]) == 1
