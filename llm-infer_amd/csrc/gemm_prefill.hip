@@ -210,7 +210,7 @@ __global__ __launch_bounds__(256) void gemm_big_kernel(const T* __restrict__ X, 
 template <class T, int BN, int BM, int WAVES, int STAGES>
 __global__ __launch_bounds__(64 * WAVES) void gemm_dma_kernel(const T* __restrict__ X, const T* __restrict__ Wt,
                                                           int K, int k_per_split, float* __restrict__ ws,
-                                                          Epilogue e) {
+                                                          int n_begin, Epilogue e) {
     typedef typename Vec<T>::v8 v8;
     constexpr int BK = 32;
     constexpr int TN = BN / 2, TM = BM / (WAVES / 2), NB = TN / 32, MB = TM / 32;   // 2 waves along N
@@ -225,7 +225,7 @@ __global__ __launch_bounds__(64 * WAVES) void gemm_dma_kernel(const T* __restric
     const int wn = wave & 1, wm = wave >> 1;
     int bx, by, bz;
     tile_of_workgroup(BM == 256 ? 4 : 8, bx, by, bz);
-    const int m0 = bx * BM, n0 = by * BN;
+    const int m0 = bx * BM, n0 = n_begin + by * BN;                  // the grid covers rows n_begin.. of W
     const int kb = bz * k_per_split, ke = min(K, kb + k_per_split);
     const int n_tiles = (ke - kb) / BK;
     const int w_blocks = (e.N + 15) >> 4, steps = K >> 5;
@@ -423,10 +423,13 @@ extern "C" int li_gemm_big(const void* X, const void* W, int tiled, int dt, void
     return LI_OK;
 }
 
-// tile: 0 = 128 x 128, 1 = 256 x 128, 2 = 256 x 256 with 8 waves (rows of W x rows of X); BK = 32; W tiled
+// tile: 0 = 128 x 128, 1 = 256 x 128, 2 = 256 x 256 with 8 waves (rows of W x rows of X); BK = 32; W tiled.
+//  The launch computes the columns n_begin .. n_begin + n_count - 1 of the product
+// (n_begin a multiple of 16; n_count 0: all from n_begin on), so that a product whose tiles do not
+// fill the last round of workgroups can finish with a smaller tile; K is split only for all columns.
 extern "C" int li_gemm_dma(const void* X, const void* Wt, int dt, void* C, int out_dt, int mode,
                            int M, int N, int K, int tile, int splits, float* ws, const RopeStore* rs,
-                           hipStream_t stream) {
+                           int n_begin, int n_count, hipStream_t stream) {
     int rc = check_common(X, Wt, C, M, N, K, mode, out_dt);
     if (rc) return rc;
     if (dt != DT_F16 && dt != DT_BF16) return LI_BAD_ARG;
@@ -434,21 +437,25 @@ extern "C" int li_gemm_dma(const void* X, const void* Wt, int dt, void* C, int o
     if (tile < 0 || tile > 2) return LI_BAD_ARG;
     if ((int64_t)M * K * 2 >= ((int64_t)1 << 32)) return LI_UNSUPPORTED;     // 32-bit offsets into X
     if (splits < 1 || (splits > 1 && !ws)) return LI_BAD_ARG;
+    if (n_begin < 0 || n_begin >= N || (n_begin & 15) || n_count < 0 || n_begin + n_count > N) return LI_BAD_ARG;
+    if (n_count == 0) n_count = N - n_begin;
+    const int bn = tile ? 256 : 128, bm = tile == 2 ? 256 : 128, bk = 32;
+    if (n_begin + n_count < N && n_count % bn != 0) return LI_BAD_ARG;       // only the last columns may end inside a tile
+    if (splits > 1 && n_count != N) return LI_BAD_ARG;
     if (M == 0) return LI_OK;
     Epilogue e;
     rc = make_epilogue(e, C, mode, out_dt, M, N, rs);
     if (rc) return rc;
-    const int bn = tile ? 256 : 128, bm = tile == 2 ? 256 : 128, bk = 32;
     const size_t lds = (size_t)3 * (bn + bm) / 16 * 1024;
     int k_per_split = ((K + splits - 1) / splits + bk - 1) / bk * bk;
     splits = (K + k_per_split - 1) / k_per_split;
-    dim3 grid((M + bm - 1) / bm, (N + bn - 1) / bn, splits), block(tile == 2 ? 512 : 256);
+    dim3 grid((M + bm - 1) / bm, (n_count + bn - 1) / bn, splits), block(tile == 2 ? 512 : 256);
 #define GO(T, BN, BM, WV, ST)                                                                                \
     do {                                                                                               \
         auto kfn = gemm_dma_kernel<T, BN, BM, WV, ST>;                                                 \
         if (hipFuncSetAttribute((const void*)kfn, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds) != hipSuccess) \
             return LI_HIP_ERROR;                                                                       \
-        kfn<<<grid, block, lds, stream>>>((const T*)X, (const T*)Wt, K, k_per_split, ws, e);           \
+        kfn<<<grid, block, lds, stream>>>((const T*)X, (const T*)Wt, K, k_per_split, ws, n_begin, e);  \
     } while (0)
 #define LAUNCH(T)                                    \
     do {                                             \

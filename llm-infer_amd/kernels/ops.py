@@ -198,12 +198,16 @@ def linear(x: torch.Tensor, w, mode: int = EPI_STORE, out: torch.Tensor | None =
     if kind.startswith("dma"):
         _need(tiled and fast_ok and m * k * 2 < (1 << 32), "gemm_dma: a tiled weight, X below 4 GiB")
         parts = kind.split(":")
-        tile, splits = _dma_shape(m, n, k)
-        if len(parts) > 1:
-            tile, splits = int(parts[1]), (int(parts[2]) if len(parts) > 2 else 1)
-        ws = _workspace(splits * m * n, x.device) if splits > 1 else None
-        _check(lib.li_gemm_dma(_ptr(x), _ptr(wd), DT[x.dtype], _ptr(out), out_dt, mode, m, n, k, tile, splits,
-                               _ptr(ws), rs, _stream()), "gemm_dma")
+        if parts[0] == "dma2":                             # "dma2:<tile>:<columns>:<tile of the rest>" for tests
+            plan = [(int(parts[1]), 1, 0, int(parts[2])), (int(parts[3]), 1, int(parts[2]), 0)]
+        elif len(parts) > 1:                               # "dma:<tile>[:<splits>]"
+            plan = [(int(parts[1]), int(parts[2]) if len(parts) > 2 else 1, 0, 0)]
+        else:
+            plan = _dma_plan(m, n, k)
+        for tile, splits, n_begin, n_count in plan:
+            ws = _workspace(splits * m * n, x.device) if splits > 1 else None
+            _check(lib.li_gemm_dma(_ptr(x), _ptr(wd), DT[x.dtype], _ptr(out), out_dt, mode, m, n, k, tile, splits,
+                                   _ptr(ws), rs, n_begin, n_count, _stream()), "gemm_dma")
         return out
     if kind == "fma":
         _check(lib.li_gemm_fma(_ptr(x), DT[x.dtype], _ptr(w), DT[w.dtype], _ptr(out), out_dt, mode,
@@ -254,18 +258,37 @@ def _stream_shape(n: int, k: int) -> tuple[int, int]:
     return 1, splits_for(g1)
 
 
-def _dma_shape(m: int, n: int, k: int) -> tuple[int, int]:
-    """Tile (0 = 128x128, 1 = 256x128, 2 = 256x256 rows of W x rows of X) and splits of K for
-    gemm_dma (measured on MI355X): the largest tile that still gives most of the 256 CUs a
-    workgroup; below that the smallest tile with K split."""
-    g2 = -(-m // 256) * -(-n // 256)
-    if g2 >= 192:
-        return 2, 1
-    g1 = -(-m // 128) * -(-n // 256)
-    if g1 >= 192:
-        return 1, 1
+_DMA_TILES = {0: (128, 128), 1: (256, 128), 2: (256, 256)}      # rows of W x rows of X
+# time of one round of workgroups (one per CU) relative to the 256 x 256 tile's, measured on MI355X
+_DMA_ROUND = {0: 0.39, 1: 0.58, 2: 1.0}
+
+
+def _dma_rounds(tile: int, m: int, n: int) -> float:
+    bn, bm = _DMA_TILES[tile]
+    return -(-(-(-m // bm) * -(-n // bn)) // 256) * _DMA_ROUND[tile]
+
+
+def _dma_plan(m: int, n: int, k: int) -> list:
+    """The launches of gemm_dma for a product: (tile, splits of K, first column, columns) each.
+    Workgroups run in rounds of one per CU, and a last round that is nearly empty costs as much as a
+    full one: the plan is the tile, or the large tile for as many columns as fill whole rounds
+    and a smaller tile for the rest, if the measured cost of a round makes that clearly faster; a product
+    too small to give most CUs a workgroup takes the smallest tile with K split."""
     g0 = -(-m // 128) * -(-n // 128)
-    return 0, (1 if g0 >= 192 else max(1, min(384 // g0, k // 512, 16)))
+    if g0 < 192:
+        return [(0, max(1, min(384 // g0, k // 512, 16)), 0, 0)]
+    best = min(range(3), key=lambda t: (_dma_rounds(t, m, n), -t))
+    plan, cost = [(best, 1, 0, 0)], _dma_rounds(best, m, n)
+    for big in (2, 1):
+        bn, bm = _DMA_TILES[big]
+        m_tiles = -(-m // bm)
+        cols = (m_tiles * -(-n // bn)) // 256 * 256 // m_tiles * bn      # columns that fill whole rounds
+        if 0 < cols < n:
+            rest = min(range(big), key=lambda t: (_dma_rounds(t, m, n - cols), -t))
+            c = _dma_rounds(big, m, cols) + _dma_rounds(rest, m, n - cols) + 0.02      # a second launch
+            if c < 0.95 * cost:                # the model is coarse: only a clear gain is taken
+                plan, cost = [(big, 1, 0, cols), (rest, 1, cols, 0)], c
+    return plan
 
 
 def _big_tile(m: int, n: int) -> int:
