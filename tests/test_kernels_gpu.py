@@ -425,3 +425,12 @@ def test_sampling_kernels(ops):
     assert t2 == [int(ops.uniform01(12, 1) * 64), int(ops.uniform01(11, 1) * 64)]
     us = [ops.uniform01(5, i) for i in range(2000)]
     assert 0.45 < sum(us) / len(us) < 0.55 and min(us) >= 0.0 and max(us) < 1.0
+    # drawn tokens follow the probabilities: 8192 sequences with generators of their own, one draw each
+    n, V = 8192, 7
+    row = torch.tensor([2.0, 0.5, -1.0, 1.5, 0.0, -3.0, 1.0])
+    p = P.probabilities(row.double(), 0.7)
+    state = torch.stack([torch.arange(n, dtype=torch.int64) + 1000, torch.zeros(n, dtype=torch.int64)], 1).to(DEV)
+    drawn = ops.sample(row.repeat(n, 1).to(DEV), 0.7, torch.arange(n, dtype=torch.int32, device=DEV), state)
+    freq = torch.bincount(drawn.cpu().long(), minlength=V).double() / n
+    sigma = torch.sqrt(p * (1 - p) / n)
+    assert ((freq - p).abs() < 5 * sigma + 1e-9).all(), (freq.tolist(), p.tolist())
