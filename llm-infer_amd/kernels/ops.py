@@ -178,12 +178,13 @@ def linear(x: torch.Tensor, w, mode: int = EPI_STORE, out: torch.Tensor | None =
     if tiled:
         _need(fast_ok and kind != "fma", "a tiled weight needs 16-bit activations of its dtype")
         # up to 16 rows (32 for a small matrix) every wave fetches the rows of X itself; up to 96
-        # rows they go through LDS once per workgroup; beyond that the tiled GEMM is faster
+        # rows (128 against a matrix of many rows) they go through LDS once per workgroup; beyond
+        # that the tiled GEMM is faster
         if kind == "gemv_mfma" or (force is None and (m <= 16 or (m <= 32 and n * k <= (1 << 25)))):
             _check(lib.li_gemv_tiled(_ptr(x), _ptr(wd), DT[x.dtype], _ptr(out), out_dt, mode, m, n, k, 0, 0,
                                      rs, _stream()), "gemv_tiled")
             return out
-        if force is None and m <= 96:
+        if force is None and (m <= 96 or (m <= 128 and n >= 16384)):
             kind = "stream"
         elif force is None and m * k * 2 < (1 << 32):
             kind = "dma"
@@ -259,34 +260,42 @@ def _stream_shape(n: int, k: int) -> tuple[int, int]:
 
 
 _DMA_TILES = {0: (128, 128), 1: (256, 128), 2: (256, 256)}      # rows of W x rows of X
-# time of one round of workgroups (one per CU) relative to the 256 x 256 tile's, measured on MI355X
-_DMA_ROUND = {0: 0.39, 1: 0.58, 2: 1.0}
+# microseconds that one round of workgroups (one per CU) takes at K = 4096, measured on MI355X
+_DMA_ROUND_US = {0: 48.0, 1: 72.0, 2: 124.0}
 
 
-def _dma_rounds(tile: int, m: int, n: int) -> float:
+def _dma_cost(tile: int, splits: int, m: int, n: int, k: int) -> float:
+    """Estimated microseconds of one gemm_dma launch (and its split-K reduction): rounds of
+    workgroups at the measured time of a round, not below the time to stream W once; a fixed cost for
+    the launch, the first tiles and the epilogue; the partial sums written and read back."""
     bn, bm = _DMA_TILES[tile]
-    return -(-(-(-m // bm) * -(-n // bn)) // 256) * _DMA_ROUND[tile]
+    rounds = -(-(-(-m // bm) * -(-n // bn) * splits) // 256)
+    k_split = -(-(-(-k // splits)) // 32) * 32
+    main = max(rounds * _DMA_ROUND_US[tile] * k_split / 4096, n * k * 2 / 5.5e6)
+    reduce = 2.5 + 2 * splits * m * n * 4 / 3.0e6 if splits > 1 else 0.0
+    return main + 5.5 + reduce
 
 
 def _dma_plan(m: int, n: int, k: int) -> list:
     """The launches of gemm_dma for a product: (tile, splits of K, first column, columns) each.
-    Workgroups run in rounds of one per CU, and a last round that is nearly empty costs as much as a
-    full one: the plan is the tile, or the large tile for as many columns as fill whole rounds
-    and a smaller tile for the rest, if the measured cost of a round makes that clearly faster; a product
-    too small to give most CUs a workgroup takes the smallest tile with K split."""
-    g0 = -(-m // 128) * -(-n // 128)
-    if g0 < 192:
-        return [(0, max(1, min(384 // g0, k // 512, 16)), 0, 0)]
-    best = min(range(3), key=lambda t: (_dma_rounds(t, m, n), -t))
-    plan, cost = [(best, 1, 0, 0)], _dma_rounds(best, m, n)
+    Tile and splits are the pair with the least estimated time (`_dma_cost`): few rows of X want
+    K split so that most CUs get a workgroup, but every split adds partial sums to write and read.
+    Workgroups run in rounds of one per CU, and a last round that is nearly empty costs as much as
+    a full one: a product of many rounds gets the large tile for as many columns as fill whole
+    rounds and a smaller tile for the rest, if that is clearly faster by the same estimate."""
+    options = [(t, s) for t in (2, 1, 0) for s in (1, 2, 3, 4, 6, 8, 12, 16) if s == 1 or k // s >= 1024]
+    tile, splits = min(options, key=lambda o: (_dma_cost(o[0], o[1], m, n, k), o[1], -o[0]))
+    plan, cost = [(tile, splits, 0, 0)], _dma_cost(tile, splits, m, n, k)
+    if splits > 1:
+        return plan
     for big in (2, 1):
         bn, bm = _DMA_TILES[big]
         m_tiles = -(-m // bm)
         cols = (m_tiles * -(-n // bn)) // 256 * 256 // m_tiles * bn      # columns that fill whole rounds
         if 0 < cols < n:
-            rest = min(range(big), key=lambda t: (_dma_rounds(t, m, n - cols), -t))
-            c = _dma_rounds(big, m, cols) + _dma_rounds(rest, m, n - cols) + 0.02      # a second launch
-            if c < 0.95 * cost:                # the model is coarse: only a clear gain is taken
+            rest = min(range(big), key=lambda t: (_dma_cost(t, 1, m, n - cols, k), -t))
+            c = _dma_cost(big, 1, m, cols, k) + _dma_cost(rest, 1, m, n - cols, k)
+            if c < 0.95 * cost:                # the estimate is coarse: only a clear gain is taken
                 plan, cost = [(big, 1, 0, cols), (rest, 1, cols, 0)], c
     return plan
 
