@@ -131,10 +131,29 @@ static __global__ void splitk_reduce_kernel(const float* __restrict__ ws, int sp
     if (i >= quads_per_row * e.M) return;
     const int m = (int)(i / quads_per_row), n = (int)(i % quads_per_row) * 4;
     float v[4] = {0.f, 0.f, 0.f, 0.f};
-    for (int s = 0; s < splits; ++s) {
-        const float* p = ws + ((int64_t)s * e.M + m) * e.N + n;
+    const int64_t stride = (int64_t)e.M * e.N;
+    const float* p = ws + (int64_t)m * e.N + n;
+    if (n + 3 < e.N && (e.N & 3) == 0) {
+        // four splits' loads in flight at a time; the sums stay in ascending split order
+        int s = 0;
+        for (; s + 4 <= splits; s += 4) {
+            f32x4 t[4];
 #pragma unroll
-        for (int q = 0; q < 4; ++q) if (n + q < e.N) v[q] += p[q];
+            for (int u = 0; u < 4; ++u) t[u] = *(const f32x4*)(p + (s + u) * stride);
+#pragma unroll
+            for (int u = 0; u < 4; ++u)
+#pragma unroll
+                for (int q = 0; q < 4; ++q) v[q] += t[u][q];
+        }
+        for (; s < splits; ++s) {
+            const f32x4 t = *(const f32x4*)(p + s * stride);
+#pragma unroll
+            for (int q = 0; q < 4; ++q) v[q] += t[q];
+        }
+    } else {
+        for (int s = 0; s < splits; ++s)
+#pragma unroll
+            for (int q = 0; q < 4; ++q) if (n + q < e.N) v[q] += p[s * stride + q];
     }
     epilogue4(e, m, n, v);
 }
