@@ -183,7 +183,7 @@ def test_the_loop_knows_beforehand_whether_all_go_on():
 def test_decode_splits_fill_the_chip_and_are_powers_of_two():
     assert decode_splits(1, 8, 32, 8192) == 64
     assert decode_splits(8, 8, 32, 8192) == 16
-    assert decode_splits(64, 8, 32, 8192) == 2
+    assert decode_splits(64, 8, 32, 8192) == 1 and decode_splits(32, 8, 32, 8192) == 4
     assert decode_splits(64, 32, 32, 4096) == 1
     assert decode_splits(1, 8, 32, 100) == 1 and decode_splits(1, 1, 64, 640) == 4
 
