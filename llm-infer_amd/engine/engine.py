@@ -5,7 +5,7 @@ import torch
 
 from ..cache import Cache, CacheError
 from ..registry import config_from_folder
-from ..weights import load_into, place_tensor, random_tensors
+from ..weights import OnDemand, load_into, place_tensor, random_tensors
 from .model import DecoderModel
 from .step import StepContext
 
@@ -59,11 +59,8 @@ class Engine:
         model = DecoderModel(config.model_spec(), dt, device)
         stored = as_dtype(stored_dtype) if stored_dtype else (dt if dt != torch.float32 else torch.bfloat16)
         params = model.params()
-        tensors = {}
-        for name, spec in params.items():
-            t = random_tensors({name: spec}, seed, stored, device)[name]
-            tensors[name] = place_tensor(t, spec.kind, dt, device)
-        model.bind(tensors)
+        model.bind(OnDemand(lambda name: place_tensor(random_tensors({name: params[name]}, seed, stored, device)[name],
+                                                      params[name].kind, dt, device)))
         return cls(config, model, max_tokens, n_slots)
 
     # -- sequences -----------------------------------------------------------------

@@ -64,12 +64,15 @@ class DecoderModel(Part):
             stack.extend(p.children())
         return out
 
-    def bind(self, tensors: dict) -> None:
+    def bind(self, tensors) -> None:
+        """``tensors``: full tensor name -> tensor.  They are asked for part by part, so a mapping that
+        makes each tensor when it is asked for (``weights.loader.OnDemand``) never holds more than one
+        part's tensors beside what the parts keep."""
         per_part: dict = {}
         for name, (part, local, _) in self._table.items():
-            per_part.setdefault(id(part), (part, {}))[1][local] = tensors[name]
-        for part, local in per_part.values():
-            part.bind(local)
+            per_part.setdefault(id(part), (part, []))[1].append((local, name))
+        for part, names in per_part.values():
+            part.bind({local: tensors[name] for local, name in names})
         if getattr(self.head, "tied", False):
             self.head.tie(self.embedding.weight)
 

@@ -152,5 +152,16 @@ def load_into(model, folder: str, config=None) -> None:
         # looks at it (frequency factors of a rotation scaling that neither it nor this library applies)
         ignorable.append("rope_freqs.weight")
     check_tensors(needed, ckpt, ignorable)
-    model.bind({name: place_tensor(ckpt.tensor(name), spec.kind, model.dtype, model.device)
-                for name, spec in needed.items()})
+    model.bind(OnDemand(lambda name: place_tensor(ckpt.tensor(name), needed[name].kind, model.dtype, model.device)))
+
+
+class OnDemand:
+    """A mapping name -> tensor that makes the tensor when it is asked for and keeps nothing: a model
+    binds its parts one after the other, so the device never holds a whole checkpoint twice (once as
+    read and once as the parts keep it: fused, interleaved, tiled)."""
+
+    def __init__(self, make):
+        self._make = make
+
+    def __getitem__(self, name: str):
+        return self._make(name)
