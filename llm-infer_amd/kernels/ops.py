@@ -5,6 +5,7 @@ checked here before the launch; nothing falls back to another implementation.
 from __future__ import annotations
 
 import ctypes
+import functools
 from ctypes import c_float, c_int, c_int64, c_uint64, c_void_p
 
 import torch
@@ -276,6 +277,7 @@ def _dma_cost(tile: int, splits: int, m: int, n: int, k: int) -> float:
     return main + 5.5 + reduce
 
 
+@functools.lru_cache(maxsize=4096)
 def _dma_plan(m: int, n: int, k: int) -> list:
     """The launches of gemm_dma for a product: (tile, splits of K, first column, columns) each.
     Tile and splits are the pair with the least estimated time (`_dma_cost`): few rows of X want
