@@ -168,8 +168,10 @@ class LlamaConfig:
         if self.rotary_dim % 2 != 0 or not 0 < self.rotary_dim <= self.head_dim:
             raise ConfigError(f"the rotated part of a head must be even and within head_dim, got "
                               f"{self.rotary_dim} of {self.head_dim}")
-        if self.hidden_act != "silu":
-            raise ConfigError(f"hidden_act {self.hidden_act!r}: this architecture's feed-forward uses silu")
+        if self.hidden_act not in ("silu", "gelu"):
+            # the reference warns and takes gelu (config.cpp:97-105); a wrong activation is refused here
+            raise ConfigError(f"hidden_act {self.hidden_act!r}: the feed-forward's gate takes 'silu' or 'gelu' "
+                              "(the tanh form, include/kernels_cpu.hpp:179-184)")
         if self.rope_pairing not in ("adjacent", "half"):
             raise ConfigError(f"rope_pairing must be 'adjacent' or 'half', got {self.rope_pairing!r}")
         if self.torch_dtype is not None and self.torch_dtype not in _DTYPES:
@@ -211,7 +213,7 @@ class LlamaConfig:
             "n_kv_heads": self.num_key_value_heads, "head_dim": self.head_dim,
             "scale": self.head_dim ** -0.5, "window": None})
         ffn = PartSpec("gated_mlp", {"hidden_size": self.hidden_size,
-                                     "intermediate_size": self.intermediate_size, "activation": "silu"})
+                                     "intermediate_size": self.intermediate_size, "activation": self.hidden_act})
         layers = []
         for i in range(self.num_hidden_layers):
             p = f"model.layers.{i}."

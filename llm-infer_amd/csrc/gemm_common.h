@@ -3,7 +3,15 @@
 #pragma once
 #include "common.h"
 
-enum { EPI_STORE = 0, EPI_ADD = 1, EPI_SWIGLU = 2, EPI_ROPE = 3 };
+enum { EPI_STORE = 0, EPI_ADD = 1, EPI_SWIGLU = 2, EPI_ROPE = 3, EPI_GEGLU = 4 };
+
+// The gate's activation: silu(x) = x / (1 + exp(-x)) (include/kernels_cpu.hpp:186) or the tanh form of
+// gelu that the reference computes, 0.5 x (1 + tanh(sqrt(2 / pi) (x + 0.044715 x^3)))
+// (include/kernels_cpu.hpp:179-184).
+__device__ __forceinline__ float gate_activation(float g, bool gelu) {
+    if (gelu) return 0.5f * g * (1.f + tanhf(0.7978845608028654f * (g + 0.044715f * g * g * g)));
+    return g / (1.f + expf(-g));
+}
 
 // What the EPI_ROPE epilogue needs: the columns of the product are the q heads, then the k heads,
 // then the v heads of a token; q and k are rotated by the token's position (adjacent pairs), q goes
@@ -82,14 +90,14 @@ __device__ __forceinline__ void epilogue4(const Epilogue& e, int m, int n, const
         }
         return;
     }
-    if (e.mode == EPI_SWIGLU) {
-        // columns 2j (gate) and 2j+1 (up) give h[m, j] = silu(gate) * up   (src/model/block.cpp:209-213)
+    if (e.mode == EPI_SWIGLU || e.mode == EPI_GEGLU) {
+        // columns 2j (gate) and 2j+1 (up) give h[m, j] = act(gate) * up   (src/model/block.cpp:203-214)
         const int64_t row = (int64_t)m * (e.N >> 1);
 #pragma unroll
         for (int j = 0; j < 4; j += 2) {
             if (n + j + 1 < e.N) {
                 const float g = v[j], u = v[j + 1];
-                store_one(e.C, e.out_dt, row + ((n + j) >> 1), g / (1.f + expf(-g)) * u);
+                store_one(e.C, e.out_dt, row + ((n + j) >> 1), gate_activation(g, e.mode == EPI_GEGLU) * u);
             }
         }
         return;
@@ -175,10 +183,10 @@ static int make_epilogue(Epilogue& e, void* C, int mode, int out_dt, int M, int 
 
 static int check_common(const void* X, const void* W, const void* C, int M, int N, int K, int mode, int out_dt) {
     if (!X || !W || (!C && mode != EPI_ROPE) || M < 0 || N <= 0 || K <= 0) return LI_BAD_ARG;
-    if (mode < EPI_STORE || mode > EPI_ROPE) return LI_BAD_ARG;
+    if (mode < EPI_STORE || mode > EPI_GEGLU) return LI_BAD_ARG;
     if (out_dt < DT_F32 || out_dt > DT_BF16) return LI_BAD_ARG;
     if (mode == EPI_ADD && out_dt != DT_F32) return LI_BAD_ARG;
-    if (mode == EPI_SWIGLU && (N & 1)) return LI_BAD_ARG;
+    if ((mode == EPI_SWIGLU || mode == EPI_GEGLU) && (N & 1)) return LI_BAD_ARG;
     return LI_OK;
 }
 

@@ -14,7 +14,8 @@ from . import build
 
 PAGE = 64
 DT = {torch.float32: 0, torch.float16: 1, torch.bfloat16: 2}
-EPI_STORE, EPI_ADD, EPI_SWIGLU, EPI_ROPE = 0, 1, 2, 3
+EPI_STORE, EPI_ADD, EPI_SWIGLU, EPI_ROPE, EPI_GEGLU = 0, 1, 2, 3, 4
+GATED = (EPI_SWIGLU, EPI_GEGLU)             # gate and up rows interleaved in W, act(gate) * up written
 _STATUS = {1: "bad argument", 2: "unsupported size or alignment", 3: "HIP launch error"}
 
 
@@ -149,15 +150,15 @@ def _workspace(n_floats: int, device) -> torch.Tensor:
 
 def linear(x: torch.Tensor, w, mode: int = EPI_STORE, out: torch.Tensor | None = None,
            out_dtype=None, force: str | None = None, _rope=None) -> torch.Tensor:
-    """C = X W^T with the epilogue ``mode``: store, add into ``out`` (float32), or SwiGLU over
-    interleaved gate/up rows of W (C has N/2 columns).  ``force`` picks a kernel for tests."""
+    """C = X W^T with the epilogue ``mode``: store, add into ``out`` (float32), or act(gate) * up over
+    interleaved gate/up rows of W (C has N/2 columns; EPI_SWIGLU: silu, EPI_GEGLU: gelu).  ``force`` picks a kernel for tests."""
     tiled = isinstance(w, TiledWeight)
     wd = w.data if tiled else w
     _dev(x, wd, out)
     _need(x.dim() == 2 and len(w.shape) == 2 and x.shape[1] == w.shape[1], f"linear: x {tuple(x.shape)} w {tuple(w.shape)}")
     m, k = x.shape
     n = w.shape[0]
-    n_out = n // 2 if mode == EPI_SWIGLU else n
+    n_out = n // 2 if mode in GATED else n
     if mode == EPI_ADD:
         _need(out is not None and out.dtype == torch.float32, "add epilogue needs a float32 output")
     rs = ctypes.byref(_rope) if _rope is not None else None
@@ -168,8 +169,8 @@ def linear(x: torch.Tensor, w, mode: int = EPI_STORE, out: torch.Tensor | None =
     if mode != EPI_ROPE:
         _need(out.shape == (m, n_out), f"linear: out {tuple(out.shape)}, expected {(m, n_out)}")
     out_dt = DT[out.dtype] if out is not None else 0
-    if mode == EPI_SWIGLU:
-        _need(n % 2 == 0, "SwiGLU epilogue needs an even number of rows of W")
+    if mode in GATED:
+        _need(n % 2 == 0, "a gated epilogue needs an even number of rows of W")
     if m == 0:
         return out
     lib = core()
@@ -308,12 +309,12 @@ def _big_tile(m: int, n: int) -> int:
     return 1 if (-(-m // 128)) * (-(-n // 256)) >= 1024 else 0
 
 
-def swiglu(gu: torch.Tensor, out_dtype) -> torch.Tensor:
-    """h[:, j] = silu(gu[:, 2j]) * gu[:, 2j+1] for float32 gu."""
+def swiglu(gu: torch.Tensor, out_dtype, gelu: bool = False) -> torch.Tensor:
+    """h[:, j] = act(gu[:, 2j]) * gu[:, 2j+1] for float32 gu; act is silu, or the reference's gelu."""
     _dev(gu)
     _need(gu.dtype == torch.float32 and gu.dim() == 2 and gu.shape[1] % 2 == 0, "gu: float32 [T, 2F]")
     h = torch.empty((gu.shape[0], gu.shape[1] // 2), dtype=out_dtype, device=gu.device)
-    _check(core().li_swiglu(_ptr(gu), _ptr(h), DT[out_dtype], c_int64(h.numel()), _stream()), "swiglu")
+    _check(core().li_swiglu(_ptr(gu), _ptr(h), DT[out_dtype], c_int64(h.numel()), int(gelu), _stream()), "swiglu")
     return h
 
 
@@ -523,7 +524,7 @@ def tile_weight(w: torch.Tensor) -> TiledWeight:
 def gemv_tiled(x, w: TiledWeight, mode=EPI_STORE, out_dtype=None, nt=0, kw=0):
     """gemv_tiled with a chosen shape of workgroup (for tuning and tests)."""
     m, k = x.shape
-    n_out = w.n // 2 if mode == EPI_SWIGLU else w.n
+    n_out = w.n // 2 if mode in GATED else w.n
     out = torch.empty((m, n_out), dtype=out_dtype or x.dtype, device=x.device)
     _check(core().li_gemv_tiled(_ptr(x), _ptr(w.data), DT[x.dtype], _ptr(out), DT[out.dtype], mode, m, w.n, k,
                                 nt, kw, None, _stream()), "gemv_tiled")

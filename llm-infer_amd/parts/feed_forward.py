@@ -10,8 +10,9 @@ from .base import Part
 
 @register_feed_forward("gated_mlp")
 class GatedMLP(Part):
-    """down(act(gate(x)) * up(x)) added into the residual stream, act = silu = x / (1 + exp(-x))
-    (src/model/block.cpp:200-222, include/kernels_cpu.hpp:186).
+    """down(act(gate(x)) * up(x)) added into the residual stream; act is silu, x / (1 + exp(-x)), or
+    gelu in the tanh form the reference computes (src/model/block.cpp:200-222,
+    include/kernels_cpu.hpp:179-186).
 
     Gate and up rows are interleaved into one matrix (row 2j = gate_j, row 2j+1 = up_j),
     so that one product yields both and its epilogue applies the activation before
@@ -19,8 +20,9 @@ class GatedMLP(Part):
     """
 
     def __init__(self, *, hidden_size, intermediate_size, activation="silu", prefix, dtype, device):
-        if activation != "silu":
-            raise ValueError(f"gated_mlp: activation {activation!r} is not built (silu is)")
+        if activation not in ("silu", "gelu"):
+            raise ValueError(f"gated_mlp: activation {activation!r} is not built (silu and gelu are)")
+        self.mode = ops.EPI_SWIGLU if activation == "silu" else ops.EPI_GEGLU
         self.hidden_size, self.intermediate_size = hidden_size, intermediate_size
         self.prefix, self.dtype, self.device = prefix, dtype, device
         self.w_gate_up = self.w_down = None
@@ -39,5 +41,5 @@ class GatedMLP(Part):
         self.w_down = ops.prepare_weight(tensors["down_proj.weight"])
 
     def forward(self, h, residual):
-        t = ops.linear(h, self.w_gate_up, ops.EPI_SWIGLU, out_dtype=self.dtype)
+        t = ops.linear(h, self.w_gate_up, self.mode, out_dtype=self.dtype)
         ops.linear(t, self.w_down, ops.EPI_ADD, out=residual)

@@ -40,6 +40,7 @@ def sizes(cfg: dict) -> dict:
         rotary=rotary,
         eps=float(cfg.get("rms_norm_eps", 1e-5)),           # config.cpp:93
         tied=bool(cfg.get("tie_word_embeddings", False)),
+        act=cfg.get("hidden_act", "silu"),                  # config.cpp:97-105
     )
 
 
@@ -120,10 +121,16 @@ def silu(x: torch.Tensor) -> torch.Tensor:
     return x / (1.0 + torch.exp(-x))
 
 
+def gelu(x: torch.Tensor) -> torch.Tensor:
+    """The tanh form: 0.5 x (1 + tanh(sqrt(2 / pi) (x + 0.044715 x^3))) (include/kernels_cpu.hpp:179-184)."""
+    return 0.5 * x * (1.0 + torch.tanh(math.sqrt(2.0 / math.pi) * (x + 0.044715 * x * x * x)))
+
+
 def swiglu(x: torch.Tensor, w_gate: torch.Tensor, w_up: torch.Tensor, w_down: torch.Tensor,
-           act_dtype=None) -> torch.Tensor:
-    """down(silu(gate(x)) * up(x)) (src/model/block.cpp:200-217)."""
-    return linear(_r(silu(linear(x, w_gate)) * linear(x, w_up), act_dtype), w_down)
+           act_dtype=None, act: str = "silu") -> torch.Tensor:
+    """down(act(gate(x)) * up(x)), act chosen by the configuration (src/model/block.cpp:200-217)."""
+    fn = {"silu": silu, "gelu": gelu}[act]                     # block.cpp:203-214
+    return linear(_r(fn(linear(x, w_gate)) * linear(x, w_up), act_dtype), w_down)
 
 
 def attention_part(x, w, prefix, s, positions, window=None, act_dtype=None):
@@ -145,7 +152,7 @@ def block(x, w, i, s, positions, act_dtype=None):
     x = x + attention_part(h, w, p + "self_attn.", s, positions, None, act_dtype)  # block.cpp:170-172
     h = _r(rmsnorm(x, w[p + "post_attention_layernorm.weight"], s["eps"]), act_dtype)   # block.cpp:177-183
     x = x + swiglu(h, w[p + "mlp.gate_proj.weight"], w[p + "mlp.up_proj.weight"],
-                   w[p + "mlp.down_proj.weight"], act_dtype)                       # block.cpp:220-222
+                   w[p + "mlp.down_proj.weight"], act_dtype, s.get("act", "silu"))  # block.cpp:220-222
     return x
 
 

@@ -42,7 +42,7 @@ def test_every_size_comes_from_the_config():
 
 @pytest.mark.parametrize("change,message", [
     ({"hidden_size": 66}, "divisible"), ({"num_key_value_heads": 3}, "multiple"),
-    ({"hidden_act": "gelu"}, "silu"), ({"partial_rotary_factor": 0.45}, "even"),
+    ({"hidden_act": "relu"}, "silu"), ({"partial_rotary_factor": 0.45}, "even"),
     ({"num_hidden_layers": 0}, "positive"), ({"torch_dtype": "int8"}, "Unsupported torch_dtype"),
     ({"rope_pairing": "odd"}, "rope_pairing"), ({"architectures": ["MambaForCausalLM"]}, "unknown architecture"),
     ({"architectures": []}, "names no architecture"),

@@ -98,6 +98,17 @@ def test_parts_alone(lib, dt):
     ffn.forward(h, res)
     f_ref = P.swiglu(h.double().cpu(), w64["f.gate_proj.weight"], w64["f.up_proj.weight"], w64["f.down_proj.weight"])
     assert (res.double().cpu() - (x_ref + f_ref)).abs().max() < tol * (1 + f_ref.abs().max())
+    # the same feed-forward with the gate's other activation
+    ffn_g = GatedMLP(hidden_size=d, intermediate_size=F, activation="gelu", prefix="f.", dtype=dt, device=DEV)
+    ffn_g.bind({n: dev["f." + n] for n in ffn_g.params()})
+    res = x.clone()
+    ffn_g.forward(h, res)
+    g_ref = P.swiglu(h.double().cpu(), w64["f.gate_proj.weight"], w64["f.up_proj.weight"], w64["f.down_proj.weight"],
+                     act="gelu")
+    assert (res.double().cpu() - (x_ref + g_ref)).abs().max() < tol * (1 + g_ref.abs().max())
+    assert (g_ref - f_ref).abs().max() > 100 * tol * (1 + f_ref.abs().max()) or dt != torch.float32
+    with pytest.raises(ValueError, match="silu and gelu"):
+        GatedMLP(hidden_size=d, intermediate_size=F, activation="relu", prefix="f.", dtype=dt, device=DEV)
     # attention over a fresh cache, two sequences of unequal length in one step
     cache = Cache([attn.cache_spec()], 256, 128, dt, DEV, 2)
     slots = [cache.alloc_slot(), cache.alloc_slot()]

@@ -59,6 +59,9 @@ def _linear_ref(x, w, mode, res=None):
     if mode == 2:
         g, u = y[:, 0::2], y[:, 1::2]
         return g / (1 + torch.exp(-g)) * u
+    if mode == 4:                                   # the gate's other activation: gelu in its tanh form
+        g, u = y[:, 0::2], y[:, 1::2]
+        return torch.nn.functional.gelu(g, approximate="tanh") * u
     return y
 
 
@@ -81,15 +84,15 @@ def test_linear_all_kernels_and_epilogues(ops, M, N, K, dt):
             kinds.append("gemv_mfma")
         kinds += ["mfma:0:1", "mfma:1:1", "mfma:2:1", "mfma:2:3", "mfma:0:2", "big:0", "big:1", "big:0:3", None]
     for kind in kinds:
-        for mode in (0, 1, 2):
-            if mode == 2 and N % 2:
+        for mode in (0, 1, 2, 4):
+            if mode in (2, 4) and N % 2:
                 continue
             ref = _linear_ref(x, w, mode, res)
             if mode == 1:
                 out = res.clone()
                 ops.linear(x, w, mode, out=out, force=kind)
                 tol = 1e-5 if dt == torch.float32 else 2e-4
-            elif mode == 2:
+            elif mode in (2, 4):
                 out = ops.linear(x, w, mode, out_dtype=torch.float32, force=kind)
                 tol = 1e-5 if dt == torch.float32 else 2e-4
             else:
@@ -125,8 +128,8 @@ def test_linear_tiled_weights(ops, M, N, K, dt):
     if M <= 128:
         kinds += ["stream", "stream:1:1", "stream:2:1", "stream:1:3", "stream:2:16"]
     for kind in kinds:
-        for mode in (0, 1, 2):
-            if mode == 2 and N % 2:
+        for mode in (0, 1, 2, 4):
+            if mode in (2, 4) and N % 2:
                 continue
             ref = _linear_ref(x, w, mode, res)
             if mode == 1:
@@ -149,6 +152,18 @@ def test_linear_tiled_weights(ops, M, N, K, dt):
         ops.linear(x, wt, force="fma")
     with pytest.raises(ops.KernelError):
         ops.tile_weight(w[:, :K - 8].contiguous())
+
+
+def test_gate_activation_alone(ops):
+    """act(gate) * up on interleaved columns, for a product that was stored unactivated."""
+    g = torch.Generator().manual_seed(3)
+    gu = (torch.randn(5, 2 * 173, generator=g) * 3).to(DEV)
+    gate, up = gu[:, 0::2].double(), gu[:, 1::2].double()
+    for gelu, ref in ((False, gate / (1 + torch.exp(-gate)) * up),
+                      (True, torch.nn.functional.gelu(gate, approximate="tanh") * up)):
+        out = ops.swiglu(gu, torch.float32, gelu=gelu)
+        assert out.shape == (5, 173) and (out.double() - ref).abs().max() < 1e-5 * (1 + ref.abs().max())
+        assert ops.swiglu(gu, torch.bfloat16, gelu=gelu).dtype == torch.bfloat16
 
 
 def test_linear_rows_do_not_depend_on_the_batch_in_float32(ops):

@@ -143,6 +143,15 @@ def test_silu_and_swiglu():
     ref = torch.nn.functional.linear(torch.nn.functional.silu(xx @ wg.t()) * (xx @ wu.t()), wd)
     assert torch.allclose(P.swiglu(xx, wg, wu, wd), ref)
     assert not torch.allclose(P.swiglu(xx, wu, wg, wd), ref)       # gate and up are not interchangeable
+    # the other activation of the gate: the library's tanh form, no other (the exact form differs by 1e-3),
+    # zero at zero, the identity far out, and chosen by name
+    g = P.gelu(x)
+    assert torch.allclose(g, torch.nn.functional.gelu(x, approximate="tanh"))
+    assert not torch.allclose(P.gelu(xx), torch.nn.functional.gelu(xx), atol=1e-5)
+    assert g[0] == 0 and abs(g[1] - 30.0) < 1e-9 and g[2] < 0
+    ref = torch.nn.functional.linear(torch.nn.functional.gelu(xx @ wg.t(), approximate="tanh") * (xx @ wu.t()), wd)
+    assert torch.allclose(P.swiglu(xx, wg, wu, wd, act="gelu"), ref)
+    assert not torch.allclose(P.swiglu(xx, wg, wu, wd, act="silu"), ref)
 
 
 @pytest.mark.parametrize("name", list(ALL))

@@ -17,13 +17,13 @@ TINY_B = {
 }
 
 # 1 layer, MHA 5/5, explicit head_dim 48 != hidden/heads, half of each head rotated,
-# odd vocabulary, long context
+# odd vocabulary, long context, the gate's other activation
 TINY_C = {
     "architectures": ["LlamaForCausalLM"], "model_type": "llama",
     "num_hidden_layers": 1, "hidden_size": 80, "num_attention_heads": 5, "head_dim": 48,
     "intermediate_size": 136, "vocab_size": 331, "rope_theta": 1000.0, "rms_norm_eps": 1e-4,
     "partial_rotary_factor": 0.5,
-    "max_position_embeddings": 1024, "tie_word_embeddings": False, "hidden_act": "silu",
+    "max_position_embeddings": 1024, "tie_word_embeddings": False, "hidden_act": "gelu",
 }
 
 ALL = {"A": TINY_A, "B": TINY_B, "C": TINY_C}
