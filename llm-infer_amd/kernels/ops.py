@@ -202,15 +202,33 @@ def linear(x: torch.Tensor, w, mode: int = EPI_STORE, out: torch.Tensor | None =
         _need(tiled and fast_ok and m * k * 2 < (1 << 32), "gemm_dma: a tiled weight, X below 4 GiB")
         parts = kind.split(":")
         if parts[0] == "dma2":                             # "dma2:<tile>:<columns>:<tile of the rest>" for tests
-            plan = [(int(parts[1]), 1, 0, int(parts[2])), (int(parts[3]), 1, int(parts[2]), 0)]
+            plan = [(int(parts[1]), 1, 0, int(parts[2]), 0, 0), (int(parts[3]), 1, int(parts[2]), 0, 0, 0)]
+        elif parts[0] == "dmarows":                        # "dmarows:<tile>:<rows>:<tile of the rest>" for tests
+            plan = [(int(parts[1]), 1, 0, 0, 0, int(parts[2])), (int(parts[3]), 1, 0, 0, int(parts[2]), 0)]
         elif len(parts) > 1:                               # "dma:<tile>[:<splits>]"
-            plan = [(int(parts[1]), int(parts[2]) if len(parts) > 2 else 1, 0, 0)]
+            plan = [(int(parts[1]), int(parts[2]) if len(parts) > 2 else 1, 0, 0, 0, 0)]
         else:
             plan = _dma_plan(m, n, k)
-        for tile, splits, n_begin, n_count in plan:
-            ws = _workspace(splits * m * n, x.device) if splits > 1 else None
-            _check(lib.li_gemm_dma(_ptr(x), _ptr(wd), DT[x.dtype], _ptr(out), out_dt, mode, m, n, k, tile, splits,
-                                   _ptr(ws), rs, n_begin, n_count, _stream()), "gemm_dma")
+        esize = {0: 4, 1: 2, 2: 2}
+        for tile, splits, n_begin, n_count, m_begin, m_count in plan:
+            rows = m_count or m - m_begin
+            _need(0 <= m_begin < m and m_begin + rows <= m, "gemm_dma: rows outside the product")
+            ws = _workspace(splits * rows * n, x.device) if splits > 1 else None
+            xp = c_void_p(x.data_ptr() + m_begin * k * x.element_size())
+            op = c_void_p(out.data_ptr() + m_begin * n_out * out.element_size()) if out is not None else c_void_p(0)
+            rp = rs
+            if _rope is not None and m_begin:
+                # the epilogue's per-row arrays and q, for the rows of this launch
+                shifted = _RopeStore()
+                ctypes.pointer(shifted)[0] = _rope
+                half = _rope.rotary_dim // 2
+                for field, step in (("pos", 4), ("tok_slot", 4), ("cos_sin", half * 2 * 4),
+                                    ("q_out", _rope.H * _rope.hd * esize[_rope.dt])):
+                    v = getattr(_rope, field)
+                    setattr(shifted, field, v + m_begin * step if v else v)
+                rp = ctypes.byref(shifted)
+            _check(lib.li_gemm_dma(xp, _ptr(wd), DT[x.dtype], op, out_dt, mode, rows, n, k, tile, splits,
+                                   _ptr(ws), rp, n_begin, n_count, _stream()), "gemm_dma")
         return out
     if kind == "fma":
         _check(lib.li_gemm_fma(_ptr(x), DT[x.dtype], _ptr(w), DT[w.dtype], _ptr(out), out_dt, mode,
@@ -280,26 +298,34 @@ def _dma_cost(tile: int, splits: int, m: int, n: int, k: int) -> float:
 
 @functools.lru_cache(maxsize=4096)
 def _dma_plan(m: int, n: int, k: int) -> list:
-    """The launches of gemm_dma for a product: (tile, splits of K, first column, columns) each.
+    """The launches of gemm_dma for a product: (tile, splits of K, first column, columns, first row,
+    rows) each (0 columns or rows: all from the first on).
     Tile and splits are the pair with the least estimated time (`_dma_cost`): few rows of X want
     K split so that most CUs get a workgroup, but every split adds partial sums to write and read.
     Workgroups run in rounds of one per CU, and a last round that is nearly empty costs as much as
-    a full one: a product of many rounds gets the large tile for as many columns as fill whole
-    rounds and a smaller tile for the rest, if that is clearly faster by the same estimate."""
+    a full one: a product of many rounds gets the large tile for as many columns (or, if that fits
+    better, rows) as fill whole rounds and a smaller tile for the rest, if that is clearly faster by
+    the same estimate."""
     options = [(t, s) for t in (2, 1, 0) for s in (1, 2, 3, 4, 6, 8, 12, 16) if s == 1 or k // s >= 1024]
     tile, splits = min(options, key=lambda o: (_dma_cost(o[0], o[1], m, n, k), o[1], -o[0]))
-    plan, cost = [(tile, splits, 0, 0)], _dma_cost(tile, splits, m, n, k)
+    plan, cost = [(tile, splits, 0, 0, 0, 0)], _dma_cost(tile, splits, m, n, k)
     if splits > 1:
         return plan
     for big in (2, 1):
         bn, bm = _DMA_TILES[big]
-        m_tiles = -(-m // bm)
-        cols = (m_tiles * -(-n // bn)) // 256 * 256 // m_tiles * bn      # columns that fill whole rounds
+        m_tiles, n_tiles = -(-m // bm), -(-n // bn)
+        whole = m_tiles * n_tiles // 256 * 256                 # workgroups of the whole rounds
+        cols, rows = whole // m_tiles * bn, whole // n_tiles * bm
         if 0 < cols < n:
             rest = min(range(big), key=lambda t: (_dma_cost(t, 1, m, n - cols, k), -t))
             c = _dma_cost(big, 1, m, cols, k) + _dma_cost(rest, 1, m, n - cols, k)
             if c < 0.95 * cost:                # the estimate is coarse: only a clear gain is taken
-                plan, cost = [(big, 1, 0, cols), (rest, 1, cols, 0)], c
+                plan, cost = [(big, 1, 0, cols, 0, 0), (rest, 1, cols, 0, 0, 0)], c
+        if 0 < rows < m:
+            rest = min(range(big), key=lambda t: (_dma_cost(t, 1, m - rows, n, k), -t))
+            c = _dma_cost(big, 1, rows, n, k) + _dma_cost(rest, 1, m - rows, n, k)
+            if c < 0.95 * cost:
+                plan, cost = [(big, 1, 0, 0, 0, rows), (rest, 1, 0, 0, rows, 0)], c
     return plan
 
 

@@ -125,6 +125,8 @@ def test_linear_tiled_weights(ops, M, N, K, dt):
     kinds += ["dma", "dma:0", "dma:1", "dma:2", "dma:0:2", "dma:1:5", "dma:2:3"]
     # the first columns with one tile, the rest with another (the first count a multiple of the first tile)
     kinds += [f"dma2:{a}:{c}:{b}" for a, c, b in ((2, 256, 1), (2, 512, 0), (1, 512, 0), (0, 128, 2)) if c < N]
+    # and the first rows with one tile, the rest with another
+    kinds += [f"dmarows:{a}:{r}:{b}" for a, r, b in ((2, 256, 0), (1, 128, 0), (0, 128, 2)) if r < M]
     if M <= 128:
         kinds += ["stream", "stream:1:1", "stream:2:1", "stream:1:3", "stream:2:16"]
     for kind in kinds:
@@ -389,7 +391,7 @@ def test_rotation_fused_into_the_projection(ops, dt, T, H, K, hd, rot, d):
         if tiled and d % 32:
             continue
         ww = ops.tile_weight(w) if tiled else w
-        for kind in kinds + ((["dma:0", "dma:1:2", "dma:2"] + (["dma2:0:128:1"] if (H + 2 * K) * hd > 128 else []) + (["stream:1:1", "stream:2:2"] if T <= 128 else [])) if tiled else []):
+        for kind in kinds + ((["dma:0", "dma:1:2", "dma:2"] + (["dma2:0:128:1"] if (H + 2 * K) * hd > 128 else []) + (["dmarows:0:128:1"] if T > 128 else []) + (["stream:1:1", "stream:2:2"] if T <= 128 else [])) if tiled else []):
             if tiled and kind == "fma":
                 continue
             c1, v1 = fresh()
