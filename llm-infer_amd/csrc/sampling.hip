@@ -73,55 +73,116 @@ __global__ __launch_bounds__(64) void argmax_final_kernel(const float* __restric
     if (threadIdx.x == 0) out[blockIdx.x] = best_i == 0x7fffffff ? 0 : best_i;
 }
 
-// state: [n_slots, 2] uint64 (key, counter); the counter advances by one per sampled token.
-__global__ __launch_bounds__(1024) void sample_kernel(const float* __restrict__ logits, int V, float temperature,
-                                                      const int* __restrict__ seq_slot,
-                                                      unsigned long long* __restrict__ state,
-                                                      const float* __restrict__ forced_r,
-                                                      int* __restrict__ out) {
+// Temperature sampling in two stages, so that a few rows still use the whole chip.
+// Stage 1: a workgroup takes one chunk of a row (a multiple of 64 elements, at most 64 chunks a row),
+// finds the chunk's maximum m and writes, for every 64 consecutive elements ("step"), the sum of
+// exp((l - m) / T), and the chunk's sum of these, all taken in index order.
+// Stage 2: one wave a row brings the chunks to the row's maximum (sum * exp((m - max) / T)), and
+// finds with scans over its lanes first the chunk, then the step, then the index at which the
+// cumulative sum exceeds r * total: the inverse CDF of tools/infer.cpp:50-60 up to float32 rounding
+// of the sums (the exponential is the hardware's 2^x).  Where rounding lets every candidate pass,
+// the last one is taken (the fallback of :60).
+#define LOG2E_F 1.4426950408889634f
+
+__device__ __forceinline__ float wave_inclusive_scan(float v, int lane) {
+#pragma unroll
+    for (int o = 1; o < WAVE; o <<= 1) {
+        const float t = __shfl_up(v, o, WAVE);
+        if (lane >= o) v += t;
+    }
+    return v;
+}
+
+// workspace per row and chunk: [0] maximum, [1] sum, [2 .. 2 + steps) step sums; steps = chunk / 64
+__global__ __launch_bounds__(256) void sample_chunks_kernel(const float* __restrict__ logits, int V, int chunk,
+                                                            float temperature, float* __restrict__ ws) {
     __shared__ float scratch[16];
-    __shared__ float sums[1024];
-    __shared__ int found;
+    __shared__ float wave_tot[4];
     const float* row = logits + (int64_t)blockIdx.x * V;
-    const int tid = threadIdx.x, nt = blockDim.x;
+    const int c0 = blockIdx.y * chunk, c1 = min(V, c0 + chunk);
+    const int steps = chunk >> 6;
+    float* out = ws + ((int64_t)blockIdx.x * gridDim.y + blockIdx.y) * (2 + steps);
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     float mx = -INFINITY;
-    for (int i = tid; i < V; i += nt) mx = fmaxf(mx, row[i]);
+    for (int i = c0 + tid; i < c1; i += 256) mx = fmaxf(mx, row[i]);
     mx = block_max(mx, scratch);
-    const int chunk = (V + nt - 1) / nt;
-    const int c0 = min(V, tid * chunk), c1 = min(V, c0 + chunk);
-    float local = 0.f;
-    for (int i = c0; i < c1; ++i) local += expf((row[i] - mx) / temperature);
-    sums[tid] = local;
-    if (tid == 0) found = V - 1;
+    const float scale2 = LOG2E_F / temperature;                   // exp(d / T) = 2^(d * log2(e) / T)
+    float total = 0.f;
+    for (int st = wave; st < steps; st += 4) {
+        const int i = c0 + st * WAVE + lane;
+        float v = i < c1 ? __builtin_amdgcn_exp2f((row[i] - mx) * scale2) : 0.f;
+        v = wave_sum(v);
+        if (lane == 0) out[2 + st] = v;
+        total += v;
+    }
+    if (lane == 0) wave_tot[wave] = total;
     __syncthreads();
     if (tid == 0) {
-        float r;
+        out[0] = mx;
+        out[1] = wave_tot[0] + wave_tot[1] + wave_tot[2] + wave_tot[3];
+    }
+}
+
+__global__ __launch_bounds__(64) void sample_final_kernel(const float* __restrict__ logits, int V, int chunk,
+                                                          int n_chunks, float temperature,
+                                                          const float* __restrict__ ws,
+                                                          const int* __restrict__ seq_slot,
+                                                          unsigned long long* __restrict__ state,
+                                                          const float* __restrict__ forced_r,
+                                                          int* __restrict__ out) {
+    const int lane = threadIdx.x;
+    const float* row = logits + (int64_t)blockIdx.x * V;
+    const int steps = chunk >> 6;
+    const float* part = ws + (int64_t)blockIdx.x * n_chunks * (2 + steps);
+    const float scale2 = LOG2E_F / temperature;
+    float r = 0.f;
+    if (lane == 0) {
         if (forced_r) r = forced_r[blockIdx.x];
         else {
             unsigned long long* st = state + 2 * (int64_t)seq_slot[blockIdx.x];
             r = uniform01(st[0], st[1]);
             st[1] += 1;
         }
-        float total = 0.f;
-        for (int i = 0; i < nt; ++i) total += sums[i];
-        const float target = r * total;
-        float c = 0.f;
-        int owner = -1;
-        for (int i = 0; i < nt; ++i) {
-            if (target < c + sums[i]) { owner = i; break; }
-            c += sums[i];
-        }
-        if (owner >= 0) {
-            const int b0 = min(V, owner * chunk), b1 = min(V, b0 + chunk);
-            int pick = b1 - 1;
-            for (int i = b0; i < b1; ++i) {
-                c += expf((row[i] - mx) / temperature);
-                if (target < c) { pick = i; break; }
-            }
-            found = pick;
-        }
-        out[blockIdx.x] = found;
     }
+    r = __shfl(r, 0, WAVE);
+    // the chunks, one a lane (n_chunks <= 64)
+    const bool have = lane < n_chunks;
+    const float m_c = have ? part[(int64_t)lane * (2 + steps)] : -INFINITY;
+    const float mx = wave_max(m_c);
+    const float f_c = have ? __builtin_amdgcn_exp2f((m_c - mx) * scale2) : 0.f;
+    const float w_c = have ? part[(int64_t)lane * (2 + steps) + 1] * f_c : 0.f;
+    float incl = wave_inclusive_scan(w_c, lane);
+    const float target = r * __shfl(incl, WAVE - 1, WAVE);
+    unsigned long long hit = __builtin_amdgcn_ballot_w64(have && target < incl);
+    const int c = hit ? __builtin_ctzll(hit) : n_chunks - 1;
+    // from here on in the chunk's own scale: sums of exp((l - m_c) / T)
+    const float f_own = __shfl(f_c, c, WAVE);
+    float left = (target - __shfl(incl - w_c, c, WAVE)) / f_own;      // what the chunk still has to cover
+    const float* sums = part + (int64_t)c * (2 + steps) + 2;
+    const int c0 = c * chunk, c1 = min(V, c0 + chunk);
+    const int live_steps = (c1 - c0 + WAVE - 1) >> 6;
+    int step = live_steps - 1;
+    for (int base = 0; base < live_steps; base += WAVE) {
+        const bool in = base + lane < live_steps;
+        const float sv = in ? sums[base + lane] : 0.f;
+        incl = wave_inclusive_scan(sv, lane);
+        hit = __builtin_amdgcn_ballot_w64(in && left < incl);
+        if (hit) {
+            const int f = __builtin_ctzll(hit);
+            step = base + f;
+            left -= __shfl(incl - sv, f, WAVE);
+            break;
+        }
+        if (base + WAVE < live_steps) left -= __shfl(incl, WAVE - 1, WAVE);
+        else left -= __shfl(incl - sv, live_steps - 1 - base, WAVE);        // nothing hit: search the last step
+    }
+    const int e0 = c0 + step * WAVE, i = e0 + lane;
+    const float m_own = __shfl(m_c, c, WAVE);
+    const float e = i < c1 ? __builtin_amdgcn_exp2f((row[i] - m_own) * scale2) : 0.f;
+    incl = wave_inclusive_scan(e, lane);
+    hit = __builtin_amdgcn_ballot_w64(i < c1 && left < incl);
+    const int pick = hit ? e0 + __builtin_ctzll(hit) : min(c1, e0 + WAVE) - 1;
+    if (lane == 0) out[blockIdx.x] = pick;
 }
 
 // part_v, part_i: workspace of n_rows * li_argmax_chunks(V) entries each
@@ -140,13 +201,26 @@ extern "C" int li_argmax(const float* logits, int n_rows, int V, float* part_v, 
     return LI_OK;
 }
 
+// chunk of a row for li_sample (a multiple of 64, at most 64 chunks) and the floats of workspace a row needs
+extern "C" int li_sample_chunk(int V) {
+    const int chunk = V <= 64 * 4096 ? 4096 : (V + 63) / 64;
+    return (min(chunk, max(V, 1)) + 63) / 64 * 64;
+}
+extern "C" int li_sample_ws_floats(int V) {
+    const int chunk = li_sample_chunk(V);
+    return ((V + chunk - 1) / chunk) * (2 + chunk / 64);
+}
+
 extern "C" int li_sample(const float* logits, int n_rows, int V, float temperature, const int* seq_slot,
-                         void* state, const float* forced_r, int* out, hipStream_t stream) {
+                         void* state, const float* forced_r, float* ws, int* out, hipStream_t stream) {
     if (n_rows <= 0) return LI_OK;
-    if (V <= 0 || temperature <= 0.f) return LI_BAD_ARG;             // greedy goes through li_argmax
+    if (V <= 0 || temperature <= 0.f || !ws) return LI_BAD_ARG;      // greedy goes through li_argmax
     if (!forced_r && (!seq_slot || !state)) return LI_BAD_ARG;
-    sample_kernel<<<n_rows, V >= 4096 ? 1024 : 256, 0, stream>>>(logits, V, temperature, seq_slot,
-                                                                  (unsigned long long*)state, forced_r, out);
+    const int chunk = li_sample_chunk(V), n_chunks = (V + chunk - 1) / chunk;
+    sample_chunks_kernel<<<dim3(n_rows, n_chunks), 256, 0, stream>>>(logits, V, chunk, temperature, ws);
+    LI_CHECK_LAUNCH();
+    sample_final_kernel<<<n_rows, 64, 0, stream>>>(logits, V, chunk, n_chunks, temperature, ws, seq_slot,
+                                                   (unsigned long long*)state, forced_r, out);
     LI_CHECK_LAUNCH();
     return LI_OK;
 }

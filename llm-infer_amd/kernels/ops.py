@@ -527,8 +527,9 @@ def sample(logits, temperature: float, seq_slot=None, state=None, forced_r=None,
               "state: int64 [slots, 2]")
     if forced_r is not None:
         _need(forced_r.dtype == torch.float32 and forced_r.numel() >= b, "forced_r: float32 [B]")
+    ws = torch.empty((b * core().li_sample_ws_floats(logits.shape[1]),), dtype=torch.float32, device=logits.device)
     _check(core().li_sample(_ptr(logits), b, logits.shape[1], c_float(temperature), _ptr(seq_slot), _ptr(state),
-                            _ptr(forced_r), _ptr(out), _stream()), "sample")
+                            _ptr(forced_r), _ptr(ws), _ptr(out), _stream()), "sample")
     return out
 
 

@@ -410,16 +410,14 @@ def test_rotation_fused_into_the_projection(ops, dt, T, H, K, hd, rot, d):
 def test_sampling_kernels(ops):
     import plain_llama as P
     g = torch.Generator().manual_seed(0)
-    for V in (256, 331, 5000, 128256):
+    for V in (7, 64, 65, 256, 331, 5000, 128256, 300007):      # one chunk, 32 chunks, chunks longer than 4,096
         logits = torch.randn(6, V, generator=g) * 3
-        logits[1, 7] = logits[1, 200] = 50.0                      # a tie: the first wins
+        logits[1, 3] = logits[1, V - 2] = 50.0                    # a tie: the first wins
         logits[2, V - 1] = 60.0
         d = logits.to(DEV)
         got = ops.argmax(d).tolist()
         assert got == [P.sample_greedy(r) for r in logits]
-        assert got[1] == 7 and got[2] == V - 1
-        if V > 5000:
-            continue
+        assert got[1] == 3 and got[2] == V - 1
         for T in (0.8, 2.0):
             rs = [0.0, 0.25, 0.5, 0.75, 0.999, 0.9999999]
             r = torch.tensor(rs, dtype=torch.float32, device=DEV)
