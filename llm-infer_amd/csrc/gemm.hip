@@ -26,9 +26,18 @@ __global__ __launch_bounds__(256) void gemm_fma_kernel(const TX* __restrict__ X,
     const int tid = threadIdx.x;
     const int tx = tid & 15, ty = tid >> 4;
     const int m0 = blockIdx.y * BT, n0 = blockIdx.x * BT;
-    float acc[4][4] = {};
+    // Every sum is taken in the same order whatever the batch: FMA chains over 256 consecutive k, the
+    // chains added up in ascending order (a single chain over a K of tens of thousands would lose
+    // several bits more than a blocked library product does).
+    float acc[4][4] = {}, total[4][4] = {};
     const int lr = tid >> 2, lk = (tid & 3) * 4;     // row of the tile and first k this thread loads
     for (int k0 = 0; k0 < K; k0 += BK) {
+        if (k0 && (k0 & 255) == 0) {
+#pragma unroll
+            for (int i = 0; i < 4; ++i)
+#pragma unroll
+                for (int j = 0; j < 4; ++j) { total[i][j] += acc[i][j]; acc[i][j] = 0.f; }
+        }
 #pragma unroll
         for (int j = 0; j < 4; ++j) {
             const int k = k0 + lk + j;
@@ -50,7 +59,11 @@ __global__ __launch_bounds__(256) void gemm_fma_kernel(const TX* __restrict__ X,
         __syncthreads();
     }
 #pragma unroll
-    for (int i = 0; i < 4; ++i) epilogue4(e, m0 + ty * 4 + i, n0 + tx * 4, acc[i]);
+    for (int i = 0; i < 4; ++i) {
+#pragma unroll
+        for (int j = 0; j < 4; ++j) total[i][j] += acc[i][j];
+        epilogue4(e, m0 + ty * 4 + i, n0 + tx * 4, total[i]);
+    }
 }
 
 // ===========================================================================
