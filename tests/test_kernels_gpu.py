@@ -418,7 +418,7 @@ def test_sampling_kernels(ops):
         got = ops.argmax(d).tolist()
         assert got == [P.sample_greedy(r) for r in logits]
         assert got[1] == 3 and got[2] == V - 1
-        for T in (0.8, 2.0):
+        for T in (0.01, 0.8, 2.0, 1e6):             # from nearly only the maximum to nearly equal chances
             rs = [0.0, 0.25, 0.5, 0.75, 0.999, 0.9999999]
             r = torch.tensor(rs, dtype=torch.float32, device=DEV)
             got = ops.sample(d, T, forced_r=r).tolist()
