@@ -77,6 +77,14 @@ __device__ __forceinline__ float block_max(float v, float* scratch) {
     return t;
 }
 
+// The gate's activation: silu(x) = x / (1 + exp(-x)) (include/kernels_cpu.hpp:186) or the tanh form of
+// gelu that the reference computes, 0.5 x (1 + tanh(sqrt(2 / pi) (x + 0.044715 x^3)))
+// (include/kernels_cpu.hpp:179-184).
+__device__ __forceinline__ float gate_activation(float g, bool gelu) {
+    if (gelu) return 0.5f * g * (1.f + tanhf(0.7978845608028654f * (g + 0.044715f * g * g * g)));
+    return g / (1.f + expf(-g));
+}
+
 // ---------------------------------------------------------------------------
 // Layout of a cache page.  A page holds PAGE (64) tokens of one layer for all
 // KV heads.  Keys and values are stored in the order in which a wave's lanes

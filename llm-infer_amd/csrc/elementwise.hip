@@ -241,16 +241,13 @@ extern "C" int li_decode_prepare(const int* seq_slot, int* lens, int* pos, int* 
 
 // out[i] = act(gate[i]) * up[i] for separate gate and up rows:  gu [T, 2F] float32 with
 // gate_j at column 2j and up_j at column 2j+1  ->  h [T, F].  (src/model/block.cpp:203-214)
-// act: silu, x / (1 + exp(-x)), or the reference's gelu, 0.5 x (1 + tanh(sqrt(2/pi) (x + 0.044715 x^3)))
-// (include/kernels_cpu.hpp:179-186).
+// act: gate_activation of common.h (silu, or the reference's gelu).
 template <class T>
 __global__ void swiglu_kernel(const float* __restrict__ gu, T* __restrict__ h, int64_t n, int gelu) {
     const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
     if (i >= n) return;
     const float g = gu[2 * i], u = gu[2 * i + 1];
-    const float a = gelu ? 0.5f * g * (1.f + tanhf(0.7978845608028654f * (g + 0.044715f * g * g * g)))
-                         : g / (1.f + expf(-g));
-    h[i] = from_f32<T>(a * u);
+    h[i] = from_f32<T>(gate_activation(g, gelu != 0) * u);
 }
 
 extern "C" int li_swiglu(const float* gu, void* h, int dt, int64_t n, int gelu, hipStream_t stream) {

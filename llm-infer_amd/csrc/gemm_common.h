@@ -5,14 +5,6 @@
 
 enum { EPI_STORE = 0, EPI_ADD = 1, EPI_SWIGLU = 2, EPI_ROPE = 3, EPI_GEGLU = 4 };
 
-// The gate's activation: silu(x) = x / (1 + exp(-x)) (include/kernels_cpu.hpp:186) or the tanh form of
-// gelu that the reference computes, 0.5 x (1 + tanh(sqrt(2 / pi) (x + 0.044715 x^3)))
-// (include/kernels_cpu.hpp:179-184).
-__device__ __forceinline__ float gate_activation(float g, bool gelu) {
-    if (gelu) return 0.5f * g * (1.f + tanhf(0.7978845608028654f * (g + 0.044715f * g * g * g)));
-    return g / (1.f + expf(-g));
-}
-
 // What the EPI_ROPE epilogue needs: the columns of the product are the q heads, then the k heads,
 // then the v heads of a token; q and k are rotated by the token's position (adjacent pairs), q goes
 // to q_out [M, H, hd], k and v into the token's cache page.
