@@ -188,6 +188,36 @@ def test_decode_splits_fill_the_chip_and_are_powers_of_two():
     assert decode_splits(1, 8, 32, 100) == 1 and decode_splits(1, 1, 64, 640) == 4
 
 
+def test_launch_plans_cover_every_product_once():
+    """What the planner of the prefill GEMM hands the kernel: launches that tile the product without
+    gap or overlap, a first part that ends on the large tile's grid, K split only for a whole product."""
+    import random as _r
+
+    from llm_infer_amd.kernels.ops import _DMA_TILES, _dma_plan
+    rng = _r.Random(0)
+    shapes = [(2048, 28672, 4096), (33186, 2048, 8192), (3000, 6144, 4096), (97, 4096, 14336), (130, 128256, 4096)]
+    shapes += [(rng.randint(97, 40000), 16 * rng.randint(1, 2000), 32 * rng.randint(1, 500)) for _ in range(300)]
+    for m, n, k in shapes:
+        plan = _dma_plan(m, n, k)
+        assert 1 <= len(plan) <= 2
+        covered = 0
+        for tile, splits, n_begin, n_count, m_begin, m_count in plan:
+            bn, bm = _DMA_TILES[tile]
+            cols, rows = n_count or n - n_begin, m_count or m - m_begin
+            assert 0 <= n_begin < n and 0 <= m_begin < m and n_begin % 16 == 0
+            assert n_begin + cols <= n and m_begin + rows <= m
+            assert splits >= 1 and (splits == 1 or (len(plan) == 1 and k // splits >= 1024))
+            if n_begin + cols < n:
+                assert cols % bn == 0             # only the last columns may end inside a tile
+            if m_begin + rows < m:
+                assert rows % bm == 0
+            covered += cols * rows
+        assert covered == m * n, (m, n, k, plan)
+        if len(plan) == 2:
+            (_, _, nb0, nc0, mb0, mc0), (_, _, nb1, _, mb1, _) = plan
+            assert (nb0, mb0) == (0, 0) and ((nb1 == nc0 and mb1 == 0 and mc0 == 0) or (mb1 == mc0 and nb1 == 0 and nc0 == 0))
+
+
 def test_command_line_follows_the_reference():
     c = parse_args(["m", "-i", "hi", "-n", "5", "-t", "0.5", "--seed", "7", "-T", "99"])
     assert (c["model"], c["prompt"], c["max_tokens"], c["temperature"], c["seed"], c["context"]) == \
