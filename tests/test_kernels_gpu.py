@@ -168,6 +168,20 @@ def test_gate_activation_alone(ops):
         assert ops.swiglu(gu, torch.bfloat16, gelu=gelu).dtype == torch.bfloat16
 
 
+@pytest.mark.parametrize("M,N,K", [(2048, 28672, 2048), (33186, 2048, 2048)])
+def test_products_that_end_with_a_smaller_tile(ops, M, N, K):
+    """Sizes at which the planner itself splits a product: the large tile for the columns (or rows) that
+    fill whole rounds of workgroups, a smaller tile for the rest."""
+    assert len(ops._dma_plan(M, N, K)) == 2
+    g = torch.Generator().manual_seed(M + N)
+    x = torch.randn(M, K, generator=g).to(torch.float16).to(DEV)
+    w = (torch.randn(N, K, generator=g) / math.sqrt(K)).to(torch.float16).to(DEV)
+    out = ops.linear(x, ops.tile_weight(w), out_dtype=torch.float32)
+    for r0 in range(0, M, 4096):                       # the reference in slices: it is float64
+        ref = x[r0:r0 + 4096].double() @ w.double().t()
+        assert (out[r0:r0 + 4096].double() - ref).abs().max().item() < 2e-4 * (1 + ref.abs().max().item())
+
+
 def test_linear_rows_do_not_depend_on_the_batch_in_float32(ops):
     g = torch.Generator().manual_seed(1)
     x = torch.randn(70, 136, generator=g).to(DEV)
