@@ -200,35 +200,7 @@ def linear(x: torch.Tensor, w, mode: int = EPI_STORE, out: torch.Tensor | None =
         return out
     if kind.startswith("dma"):
         _need(tiled and fast_ok and m * k * 2 < (1 << 32), "gemm_dma: a tiled weight, X below 4 GiB")
-        parts = kind.split(":")
-        if parts[0] == "dma2":                             # "dma2:<tile>:<columns>:<tile of the rest>" for tests
-            plan = [(int(parts[1]), 1, 0, int(parts[2]), 0, 0), (int(parts[3]), 1, int(parts[2]), 0, 0, 0)]
-        elif parts[0] == "dmarows":                        # "dmarows:<tile>:<rows>:<tile of the rest>" for tests
-            plan = [(int(parts[1]), 1, 0, 0, 0, int(parts[2])), (int(parts[3]), 1, 0, 0, int(parts[2]), 0)]
-        elif len(parts) > 1:                               # "dma:<tile>[:<splits>]"
-            plan = [(int(parts[1]), int(parts[2]) if len(parts) > 2 else 1, 0, 0, 0, 0)]
-        else:
-            plan = _dma_plan(m, n, k)
-        esize = {0: 4, 1: 2, 2: 2}
-        for tile, splits, n_begin, n_count, m_begin, m_count in plan:
-            rows = m_count or m - m_begin
-            _need(0 <= m_begin < m and m_begin + rows <= m, "gemm_dma: rows outside the product")
-            ws = _workspace(splits * rows * n, x.device) if splits > 1 else None
-            xp = c_void_p(x.data_ptr() + m_begin * k * x.element_size())
-            op = c_void_p(out.data_ptr() + m_begin * n_out * out.element_size()) if out is not None else c_void_p(0)
-            rp = rs
-            if _rope is not None and m_begin:
-                # the epilogue's per-row arrays and q, for the rows of this launch
-                shifted = _RopeStore()
-                ctypes.pointer(shifted)[0] = _rope
-                half = _rope.rotary_dim // 2
-                for field, step in (("pos", 4), ("tok_slot", 4), ("cos_sin", half * 2 * 4),
-                                    ("q_out", _rope.H * _rope.hd * esize[_rope.dt])):
-                    v = getattr(_rope, field)
-                    setattr(shifted, field, v + m_begin * step if v else v)
-                rp = ctypes.byref(shifted)
-            _check(lib.li_gemm_dma(xp, _ptr(wd), DT[x.dtype], op, out_dt, mode, rows, n, k, tile, splits,
-                                   _ptr(ws), rp, n_begin, n_count, _stream()), "gemm_dma")
+        _run_dma(x, wd, out, out_dt, mode, m, n, k, n_out, _forced_dma_plan(kind) or _dma_plan(m, n, k), _rope)
         return out
     if kind == "fma":
         _check(lib.li_gemm_fma(_ptr(x), DT[x.dtype], _ptr(w), DT[w.dtype], _ptr(out), out_dt, mode,
@@ -261,6 +233,45 @@ def linear(x: torch.Tensor, w, mode: int = EPI_STORE, out: torch.Tensor | None =
         _check(lib.li_gemm_mfma(_ptr(x), _ptr(wd), int(tiled), DT[x.dtype], _ptr(out), out_dt, mode, m, n, k,
                                 tile, splits, _ptr(ws), rs, _stream()), "gemm_mfma")
     return out
+
+
+def _forced_dma_plan(kind: str):
+    """The plan that a test asks for: "dma:<tile>[:<splits>]", "dma2:<tile>:<columns>:<tile of the rest>",
+    "dmarows:<tile>:<rows>:<tile of the rest>"; None for plain "dma" (the planner decides)."""
+    parts = kind.split(":")
+    if parts[0] == "dma2":
+        return [(int(parts[1]), 1, 0, int(parts[2]), 0, 0), (int(parts[3]), 1, int(parts[2]), 0, 0, 0)]
+    if parts[0] == "dmarows":
+        return [(int(parts[1]), 1, 0, 0, 0, int(parts[2])), (int(parts[3]), 1, 0, 0, int(parts[2]), 0)]
+    if len(parts) > 1:
+        return [(int(parts[1]), int(parts[2]) if len(parts) > 2 else 1, 0, 0, 0, 0)]
+    return None
+
+
+def _run_dma(x, wd, out, out_dt, mode, m, n, k, n_out, plan, rope) -> None:
+    """The launches of a plan (`_dma_plan`): each covers a range of columns and of rows of the product;
+    a launch that does not start at row 0 gets X, the output and the rotation epilogue's per-row
+    arrays from its first row on."""
+    lib = core()
+    element_bytes = {0: 4, 1: 2, 2: 2}                     # by dtype code
+    for tile, splits, n_begin, n_count, m_begin, m_count in plan:
+        rows = m_count or m - m_begin
+        _need(0 <= m_begin < m and m_begin + rows <= m, "gemm_dma: rows outside the product")
+        ws = _workspace(splits * rows * n, x.device) if splits > 1 else None
+        xp = c_void_p(x.data_ptr() + m_begin * k * x.element_size())
+        op = c_void_p(out.data_ptr() + m_begin * n_out * out.element_size()) if out is not None else c_void_p(0)
+        rp = ctypes.byref(rope) if rope is not None else None
+        if rope is not None and m_begin:
+            shifted = _RopeStore()
+            ctypes.pointer(shifted)[0] = rope
+            per_row = (("pos", 4), ("tok_slot", 4), ("cos_sin", rope.rotary_dim // 2 * 2 * 4),
+                       ("q_out", rope.H * rope.hd * element_bytes[rope.dt]))
+            for field, step in per_row:
+                v = getattr(rope, field)
+                setattr(shifted, field, v + m_begin * step if v else v)
+            rp = ctypes.byref(shifted)
+        _check(lib.li_gemm_dma(xp, _ptr(wd), DT[x.dtype], op, out_dt, mode, rows, n, k, tile, splits,
+                               _ptr(ws), rp, n_begin, n_count, _stream()), "gemm_dma")
 
 
 def _stream_shape(n: int, k: int) -> tuple[int, int]:
