@@ -185,6 +185,27 @@ __global__ __launch_bounds__(64) void sample_final_kernel(const float* __restric
     if (lane == 0) out[blockIdx.x] = pick;
 }
 
+// Probability of one given token of each row: softmax at temperature 1 (tools/infer.cpp:77-81; a token
+// outside the vocabulary has probability 0).  Reads the chunk maxima and sums that
+// sample_chunks_kernel left at temperature 1.
+__global__ __launch_bounds__(64) void token_prob_kernel(const float* __restrict__ logits, int V, int chunk,
+                                                        int n_chunks, const float* __restrict__ ws,
+                                                        const int* __restrict__ tokens, float* __restrict__ out) {
+    const int lane = threadIdx.x;
+    const int steps = chunk >> 6;
+    const float* part = ws + (int64_t)blockIdx.x * n_chunks * (2 + steps);
+    const bool have = lane < n_chunks;
+    const float m_c = have ? part[(int64_t)lane * (2 + steps)] : -INFINITY;
+    const float mx = wave_max(m_c);
+    const float total = wave_sum(have ? part[(int64_t)lane * (2 + steps) + 1] * __builtin_amdgcn_exp2f((m_c - mx) * LOG2E_F)
+                                      : 0.f);
+    if (lane == 0) {
+        const int t = tokens[blockIdx.x];
+        out[blockIdx.x] = (t >= 0 && t < V)
+            ? __builtin_amdgcn_exp2f((logits[(int64_t)blockIdx.x * V + t] - mx) * LOG2E_F) / total : 0.f;
+    }
+}
+
 // part_v, part_i: workspace of n_rows * li_argmax_chunks(V) entries each
 extern "C" int li_argmax_chunks(int V) { return V <= 4096 ? 1 : (V + 4095) / 4096; }
 
@@ -221,6 +242,19 @@ extern "C" int li_sample(const float* logits, int n_rows, int V, float temperatu
     LI_CHECK_LAUNCH();
     sample_final_kernel<<<n_rows, 64, 0, stream>>>(logits, V, chunk, n_chunks, temperature, ws, seq_slot,
                                                    (unsigned long long*)state, forced_r, out);
+    LI_CHECK_LAUNCH();
+    return LI_OK;
+}
+
+// out[r] = softmax(logits[r])[tokens[r]]; ws as for li_sample
+extern "C" int li_token_prob(const float* logits, int n_rows, int V, const int* tokens, float* ws, float* out,
+                             hipStream_t stream) {
+    if (n_rows <= 0) return LI_OK;
+    if (V <= 0 || !logits || !tokens || !ws || !out) return LI_BAD_ARG;
+    const int chunk = li_sample_chunk(V), n_chunks = (V + chunk - 1) / chunk;
+    sample_chunks_kernel<<<dim3(n_rows, n_chunks), 256, 0, stream>>>(logits, V, chunk, 1.0f, ws);
+    LI_CHECK_LAUNCH();
+    token_prob_kernel<<<n_rows, 64, 0, stream>>>(logits, V, chunk, n_chunks, ws, tokens, out);
     LI_CHECK_LAUNCH();
     return LI_OK;
 }

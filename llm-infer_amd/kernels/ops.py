@@ -544,6 +544,20 @@ def sample(logits, temperature: float, seq_slot=None, state=None, forced_r=None,
     return out
 
 
+def token_prob(logits: torch.Tensor, tokens: torch.Tensor) -> torch.Tensor:
+    """softmax(logits[r])[tokens[r]] at temperature 1, float32 [B]; 0 for a token outside the vocabulary
+    (tools/infer.cpp:77-81)."""
+    _dev(logits, tokens)
+    _need(logits.dtype == torch.float32 and logits.dim() == 2, "logits: float32 [B, V]")
+    b = logits.shape[0]
+    _need(tokens.dtype == torch.int32 and tokens.numel() == b, "tokens: int32 [B]")
+    out = torch.empty((b,), dtype=torch.float32, device=logits.device)
+    ws = torch.empty((b * core().li_sample_ws_floats(logits.shape[1]),), dtype=torch.float32, device=logits.device)
+    _check(core().li_token_prob(_ptr(logits), b, logits.shape[1], _ptr(tokens), _ptr(ws), _ptr(out), _stream()),
+           "token_prob")
+    return out
+
+
 def uniform01(key: int, counter: int) -> float:
     """The generator's value for (key, counter), computed on the host by the same function."""
     return float(core().li_uniform01(c_uint64(key & (2 ** 64 - 1)), c_uint64(counter & (2 ** 64 - 1))))

@@ -39,6 +39,11 @@ class Sampler:
             return ops.argmax(logits, out)
         return ops.sample(logits, self.temperature, seq_slot, cache.seq_state, out=out)
 
+    @staticmethod
+    def token_prob(logits: torch.Tensor, tokens: torch.Tensor) -> torch.Tensor:
+        """Probability of tokens[r] under softmax(logits[r]) at temperature 1 (infer.cpp:77-81)."""
+        return ops.token_prob(logits, tokens)
+
     def uniform(self, request_index: int, n: int) -> float:
         """The n-th uniform number of a request's stream (host twin of the device generator)."""
         return ops.uniform01(request_key(self.seed, request_index), n)

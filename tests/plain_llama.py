@@ -189,6 +189,11 @@ def probabilities(logits: torch.Tensor, temperature: float) -> torch.Tensor:
     return e / e.sum()
 
 
+def token_prob(logits: torch.Tensor, token: int) -> float:
+    """Probability of one token at temperature 1; 0 outside the vocabulary (tools/infer.cpp:77-81)."""
+    return probabilities(logits, 1.0)[token].item() if 0 <= token < logits.numel() else 0.0
+
+
 def sample_temperature(logits: torch.Tensor, temperature: float, r: float) -> int:
     """argmax if T <= 0, else the first i with r < cumsum_i, fallback V-1 (infer.cpp:40-61)."""
     if temperature <= 0.0:

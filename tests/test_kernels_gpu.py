@@ -421,6 +421,25 @@ def test_rotation_fused_into_the_projection(ops, dt, T, H, K, hd, rot, d):
                 assert (b != 0).sum().item() >= 0.9 * T * 2 * K * hd
 
 
+def test_token_probability(ops):
+    import plain_llama as P
+    g = torch.Generator().manual_seed(5)
+    for V in (7, 65, 331, 5000, 128256, 300007):
+        logits = torch.randn(5, V, generator=g) * 4
+        logits[0, V // 2] = 40.0                                   # nearly all the mass on one token
+        tokens = [V // 2, 0, V - 1, V, -1]                         # the last two lie outside the vocabulary
+        got = ops.token_prob(logits.to(DEV), torch.tensor(tokens, dtype=torch.int32, device=DEV)).cpu()
+        want = torch.tensor([P.token_prob(logits[i].double(), t) for i, t in enumerate(tokens)])
+        assert got[3] == 0 and got[4] == 0
+        torch.testing.assert_close(got, want.float(), rtol=2e-5, atol=1e-12)
+        assert got[0] > 0.999
+        # all tokens of a row add up to one
+        row = logits[1:2].expand(V, V).contiguous().to(DEV) if V <= 331 else None
+        if row is not None:
+            every = ops.token_prob(row, torch.arange(V, dtype=torch.int32, device=DEV))
+            assert abs(every.double().sum().item() - 1.0) < 1e-5
+
+
 def test_sampling_kernels(ops):
     import plain_llama as P
     g = torch.Generator().manual_seed(0)

@@ -209,6 +209,8 @@ def test_sampling_rules():
     assert P.sample_temperature(l, 0.8, float(p[0]) + 1e-4) == 1
     assert P.sample_temperature(l, 0.8, 0.99999999) == 3
     assert P.sample_temperature(l, 1e-4, 0.9) in (1, 2)
+    assert abs(P.token_prob(l, 3) - torch.softmax(l, 0)[3].item()) < 1e-7       # temperature 1, whatever the sampler's
+    assert P.token_prob(l, 4) == 0.0 and P.token_prob(l, -1) == 0.0
 
 
 def test_generate_stops_before_keeping_the_stop_token():
