@@ -13,17 +13,18 @@ __version__ = "0.1.0"
 register_architecture("LlamaForCausalLM", LlamaConfig)
 
 
-def load(folder: str, dtype: str = "bfloat16", max_tokens: int = 8192, n_slots=None):
+def load(folder: str, dtype: str = "bfloat16", max_tokens: int = 8192, n_slots=None, kv_round=None):
     """Open a model on the GPU: a folder with config.json and model.safetensors, or a GGUF file
-    with unquantized tensors (the reference's own format) or the folder that holds one."""
+    with unquantized tensors (the reference's own format) or the folder that holds one.
+    ``kv_round="float16"`` with ``dtype="float32"`` rounds keys and values as the reference's cache does."""
     from .engine import Engine
-    return Engine.from_folder(folder, dtype=dtype, max_tokens=max_tokens, n_slots=n_slots)
+    return Engine.from_folder(folder, dtype=dtype, max_tokens=max_tokens, n_slots=n_slots, kv_round=kv_round)
 
 
-def random_model(config, seed: int = 0, dtype: str = "bfloat16", max_tokens: int = 8192, n_slots=None):
+def random_model(config, seed: int = 0, dtype: str = "bfloat16", max_tokens: int = 8192, n_slots=None, kv_round=None):
     """An engine with random weights made on the GPU from a configuration and a seed."""
     from .engine import Engine
-    return Engine.from_random(config, seed=seed, dtype=dtype, max_tokens=max_tokens, n_slots=n_slots)
+    return Engine.from_random(config, seed=seed, dtype=dtype, max_tokens=max_tokens, n_slots=n_slots, kv_round=kv_round)
 
 
 def write_random_model(folder: str, config, seed: int = 0, dtype: str = "bfloat16") -> None:

@@ -39,6 +39,7 @@ class KVView:
     page_stride: int           # elements from one page to the next
     page_table: torch.Tensor   # int32 [slots, pages per sequence]
     spec: KVSpec
+    round_to: torch.dtype | None = None   # keys and values take this type's values before they are stored
 
     def as_tuple(self):
         return (self.k, self.v, self.page_stride, self.page_table)
@@ -51,8 +52,8 @@ class StateView:
 
 
 class KVGroup:
-    def __init__(self, spec: KVSpec, entries, n_slots, n_pages, max_positions, dtype, device):
-        self.spec, self.entries = spec, list(entries)
+    def __init__(self, spec: KVSpec, entries, n_slots, n_pages, max_positions, dtype, device, round_to=None):
+        self.spec, self.entries, self.round_to = spec, list(entries), round_to
         self.k_elems = spec.n_kv_heads * PAGE * spec.head_dim
         self.v_elems = spec.n_kv_heads * PAGE * _round_up(spec.head_dim, 32)
         self.layer_elems = self.k_elems + self.v_elems
@@ -77,7 +78,7 @@ class KVGroup:
         flat = self.storage.view(-1)
         k = flat[i * self.layer_elems:]
         v = flat[i * self.layer_elems + self.k_elems:]
-        return KVView(k, v, self.page_elems, self.page_table, self.spec)
+        return KVView(k, v, self.page_elems, self.page_table, self.spec, self.round_to)
 
     def first_needed_page(self, length: int) -> int:
         """First page that a token at position ``length`` (the next one) still reads."""
@@ -155,7 +156,10 @@ class Cache:
     ``max_tokens`` bounds the tokens all live sequences hold together, each sequence's count
     rounded up to a whole page."""
 
-    def __init__(self, specs, max_tokens: int, max_positions: int, dtype, device, n_slots: int | None = None):
+    def __init__(self, specs, max_tokens: int, max_positions: int, dtype, device, n_slots: int | None = None,
+                 kv_round=None):
+        if kv_round is not None and (dtype != torch.float32 or kv_round not in (torch.float16, torch.bfloat16)):
+            raise CacheError("kv_round: float16 or bfloat16, for a float32 cache (a 16-bit cache rounds to its own type)")
         self.max_positions = max_positions
         self.n_pages = max(1, (max_tokens + PAGE - 1) // PAGE) + 1          # page 0 is never handed out
         self.n_slots = n_slots or max(1, min(self.n_pages - 1, 4096))
@@ -170,7 +174,7 @@ class Cache:
                 by_spec.setdefault(s, []).append(i)
         for s, entries in by_spec.items():
             if isinstance(s, KVSpec):
-                g = KVGroup(s, entries, self.n_slots, self.n_pages, max_positions, dtype, device)
+                g = KVGroup(s, entries, self.n_slots, self.n_pages, max_positions, dtype, device, kv_round)
             elif isinstance(s, StateSpec):
                 g = StateGroup(s, entries, self.n_slots, device)
             else:

@@ -31,6 +31,7 @@ Options:
   -T <int>              Context length override (default: model max)
   --seed <int>          Random seed (default: 0)
   --dtype <name>        bfloat16 (default), float16 or float32
+  --kv-round <name>     With --dtype float32: keys and values rounded to float16 (the reference's cache) or bfloat16
   --slots <int>         Most sequences that run as one batch (default: all requests given)
   --random-weights      Ignore the model's tensors: random weights from --seed-weights
   --seed-weights <int>  Seed of the random weights (default: 0)
@@ -45,7 +46,7 @@ def parse_ids(text: str) -> list:
 def parse_args(argv):
     cfg = dict(model=None, device="hip", prompt=None, prompt_file=None, tokens=[], tokens_file=None,
                max_tokens=256, temperature=1.0, seed=0, context=None, dtype="bfloat16", random=False,
-               seed_weights=0, graph=True, help=False, slots=None, config=None)
+               seed_weights=0, graph=True, help=False, slots=None, config=None, kv_round=None)
     if any(a in ("-h", "--help") for a in argv):
         cfg["help"] = True
         return cfg
@@ -55,7 +56,7 @@ def parse_args(argv):
     takes = {"-d": ("device", str), "-i": ("prompt", str), "-f": ("prompt_file", str), "-n": ("max_tokens", int),
              "-t": ("temperature", float), "-T": ("context", int), "--seed": ("seed", int),
              "--dtype": ("dtype", str), "--tokens-file": ("tokens_file", str), "--seed-weights": ("seed_weights", int),
-             "--slots": ("slots", int), "--config": ("config", str)}
+             "--slots": ("slots", int), "--config": ("config", str), "--kv-round": ("kv_round", str)}
     i = 1
     while i < len(argv):
         a = argv[i]
@@ -142,9 +143,10 @@ def run(cfg) -> int:
     need = sum(each[:n_slots])                       # the largest batch that can be live at once
     if cfg["random"]:
         engine = Engine.from_random(config, seed=cfg["seed_weights"], dtype=cfg["dtype"], max_tokens=need,
-                                    n_slots=n_slots)
+                                    n_slots=n_slots, kv_round=cfg["kv_round"])
     else:
-        engine = Engine.from_folder(cfg["model"], dtype=cfg["dtype"], max_tokens=need, n_slots=n_slots)
+        engine = Engine.from_folder(cfg["model"], dtype=cfg["dtype"], max_tokens=need, n_slots=n_slots,
+                                    kv_round=cfg["kv_round"])
         engine.config = config
         if cfg["context"]:
             engine.max_positions = min(engine.max_positions, cfg["context"])

@@ -133,7 +133,7 @@ __global__ void rope_store_kernel(const float* __restrict__ qkv, int row_stride,
                                   const int* __restrict__ pos, const int* __restrict__ tok_slot,
                                   const int* __restrict__ page_table, int max_pages, int64_t page_stride,
                                   T* __restrict__ q_out, T* __restrict__ k_pages, T* __restrict__ v_pages,
-                                  int H, int K, int hd) {
+                                  int H, int K, int hd, int kv_round) {
     const int t = blockIdx.x;
     const int p = pos[t];
     const int half = hd >> 1;
@@ -158,6 +158,11 @@ __global__ void rope_store_kernel(const float* __restrict__ qkv, int row_stride,
             const float ra = a * c - b * s, rb = a * s + b * c;
             a = ra; b = rb;
         }
+        if (head >= H && kv_round != DT_F32) {
+            // what goes into the cache takes a 16-bit type's values on its way (block.cpp:145-148)
+            if (kv_round == DT_F16) { a = (float)(f16)a; b = (float)(f16)b; }
+            else { a = (float)(bf16)a; b = (float)(bf16)b; }
+        }
         if (head < H) {
             T* q = q_out + ((int64_t)t * H + head) * hd;
             q[d0] = from_f32<T>(a); q[d1] = from_f32<T>(b);
@@ -174,8 +179,9 @@ __global__ void rope_store_kernel(const float* __restrict__ qkv, int row_stride,
 extern "C" int li_rope_store(const float* qkv, int row_stride, const float* inv_freq, int rotary_dim,
                              int half_pairing, const int* pos, const int* tok_slot, const int* page_table,
                              int max_pages, int64_t page_stride, void* q_out, void* k_pages, void* v_pages, int dt,
-                             int n_tokens, int H, int K, int hd, hipStream_t stream) {
+                             int n_tokens, int H, int K, int hd, int kv_round, hipStream_t stream) {
     if (n_tokens <= 0) return LI_OK;
+    if (kv_round < DT_F32 || kv_round > DT_BF16) return LI_BAD_ARG;
     if (hd <= 0 || (hd & 1) || H <= 0 || K < 0 || rotary_dim < 0 || rotary_dim > hd || (rotary_dim & 1) ||
         row_stride < (H + 2 * K) * hd)
         return LI_BAD_ARG;
@@ -184,7 +190,7 @@ extern "C" int li_rope_store(const float* qkv, int row_stride, const float* inv_
 #define LAUNCH(T)                                                                                        \
     rope_store_kernel<T><<<grid, block, 0, stream>>>(qkv, row_stride, inv_freq, rotary_dim, half_pairing, \
                                                      pos, tok_slot, page_table, max_pages, page_stride, (T*)q_out, \
-                                                     (T*)k_pages, (T*)v_pages, H, K, hd)
+                                                     (T*)k_pages, (T*)v_pages, H, K, hd, kv_round)
     if (dt == DT_F32) LAUNCH(float);
     else if (dt == DT_F16) LAUNCH(f16);
     else if (dt == DT_BF16) LAUNCH(bf16);

@@ -32,27 +32,31 @@ class Engine:
     one token each.  It runs only the tokens it is given, against what earlier steps left in
     the cache, and returns the logits at the wanted places."""
 
-    def __init__(self, config, model: DecoderModel, max_tokens: int, n_slots: int | None = None):
+    def __init__(self, config, model: DecoderModel, max_tokens: int, n_slots: int | None = None, kv_round=None):
         self.config, self.model = config, model
         self.dtype, self.device = model.dtype, model.device
         self.max_positions = model.spec.max_positions
         self.vocab_size = model.spec.vocab_size
-        self.cache = Cache(model.cache_specs(), max_tokens, self.max_positions, model.dtype, model.device, n_slots)
+        # kv_round="float16" with dtype float32 is the reference's own mix: float32 activations, keys and
+        # values rounded to float16 on their way into the cache (src/model/block.cpp:145-148)
+        self.cache = Cache(model.cache_specs(), max_tokens, self.max_positions, model.dtype, model.device, n_slots,
+                           as_dtype(kv_round) if kv_round else None)
         self._graphs = {}
         self._graph_bufs = None
 
     # -- construction ----------------------------------------------------------
     @classmethod
-    def from_folder(cls, folder: str, dtype="bfloat16", max_tokens: int = 8192, n_slots=None, device="cuda"):
+    def from_folder(cls, folder: str, dtype="bfloat16", max_tokens: int = 8192, n_slots=None, device="cuda",
+                    kv_round=None):
         _require_gpu()
         config = config_from_folder(folder)
         model = DecoderModel(config.model_spec(), as_dtype(dtype), device)
         load_into(model, folder, config)
-        return cls(config, model, max_tokens, n_slots)
+        return cls(config, model, max_tokens, n_slots, kv_round)
 
     @classmethod
     def from_random(cls, config, seed: int = 0, dtype="bfloat16", max_tokens: int = 8192, n_slots=None,
-                    device="cuda", stored_dtype=None):
+                    device="cuda", stored_dtype=None, kv_round=None):
         """Random weights made on the device (no folder): matrices as ``stored_dtype`` would store them."""
         _require_gpu()
         dt = as_dtype(dtype)
@@ -61,7 +65,7 @@ class Engine:
         params = model.params()
         model.bind(OnDemand(lambda name: place_tensor(random_tensors({name: params[name]}, seed, stored, device)[name],
                                                       params[name].kind, dt, device)))
-        return cls(config, model, max_tokens, n_slots)
+        return cls(config, model, max_tokens, n_slots, kv_round)
 
     # -- sequences -----------------------------------------------------------------
     def alloc_slot(self) -> int:

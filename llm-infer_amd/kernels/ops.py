@@ -356,9 +356,10 @@ def swiglu(gu: torch.Tensor, out_dtype, gelu: bool = False) -> torch.Tensor:
 
 
 def rope_store(qkv, inv_freq, rotary_dim, half_pairing, pos, tok_slot, page_table, page_stride, k_pages, v_pages,
-               n_heads, n_kv_heads, head_dim, out_dtype) -> torch.Tensor:
+               n_heads, n_kv_heads, head_dim, out_dtype, kv_round=None) -> torch.Tensor:
     """Rotate q and k by position, write k and v into the pages; returns q [T, H, hd].
-    With n_kv_heads == 0 only q is rotated (a layer that reads another layer's cache)."""
+    With n_kv_heads == 0 only q is rotated (a layer that reads another layer's cache).
+    ``kv_round`` (a 16-bit dtype): k and v take that type's values before they are stored."""
     _dev(qkv, inv_freq, pos, tok_slot, page_table, k_pages, v_pages)
     t = qkv.shape[0]
     _need(qkv.dtype == torch.float32 and qkv.dim() == 2, "qkv: float32 [T, (H+2K) hd]")
@@ -376,7 +377,8 @@ def rope_store(qkv, inv_freq, rotary_dim, half_pairing, pos, tok_slot, page_tabl
         _ptr(qkv), qkv.shape[1], _ptr(inv_freq), rotary_dim, int(half_pairing), _ptr(pos), _ptr(tok_slot),
         _ptr(page_table), page_table.shape[1] if page_table is not None else 0, c_int64(page_stride or 0),
         _ptr(q), _ptr(k_pages),
-        _ptr(v_pages), DT[out_dtype], t, n_heads, n_kv_heads, head_dim, _stream()), "rope_store")
+        _ptr(v_pages), DT[out_dtype], t, n_heads, n_kv_heads, head_dim, DT[kv_round or torch.float32], _stream()),
+        "rope_store")
     return q
 
 

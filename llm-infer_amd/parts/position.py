@@ -31,7 +31,8 @@ class RotaryPosition:
         if n_kv_heads > 0:
             k, v, table, stride = kv_view.k, kv_view.v, kv_view.page_table, kv_view.page_stride
         return ops.rope_store(qkv, self.inv_freq, self.rotary_dim, self.pairing == "half", ctx.pos, ctx.tok_slot,
-                              table, stride, k, v, n_heads, n_kv_heads, head_dim, self.dtype)
+                              table, stride, k, v, n_heads, n_kv_heads, head_dim, self.dtype,
+                              kv_round=getattr(kv_view, "round_to", None))
 
     def project_rotate_store(self, h, w, ctx, kv_view, n_heads, n_kv_heads, head_dim):
         """q, k, v = h W^T, rotated and stored; with adjacent pairing and 16-bit storage the rotation
@@ -76,7 +77,7 @@ class NoPosition:
         if n_kv_heads > 0:
             k, v, table, stride = kv_view.k, kv_view.v, kv_view.page_table, kv_view.page_stride
         return ops.rope_store(qkv, None, 0, False, ctx.pos, ctx.tok_slot, table, stride, k, v, n_heads, n_kv_heads,
-                              head_dim, self.dtype)
+                              head_dim, self.dtype, kv_round=getattr(kv_view, "round_to", None))
 
     def project_rotate_store(self, h, w, ctx, kv_view, n_heads, n_kv_heads, head_dim):
         return _project(self, h, w, ctx, kv_view, n_heads, n_kv_heads, head_dim, None, 0, True)

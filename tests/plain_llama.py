@@ -133,7 +133,7 @@ def swiglu(x: torch.Tensor, w_gate: torch.Tensor, w_up: torch.Tensor, w_down: to
     return linear(_r(fn(linear(x, w_gate)) * linear(x, w_up), act_dtype), w_down)
 
 
-def attention_part(x, w, prefix, s, positions, window=None, act_dtype=None):
+def attention_part(x, w, prefix, s, positions, window=None, act_dtype=None, kv_dtype=None):
     """Projections, rotation of q and k, attention, output projection (block.cpp:125-167)."""
     n = x.shape[0]
     q = linear(x, w[prefix + "q_proj.weight"]).view(n, s["n_heads"], s["hd"])
@@ -141,31 +141,33 @@ def attention_part(x, w, prefix, s, positions, window=None, act_dtype=None):
     v = linear(x, w[prefix + "v_proj.weight"]).view(n, s["n_kv"], s["hd"])
     q = _r(rope(q, positions, s["theta"], s["rotary"]), act_dtype)          # block.cpp:141
     k = _r(rope(k, positions, s["theta"], s["rotary"]), act_dtype)          # block.cpp:142
+    k, v = _r(k, kv_dtype), _r(v, kv_dtype)               # the cache holds float16 (block.cpp:145-148)
     a = attention(q, k, _r(v, act_dtype), window, act_dtype).reshape(n, s["n_heads"] * s["hd"])
     return linear(_r(a, act_dtype), w[prefix + "o_proj.weight"])            # block.cpp:167
 
 
-def block(x, w, i, s, positions, act_dtype=None):
+def block(x, w, i, s, positions, act_dtype=None, kv_dtype=None):
     """Pre-norm decoder layer: x += attn(norm(x)); x += ffn(norm(x)) (block.cpp:106-224)."""
     p = f"model.layers.{i}."
     h = _r(rmsnorm(x, w[p + "input_layernorm.weight"], s["eps"]), act_dtype)      # block.cpp:113-119
-    x = x + attention_part(h, w, p + "self_attn.", s, positions, None, act_dtype)  # block.cpp:170-172
+    x = x + attention_part(h, w, p + "self_attn.", s, positions, None, act_dtype, kv_dtype)  # block.cpp:170-172
     h = _r(rmsnorm(x, w[p + "post_attention_layernorm.weight"], s["eps"]), act_dtype)   # block.cpp:177-183
     x = x + swiglu(h, w[p + "mlp.gate_proj.weight"], w[p + "mlp.up_proj.weight"],
                    w[p + "mlp.down_proj.weight"], act_dtype, s.get("act", "silu"))  # block.cpp:220-222
     return x
 
 
-def forward(weights: dict, cfg: dict, tokens, dtype=torch.float32, act_dtype=None) -> torch.Tensor:
+def forward(weights: dict, cfg: dict, tokens, dtype=torch.float32, act_dtype=None, kv_dtype=None) -> torch.Tensor:
     """Logits [n, vocab] at every position of one whole sequence (model.cpp:60-99).
-    ``act_dtype`` rounds the activations that a 16-bit engine stores between its kernels."""
+    ``act_dtype`` rounds the activations that a 16-bit engine stores between its kernels; ``kv_dtype``
+    rounds keys (after the rotation) and values as the reference's float16 cache does."""
     s = sizes(cfg)
     w = {k: v.to(dtype) for k, v in weights.items()}
     tokens = torch.as_tensor(tokens, dtype=torch.long)
     positions = torch.arange(tokens.numel())
     x = embed(w["model.embed_tokens.weight"], tokens)
     for i in range(s["n_layers"]):
-        x = block(x, w, i, s, positions, act_dtype)
+        x = block(x, w, i, s, positions, act_dtype, kv_dtype)
     x = _r(rmsnorm(x, w["model.norm.weight"], s["eps"]), act_dtype)                # model.cpp:79-90
     head = w["model.embed_tokens.weight"] if s["tied"] or "lm_head.weight" not in w else w["lm_head.weight"]
     return linear(x, head)                                                          # model.cpp:93-98

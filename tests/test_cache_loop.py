@@ -218,6 +218,15 @@ def test_launch_plans_cover_every_product_once():
             assert (nb0, mb0) == (0, 0) and ((nb1 == nc0 and mb1 == 0 and mc0 == 0) or (mb1 == mc0 and nb1 == 0 and nc0 == 0))
 
 
+def test_cache_rounding_option_is_for_a_float32_cache():
+    with pytest.raises(CacheError, match="kv_round"):
+        Cache([KVSpec(1, 16)], 256, 128, torch.bfloat16, None, 2, kv_round=torch.float16)
+    with pytest.raises(CacheError, match="kv_round"):
+        Cache([KVSpec(1, 16)], 256, 128, torch.float32, None, 2, kv_round=torch.float32)
+    c = Cache([KVSpec(1, 16)], 256, 128, torch.float32, None, 2, kv_round=torch.float16)
+    assert c.groups[0].round_to == torch.float16
+
+
 def test_command_line_follows_the_reference():
     c = parse_args(["m", "-i", "hi", "-n", "5", "-t", "0.5", "--seed", "7", "-T", "99"])
     assert (c["model"], c["prompt"], c["max_tokens"], c["temperature"], c["seed"], c["context"]) == \
@@ -230,6 +239,8 @@ def test_command_line_follows_the_reference():
     c = parse_args(["-", "--tokens", "1", "--random-weights", "--config", "c.json", "--slots", "2", "--dtype", "float16"])
     assert (c["random"], c["config"], c["slots"], c["dtype"]) == (True, "c.json", 2, "float16")
     assert parse_args(["m", "--tokens", "1", "--slots", "two"]) is None
+    c = parse_args(["m", "--tokens", "1", "--dtype", "float32", "--kv-round", "float16"])
+    assert (c["dtype"], c["kv_round"]) == ("float32", "float16") and parse_args(["m", "--tokens", "1"])["kv_round"] is None
 
 
 def test_tokenizer_longest_match_and_bytes():

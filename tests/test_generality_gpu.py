@@ -181,6 +181,49 @@ def test_long_decoding_and_first_tokens(lib, folders, dtype):
     eng.free_slot(s)
 
 
+@pytest.mark.parametrize("name,cfg", [("A", TINY_A), ("B", TINY_B)])
+def test_float32_with_the_references_float16_cache(lib, folders, name, cfg):
+    """float32 activations with keys and values rounded to float16 on their way into the cache is the
+    reference's own mix (src/model/block.cpp:145-148).  Rounding is not continuous: two correct
+    implementations whose float32 sums differ in the last bit round a few elements to different
+    neighbours, each a whole float16 step apart, so the largest difference of the logits is that of
+    one unlucky element.  What is exact is checked exactly (the first layer's pages, whose inputs do
+    not depend on the cache, and the result however the tokens are cut); the logits are compared by
+    their root mean square, with the measure that the other tests use."""
+    folder = folders[name]
+    weights = P.load_weights(folder)
+    n = 90
+    toks = torch.randint(0, cfg["vocab_size"], (n,), generator=torch.Generator().manual_seed(4)).tolist()
+    ref = P.forward(weights, cfg, toks, torch.float64, kv_dtype=torch.float16)
+    own = P.forward(weights, cfg, toks, torch.float32, kv_dtype=torch.float16)
+    unrounded = P.forward(weights, cfg, toks, torch.float64)
+    rms = lambda a, b: (a.double() - b.double()).pow(2).mean().sqrt().item()
+    eng = lib.load(folder, dtype="float32", max_tokens=256, kv_round="float16")
+    s = eng.alloc_slot()
+    got = [eng.step([s], [toks[:n - 8]], [list(range(n - 8))])]
+    for t in toks[n - 8:]:
+        got.append(eng.step([s], [[t]]))
+    got = torch.cat(got).cpu()
+    assert rms(got, ref) < 3 * rms(own, ref) + 1e-7
+    # the rounding is there: an engine that did not round would fail the line above
+    assert rms(got, unrounded) > 0.5 * rms(ref, unrounded) and rms(got, unrounded) > 2 * (3 * rms(own, ref) + 1e-7)
+    whole = lib.load(folder, dtype="float32", max_tokens=256, kv_round="float16")
+    assert whole.alloc_slot() == s
+    assert torch.equal(whole.step([s], [toks], [list(range(n))]).cpu(), got)       # however it is cut
+    # the first layer's keys and values: exactly the float16 neighbours of what an engine without the
+    # option stores (round to nearest even, as f32_to_f16 of include/kernels_cpu.hpp:17)
+    plain_cache = lib.load(folder, dtype="float32", max_tokens=256)
+    assert plain_cache.alloc_slot() == s
+    plain_cache.step([s], [toks], [[n - 1]])
+    def first_layer(e):
+        g = e.cache.groups[0]
+        return g.storage.view(g.storage.shape[0], len(g.entries), g.layer_elems)[:, g.entries.index(0)]
+    a, b = first_layer(whole), first_layer(plain_cache)
+    assert torch.equal(a, b.half().float()) and not torch.equal(a, b) and int((b != 0).sum()) > n
+    with pytest.raises(Exception, match="kv_round"):
+        lib.load(folder, dtype="bfloat16", max_tokens=256, kv_round="float16")
+
+
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 def test_recorded_steps_replay_like_eager_steps(lib, folders, dtype):
     """Greedy generation of 150 tokens for a ragged batch whose sequences end at different times:

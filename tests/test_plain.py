@@ -174,6 +174,26 @@ def test_attention_part_shift_invariance():
     assert torch.allclose(a, b, atol=1e-10)
 
 
+def test_cache_rounding_touches_keys_after_rotation_and_values_only():
+    """block.cpp:141-148: q and k are rotated, then k and v go into the cache as float16; q does not."""
+    s = P.sizes(TINY_A)
+    w = {k: v.double() for k, v in P.random_weights(TINY_A, 3, std=0.3).items()}
+    x = torch.randn(6, s["d"], dtype=F64)
+    pre = "model.layers.0.self_attn."
+    pos = torch.arange(6) + 3
+    got = P.attention_part(x, w, pre, s, pos, kv_dtype=torch.float16)
+    q = P.rope(P.linear(x, w[pre + "q_proj.weight"]).view(6, s["n_heads"], s["hd"]), pos, s["theta"], s["rotary"])
+    k = P.rope(P.linear(x, w[pre + "k_proj.weight"]).view(6, s["n_kv"], s["hd"]), pos, s["theta"], s["rotary"])
+    v = P.linear(x, w[pre + "v_proj.weight"]).view(6, s["n_kv"], s["hd"])
+    a = P.attention(q, k.half().double(), v.half().double()).reshape(6, -1)
+    assert torch.equal(got, P.linear(a, w[pre + "o_proj.weight"]))
+    assert not torch.equal(got, P.attention_part(x, w, pre, s, pos))
+    # a single token: the output is its own value row, rounded
+    one = P.attention_part(x[:1], w, pre, s, pos[:1], kv_dtype=torch.float16)
+    v0 = v[:1].half().double().repeat_interleave(s["n_heads"] // s["n_kv"], dim=1).reshape(1, -1)
+    assert torch.allclose(one, P.linear(v0, w[pre + "o_proj.weight"]), atol=1e-12)
+
+
 def test_sizes_defaults():
     s = P.sizes({"hidden_size": 64, "num_attention_heads": 4, "num_hidden_layers": 1,
                  "intermediate_size": 8, "vocab_size": 10})
