@@ -44,9 +44,8 @@ def build_dir() -> str:
     d = os.environ.get("LLM_INFER_AMD_BUILD_DIR") or os.path.join(CSRC, "_build")
     try:
         os.makedirs(d, exist_ok=True)
-        probe = os.path.join(d, f".w{os.getpid()}")
-        with open(probe, "w"):
-            pass
+        fd, probe = tempfile.mkstemp(prefix=".w", dir=d)       # a name of its own: builds run side by side
+        os.close(fd)
         os.remove(probe)
         return d
     except OSError:

@@ -1,4 +1,5 @@
 """The cache's bookkeeping and the generation loop's decisions (no GPU)."""
+import os
 import random
 
 import pytest
@@ -225,6 +226,18 @@ def test_cache_rounding_option_is_for_a_float32_cache():
         Cache([KVSpec(1, 16)], 256, 128, torch.float32, None, 2, kv_round=torch.float32)
     c = Cache([KVSpec(1, 16)], 256, 128, torch.float32, None, 2, kv_round=torch.float16)
     assert c.groups[0].round_to == torch.float16
+
+
+def test_build_folder_is_the_same_for_builds_that_run_side_by_side(tmp_path, monkeypatch):
+    """Every library of one build lands in one folder: the probe for a writable folder must not
+    collide between threads (a collision once sent some libraries to the temporary folder)."""
+    from concurrent.futures import ThreadPoolExecutor
+    from llm_infer_amd.kernels import build
+    want = str(tmp_path / "libs")
+    monkeypatch.setenv("LLM_INFER_AMD_BUILD_DIR", want)
+    with ThreadPoolExecutor(max_workers=16) as pool:
+        got = set(pool.map(lambda _: build.build_dir(), range(800)))
+    assert got == {want} and os.listdir(want) == []
 
 
 def test_command_line_follows_the_reference():
