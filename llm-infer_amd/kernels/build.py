@@ -40,8 +40,14 @@ def _say(msg: str) -> None:
     print(f"[llm_infer_amd] {msg}", file=sys.stderr, flush=True)
 
 
+def _preferred_dir() -> str:
+    return os.environ.get("LLM_INFER_AMD_BUILD_DIR") or os.path.join(CSRC, "_build")
+
+
 def build_dir() -> str:
-    d = os.environ.get("LLM_INFER_AMD_BUILD_DIR") or os.path.join(CSRC, "_build")
+    """Where libraries are built: the preferred folder, or one under the temporary folder if that
+    cannot be written (a checkout that belongs to someone else)."""
+    d = _preferred_dir()
     try:
         os.makedirs(d, exist_ok=True)
         fd, probe = tempfile.mkstemp(prefix=".w", dir=d)       # a name of its own: builds run side by side
@@ -89,14 +95,19 @@ def _run(cmd, what):
 
 
 def _build_library(lib_name: str, sources, defines=(), force=False) -> str:
+    stamp = _stamp(sources, defines)
+    if not force:
+        # a library built from these very sources is taken where it lies, also from a folder that
+        # cannot be written
+        for d in dict.fromkeys((_preferred_dir(), build_dir())):
+            lib = os.path.join(d, lib_name)
+            if os.path.isfile(lib) and os.path.isfile(lib + ".stamp"):
+                with open(lib + ".stamp") as f:
+                    if f.read().strip() == stamp:
+                        return lib
     d = build_dir()
     lib = os.path.join(d, lib_name)
     stamp_file = lib + ".stamp"
-    stamp = _stamp(sources, defines)
-    if not force and os.path.isfile(lib) and os.path.isfile(stamp_file):
-        with open(stamp_file) as f:
-            if f.read().strip() == stamp:
-                return lib
     hipcc = _hipcc()
     _say(f"compiling {lib_name} for {ARCH} ...")
     t0 = time.time()

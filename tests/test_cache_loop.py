@@ -240,6 +240,23 @@ def test_build_folder_is_the_same_for_builds_that_run_side_by_side(tmp_path, mon
     assert got == {want} and os.listdir(want) == []
 
 
+def test_a_current_library_is_taken_from_a_folder_that_cannot_be_written(tmp_path, monkeypatch):
+    from llm_infer_amd.kernels import build
+    kept, other = tmp_path / "kept", tmp_path / "other"
+    kept.mkdir(); other.mkdir()
+    monkeypatch.setenv("LLM_INFER_AMD_BUILD_DIR", str(kept))
+    monkeypatch.setattr(build, "build_dir", lambda: str(other))            # as if `kept` were read-only
+    def no_compiler():
+        raise AssertionError("nothing has to be compiled")
+    monkeypatch.setattr(build, "_hipcc", no_compiler)
+    (kept / "libx.so").write_bytes(b"x")
+    (kept / "libx.so.stamp").write_text(build._stamp((build.ATTN_SOURCE,), ("-DHEAD_DIM=16",)))
+    assert build._build_library("libx.so", (build.ATTN_SOURCE,), ("-DHEAD_DIM=16",)) == str(kept / "libx.so")
+    (kept / "libx.so.stamp").write_text("built from other sources")
+    with pytest.raises(AssertionError, match="compiled"):
+        build._build_library("libx.so", (build.ATTN_SOURCE,), ("-DHEAD_DIM=16",))
+
+
 def test_command_line_follows_the_reference():
     c = parse_args(["m", "-i", "hi", "-n", "5", "-t", "0.5", "--seed", "7", "-T", "99"])
     assert (c["model"], c["prompt"], c["max_tokens"], c["temperature"], c["seed"], c["context"]) == \
