@@ -278,15 +278,26 @@ __global__ __launch_bounds__(256, HD <= 128 ? 2 : 1) void attn_prefill_kernel(
     fetch(p_lo);
     stash(smem);
     __syncthreads();
-    for (int p = p_lo; p <= p_hi; ++p) {
+    // Every wave walks all pages of the workgroup (p_lo..p_hi) and works on its own (wp_lo..wp_hi).
+    // Three loops, the middle one without a condition around the page's work: with one, the
+    // compiler kept the output accumulators in a second set of registers and copied all 64 back
+    // after every page.
+    auto pass = [&](int p, auto&& work) {
         T* cur = smem + ((p - p_lo) & 1) * (KE + VE);
         T* nxt = smem + ((p - p_lo + 1) & 1) * (KE + VE);
         if (p < p_hi) fetch(p + 1);
-        if (p >= wp_lo && p <= wp_hi)
-            a.page(cur, cur + KE, p * PAGE, lo, pos, scale2, p * PAGE < lo_max || p * PAGE + PAGE - 1 > hi_min);
+        work(cur);
         if (p < p_hi) stash(nxt);
         __syncthreads();
-    }
+    };
+    const int own_lo = max(p_lo, wp_lo), own_hi = min(p_hi, wp_hi);
+    int p = p_lo;
+    for (; p < own_lo && p <= p_hi; ++p) pass(p, [](T*) {});
+    for (; p <= own_hi; ++p)
+        pass(p, [&](T* cur) {
+            a.page(cur, cur + KE, p * PAGE, lo, pos, scale2, p * PAGE < lo_max || p * PAGE + PAGE - 1 > hi_min);
+        });
+    for (; p <= p_hi; ++p) pass(p, [](T*) {});
     const float inv = 1.f / a.total();
     if (!live) return;
     T* orow = out + (tok * H + h) * HD;
