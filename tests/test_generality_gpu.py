@@ -289,6 +289,27 @@ def test_reused_slots_and_batch_composition(lib, folders, dtype):
         eng.step(slots, [reqs[0] + reqs[0], reqs[0] + reqs[0], reqs[0] + reqs[0]])
 
 
+def test_many_sequences_in_one_batch(lib, folders):
+    """150 sequences of unequal lengths as one batch (more rows than the decode kernels' small-batch
+    paths take, page tables of many slots): in float32 every sequence's logits and greedy tokens are
+    bit-equal to those it has alone."""
+    import random
+    cfg, folder = TINY_C, folders["C"]
+    rng = random.Random(3)
+    prompts = [[rng.randrange(cfg["vocab_size"]) for _ in range(rng.choice([1, 2, 5, 17, 40, 63, 64, 65]))]
+               for _ in range(150)]
+    eng = lib.load(folder, dtype="float32", max_tokens=150 * 128)
+    out = eng.generate(prompts, max_new_tokens=12, temperature=0.0)
+    slots = [eng.alloc_slot() for _ in prompts]
+    together = eng.step(slots, prompts).cpu()
+    one = lib.load(folder, dtype="float32", max_tokens=1024)
+    for i in range(0, 150, 11):
+        assert one.generate([prompts[i]], max_new_tokens=12, temperature=0.0)[0] == out[i], i
+        s = one.alloc_slot()
+        assert torch.equal(one.step([s], [prompts[i]]).cpu()[0], together[i]), i
+        one.free_slot(s)
+
+
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 def test_prompt_in_several_chunks(lib, folders, dtype):
     """A prompt fed in chunks of several tokens (each chunk attends to the cache of the chunks before
