@@ -5,6 +5,8 @@
 // r comes from a counter-based generator with a key and a counter for every
 // sequence slot, so a sequence's tokens do not depend on what else is in the batch.
 #include "common.h"
+#include "no_alloc.h"
+#include <mutex>
 
 __host__ __device__ __forceinline__ uint64_t mix64(uint64_t z) {
     z = (z ^ (z >> 30)) * 0xBF58476D1CE4E5B9ULL;
@@ -220,6 +222,49 @@ extern "C" int li_argmax(const float* logits, int n_rows, int V, float* part_v, 
     argmax_final_kernel<<<n_rows, 64, 0, stream>>>(part_v, part_i, n_chunks, out);
     LI_CHECK_LAUNCH();
     return LI_OK;
+}
+
+// ---------------------------------------------------------------------------
+// li_argmax_static: li_argmax with its partial results in an array of the library (no_alloc.h).
+// In host code the array's name is only a stand-in for the symbol; its address on a device is
+// asked for once per device and that pointer is what the kernels get.
+// ---------------------------------------------------------------------------
+static __device__ __align__(256) unsigned char scratch[LI_ARGMAX_STATIC_BYTES];
+
+constexpr int MAX_DEVICES = 64;
+static void* scratch_ptr[MAX_DEVICES] = {};
+static std::mutex scratch_mutex;
+
+// the array's address on the current device, or null
+static void* scratch_of_current_device() {
+    int dev = -1;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= MAX_DEVICES) return nullptr;
+    std::lock_guard<std::mutex> guard(scratch_mutex);
+    if (!scratch_ptr[dev]) {
+        void* p = nullptr;
+        if (hipGetSymbolAddress(&p, HIP_SYMBOL(scratch)) != hipSuccess || !p) return nullptr;
+        scratch_ptr[dev] = p;
+    }
+    return scratch_ptr[dev];
+}
+
+extern "C" int li_argmax_static_init(void) { return scratch_of_current_device() ? LI_OK : LI_HIP_ERROR; }
+
+extern "C" int li_argmax_static_capacity(int V) {
+    return V <= 0 ? 0 : LI_ARGMAX_STATIC_ENTRIES / li_argmax_chunks(V);
+}
+
+extern "C" int li_argmax_static(const float* logits, int n_rows, int V, int* out, hipStream_t stream) {
+    if (n_rows <= 0) return LI_OK;
+    if (V <= 0 || !logits || !out) return LI_BAD_ARG;
+    const int n_chunks = li_argmax_chunks(V);
+    if ((int64_t)n_rows * n_chunks > LI_ARGMAX_STATIC_ENTRIES) return LI_UNSUPPORTED;
+    unsigned char* ptr = (unsigned char*)scratch_of_current_device();
+    if (!ptr) return LI_HIP_ERROR;
+    // maxima in the first half of the array, indices in the second
+    float* part_v = (float*)ptr;
+    int* part_i = (int*)(ptr + LI_ARGMAX_STATIC_ENTRIES * 4);
+    return li_argmax(logits, n_rows, V, part_v, part_i, out, stream);
 }
 
 // chunk of a row for li_sample (a multiple of 64, at most 64 chunks) and the floats of workspace a row needs

@@ -24,7 +24,7 @@ CSRC = os.path.join(os.path.dirname(os.path.dirname(os.path.abspath(__file__))),
 ARCH = "gfx950"
 CORE_SOURCES = ("elementwise.hip", "gemm.hip", "gemm_prefill.hip", "sampling.hip")
 ATTN_SOURCE = "attention.hip"
-HEADERS = ("common.h", "gemm_common.h")
+HEADERS = ("common.h", "gemm_common.h", "no_alloc.h")
 FLAGS = ["--offload-arch=" + ARCH, "-O3", "-std=c++17", "-fPIC",
          "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops", "-Wno-unused-command-line-argument"]
 
