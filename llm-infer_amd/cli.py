@@ -1,7 +1,7 @@
 """``infer``: the command line, in the manner of the reference's tool (tools/infer.cpp:112-349).
 
     infer <model_dir> [-i <prompt> | -f <file> | --tokens 1,2,3 | --tokens-file F]
-          [-n 256] [-t 1.0] [--seed 0] [-T <context>] [-d hip] [--dtype bfloat16]
+          [-n 256] [-t 1.0] [--seed 0] [-T <context>] [-d hip] [--dtype <name>]
 
 Options the reference has keep their names and meanings: -i, -f, -n (tokens to generate,
 256), -t (temperature, 1.0; <= 0 is greedy), --seed, -T (context length override), -d (device;
@@ -30,7 +30,7 @@ Options:
   -t <float>            Temperature for sampling (default: 1.0)
   -T <int>              Context length override (default: model max)
   --seed <int>          Random seed (default: 0)
-  --dtype <name>        bfloat16 (default), float16 or float32
+  --dtype <name>        bfloat16, float16 or float32 (default: the model's own)
   --kv-round <name>     With --dtype float32: keys and values rounded to float16 (the reference's cache) or bfloat16
   --slots <int>         Most sequences that run as one batch (default: all requests given)
   --random-weights      Ignore the model's tensors: random weights from --seed-weights
@@ -45,7 +45,7 @@ def parse_ids(text: str) -> list:
 
 def parse_args(argv):
     cfg = dict(model=None, device="hip", prompt=None, prompt_file=None, tokens=[], tokens_file=None,
-               max_tokens=256, temperature=1.0, seed=0, context=None, dtype="bfloat16", random=False,
+               max_tokens=256, temperature=1.0, seed=0, context=None, dtype=None, random=False,
                seed_weights=0, graph=True, help=False, slots=None, config=None, kv_round=None)
     if any(a in ("-h", "--help") for a in argv):
         cfg["help"] = True

@@ -3,7 +3,11 @@
 Keys and defaults are those of the reference's HF constructor
 (src/model/config.cpp:74-137): ``num_key_value_heads`` defaults to the number of
 heads (:81), ``head_dim`` to hidden/heads (:82), ``rope_theta`` to 10000 (:88),
-``partial_rotary_factor`` to 1 (:89-90), ``rms_norm_eps`` to 1e-5 (:93).  The
+``partial_rotary_factor`` to 1 (:89-90), ``rms_norm_eps`` to 1e-5 (:93).  One default
+departs from that constructor on purpose: a config.json without ``hidden_act`` gets
+"silu", the activation of the Llama decoder and what the reference's GGUF constructor,
+the only one wired to its model, fixes (config.cpp:163); the HF constructor would take
+"gelu" (config.cpp:97).  The
 reference's model reads no ``tie_word_embeddings``, ``eos_token_id`` or
 ``architectures``; those are read here because a generation library needs them.
 """
@@ -60,7 +64,7 @@ class LlamaConfig:
         rotary_dim = int(head_dim * float(c.get("partial_rotary_factor", 1.0)))
         eos = c.get("eos_token_id")
         eos_ids = () if eos is None else tuple(int(e) for e in (eos if isinstance(eos, list) else [eos]))
-        act = c.get("hidden_act", "silu")
+        act = c.get("hidden_act", "silu")          # not config.cpp:97's "gelu": see the module's docstring
         if c.get("rope_scaling") not in (None, {}):
             # the reference parses a rope scale and never uses it (include/llama.hpp:14)
             print("warning: rope_scaling is ignored, positions are rotated unscaled", file=sys.stderr)

@@ -1,11 +1,14 @@
 """The engine: a model, its cache, and the one step function."""
 from __future__ import annotations
 
+import sys
+
 import torch
 
 from ..cache import Cache, CacheError
 from ..registry import config_from_folder
-from ..weights import OnDemand, load_into, place_tensor, random_tensors
+from ..weights import (OnDemand, choose_dtype, load_into, place_tensor, random_tensors, read_checkpoint,
+                       stored_matrix_dtype)
 from .model import DecoderModel
 from .step import StepContext
 
@@ -19,6 +22,10 @@ def as_dtype(d):
     if d not in _DTYPES:
         raise ValueError(f"dtype {d!r}: one of bfloat16, float16, float32")
     return _DTYPES[d]
+
+
+def _say(msg: str) -> None:
+    print(f"[llm_infer_amd] {msg}", file=sys.stderr, flush=True)
 
 
 def _require_gpu():
@@ -46,20 +53,27 @@ class Engine:
 
     # -- construction ----------------------------------------------------------
     @classmethod
-    def from_folder(cls, folder: str, dtype="bfloat16", max_tokens: int = 8192, n_slots=None, device="cuda",
+    def from_folder(cls, folder: str, dtype=None, max_tokens: int = 8192, n_slots=None, device="cuda",
                     kv_round=None):
+        """``dtype`` None: the model's own (``torch_dtype`` of config.json, else the type its matrices are
+        stored in); a dtype that narrows what is stored, or swaps the 16-bit type, is said in one line."""
         _require_gpu()
         config = config_from_folder(folder)
-        model = DecoderModel(config.model_spec(), as_dtype(dtype), device)
-        load_into(model, folder, config)
+        spec = config.model_spec()
+        table = DecoderModel(spec, torch.float32, device, allocate=False).params()
+        ckpt = read_checkpoint(folder, table, config)
+        dt = choose_dtype(dtype, getattr(config, "torch_dtype", None), stored_matrix_dtype(table, ckpt), _say)
+        model = DecoderModel(spec, dt, device)
+        load_into(model, folder, config, ckpt)
         return cls(config, model, max_tokens, n_slots, kv_round)
 
     @classmethod
-    def from_random(cls, config, seed: int = 0, dtype="bfloat16", max_tokens: int = 8192, n_slots=None,
+    def from_random(cls, config, seed: int = 0, dtype=None, max_tokens: int = 8192, n_slots=None,
                     device="cuda", stored_dtype=None, kv_round=None):
-        """Random weights made on the device (no folder): matrices as ``stored_dtype`` would store them."""
+        """Random weights made on the device (no folder): matrices as ``stored_dtype`` would store them.
+        ``dtype`` None: the configuration's ``torch_dtype``, else bfloat16."""
         _require_gpu()
-        dt = as_dtype(dtype)
+        dt = choose_dtype(dtype, getattr(config, "torch_dtype", None), None)
         model = DecoderModel(config.model_spec(), dt, device)
         stored = as_dtype(stored_dtype) if stored_dtype else (dt if dt != torch.float32 else torch.bfloat16)
         params = model.params()

@@ -142,10 +142,65 @@ def place_tensor(t: torch.Tensor, kind: str, compute: torch.dtype, device) -> to
     return t.to(device=device, dtype=kept_dtype(t.dtype, kind, compute)).contiguous()
 
 
-def load_into(model, folder: str, config=None) -> None:
+_DTYPE_NAMES = {"float32": torch.float32, "float16": torch.float16, "bfloat16": torch.bfloat16}
+
+
+def stored_matrix_dtype(needed: dict, found) -> torch.dtype | None:
+    """The type in which a checkpoint stores its matrices: the widest among the matrices of the model's
+    table that the checkpoint holds (the reference reads it off blk.0.attn_q/k/v and ffn_up and rejects
+    a mix, src/model/config.cpp:36-70)."""
+    have = set(found.names())
+    seen = set()
+    for n, spec in needed.items():
+        if spec.kind == "matrix" and n in have:
+            try:
+                dtype = found.info(n)[0]
+            except ValueError:
+                continue                 # a tensor type that is not read: the check of the table says so
+            if dtype.is_floating_point:
+                seen.add(dtype)
+    if not seen:
+        return None
+    return next(iter(seen)) if len(seen) == 1 else torch.float32      # a mix: the type that holds them all
+
+
+def choose_dtype(requested, config_dtype: str | None, stored: torch.dtype | None, say=None) -> torch.dtype:
+    """The compute dtype of an engine.  ``requested`` None: what the model's own files say, ``torch_dtype``
+    of config.json first, else the type its matrices are stored in (a GGUF file has no other word on
+    it), else bfloat16; a float32 model so runs the 32-bit path (the reference takes the type from the
+    file in the same way and knows float32 and float16, src/model/config.cpp:119-129).  When the
+    result narrows what is stored, or turns one 16-bit type into the other, ``say`` gets one line."""
+    if requested is not None and not isinstance(requested, torch.dtype):
+        if requested not in _DTYPE_NAMES and requested not in ("bf16", "fp16", "fp32"):
+            raise ValueError(f"dtype {requested!r}: one of bfloat16, float16, float32")
+        requested = {**_DTYPE_NAMES, "bf16": torch.bfloat16, "fp16": torch.float16, "fp32": torch.float32}[requested]
+    if requested is not None:
+        chosen, by = requested, "as asked for"
+    elif config_dtype is not None:
+        if config_dtype not in _DTYPE_NAMES:
+            raise ValueError(f"Unsupported torch_dtype: {config_dtype}")
+        chosen, by = _DTYPE_NAMES[config_dtype], "by the configuration's torch_dtype"
+    elif stored is not None:
+        chosen, by = (torch.float32 if stored == torch.float64 else stored), "as stored"
+    else:
+        chosen, by = torch.bfloat16, "by default"
+    if say is not None and stored is not None and chosen != stored:
+        name = lambda d: str(d).replace("torch.", "")
+        if stored in (torch.float32, torch.float64) and chosen != torch.float32:
+            say(f"the matrices are stored in {name(stored)} and run in {name(chosen)} ({by}): they are rounded")
+        elif stored == torch.float16 and chosen == torch.bfloat16:
+            say(f"the matrices are stored in float16 and run in bfloat16 ({by}): three bits of every mantissa are lost")
+        elif stored == torch.bfloat16 and chosen == torch.float16:
+            say(f"the matrices are stored in bfloat16 and run in float16 ({by}): values beyond 65504 become infinite, "
+                "tiny ones lose bits")
+    return chosen
+
+
+def load_into(model, folder: str, config=None, ckpt=None) -> None:
     """Check the folder's tensors against ``model.params()`` and hand each part its tensors."""
     needed = model.params()
-    ckpt = read_checkpoint(folder, needed, config)
+    if ckpt is None:
+        ckpt = read_checkpoint(folder, needed, config)
     ignorable = list(model.ignorable_names())
     if isinstance(ckpt, GGUFCheckpoint):
         # exported beside the weights by other tools; the reference binds tensors by name and never

@@ -40,7 +40,9 @@ def sizes(cfg: dict) -> dict:
         rotary=rotary,
         eps=float(cfg.get("rms_norm_eps", 1e-5)),           # config.cpp:93
         tied=bool(cfg.get("tie_word_embeddings", False)),
-        act=cfg.get("hidden_act", "silu"),                  # config.cpp:97-105
+        # absent: silu, the Llama decoder's activation and what the reference's GGUF constructor fixes
+        # (config.cpp:163); its HF constructor would default to gelu (config.cpp:97), a departure on purpose
+        act=cfg.get("hidden_act", "silu"),
     )
 
 

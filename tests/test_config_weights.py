@@ -24,6 +24,11 @@ def test_defaults_follow_the_reference():
     assert c.rope_theta == 10000.0 and c.rotary_dim == 16             # config.cpp:88-90
     assert c.rms_norm_eps == 1e-5 and not c.tie_word_embeddings       # config.cpp:93
     assert c.eos_token_ids == () and c.rope_pairing == "adjacent"
+    # the one default that departs from the reference's HF constructor ("gelu", config.cpp:97): a Llama
+    # folder without hidden_act runs silu, as the reference's GGUF constructor fixes it (config.cpp:163)
+    assert c.hidden_act == "silu" and c.torch_dtype is None
+    raw = {"hidden_size": 8, "num_attention_heads": 2, "num_hidden_layers": 1, "intermediate_size": 8, "vocab_size": 4}
+    assert P.sizes(raw)["act"] == "silu" and P.sizes(dict(raw, hidden_act="gelu"))["act"] == "gelu"
 
 
 def test_every_size_comes_from_the_config():
@@ -177,6 +182,38 @@ def test_kept_dtypes():
     assert kept_dtype(f32, "matrix", bf) == f32                      # stored in 32-bit stays so
     assert kept_dtype(bf, "vector", bf) == f32 and kept_dtype(bf, "matrix", f32) == f32
     assert kept_dtype(torch.int64, "int", bf) == torch.int32
+
+
+def test_the_model_files_choose_the_compute_dtype(tmp_path):
+    from llm_infer_amd.weights import choose_dtype, stored_matrix_dtype
+    bf, f16, f32 = torch.bfloat16, torch.float16, torch.float32
+    said = []
+    # nothing asked for: torch_dtype of config.json, else what is stored, else bfloat16; no word about it
+    assert choose_dtype(None, "float16", f16, said.append) == f16
+    assert choose_dtype(None, None, f16, said.append) == f16 and choose_dtype(None, None, f32, said.append) == f32
+    assert choose_dtype(None, None, None, said.append) == bf and choose_dtype(None, "float32", None) == f32
+    assert choose_dtype("float32", "float16", f16, said.append) == f32          # widening loses nothing
+    assert said == []
+    # one line when the stored values are narrowed or change their 16-bit type
+    assert choose_dtype("bfloat16", "float16", f16, said.append) == bf and "three bits" in said[-1]
+    assert choose_dtype("float16", None, bf, said.append) == f16 and "65504" in said[-1]
+    assert choose_dtype("bf16", None, f32, said.append) == bf and "rounded" in said[-1]
+    assert choose_dtype(None, "bfloat16", f16, said.append) == bf and "torch_dtype" in said[-1]
+    assert len(said) == 4
+    with pytest.raises(ValueError, match="one of bfloat16, float16, float32"):
+        choose_dtype("int8", None, None)
+    # a float16 folder opened with no option keeps float16 matrices (and float32 norms)
+    cfg = llm_infer_amd.config_from_dict(TINY_A)
+    for name, dt in (("float16", f16), ("float32", f32), ("bfloat16", bf)):
+        folder = str(tmp_path / name)
+        write_random_model(folder, cfg, seed=1, dtype=name)
+        table = _model(TINY_A).params()
+        ckpt = read_checkpoint(folder)
+        stored = stored_matrix_dtype(table, ckpt)
+        assert stored == dt and llm_infer_amd.config_from_folder(folder).torch_dtype == name
+        compute = choose_dtype(None, llm_infer_amd.config_from_folder(folder).torch_dtype, stored, said.append)
+        assert compute == dt and kept_dtype(stored, "matrix", compute) == dt and kept_dtype(f32, "vector", compute) == f32
+    assert len(said) == 4
 
 
 def test_random_weights_mode_writes_a_model_folder(tmp_path):

@@ -17,60 +17,74 @@ pytestmark = pytest.mark.gpu
 LENGTHS = {"A": [40, 7, 100, 1, 64, 65, 33, 127], "B": [200, 1, 4, 9, 16, 31, 130, 255], "C": [300, 70, 5, 640, 129]}
 
 
-def make_weights(cfg, seed):
+def make_weights(cfg, seed, matrix_dtype=torch.bfloat16):
     """Random weights with sharper attention than N(0, 0.02) gives: q and k projections are
     scaled up so that scores differ by a unit or two and a wrong key or position shows, yet
-    bfloat16 rounding of the scores stays small."""
-    w = P.random_weights(cfg, seed, std=0.05)
+    16-bit rounding of the scores stays small."""
+    w = P.random_weights(cfg, seed, std=0.05, matrix_dtype=matrix_dtype)
     for name in w:
         if "q_proj" in name or "k_proj" in name:
             w[name] = (w[name].float() * 2).to(w[name].dtype)
     return w
 
 
+DTYPES = ["float32", "bfloat16", "float16"]
+STORED = {"float32": "bfloat16", "bfloat16": "bfloat16", "float16": "float16"}    # the folder a run opens
+TORCH = {"bfloat16": torch.bfloat16, "float16": torch.float16}
+
+
+class Model:
+    """A tiny configuration with its requests and, for each storage type of the matrices, a model folder,
+    the float64 logits of the plain implementation and that implementation's own error."""
+
+    def __init__(self, name, tmp_path_factory):
+        self.name, self.cfg = name, ALL[name]
+        g = torch.Generator().manual_seed(7)
+        self.requests = {f"r{i}": torch.randint(0, self.cfg["vocab_size"], (n,), generator=g).tolist()
+                         for i, n in enumerate(LENGTHS[name])}
+        self.folder, self.refs, self.own_error = {}, {}, {}
+        for stored, dt in TORCH.items():
+            folder = str(tmp_path_factory.mktemp(f"tiny_{name}_{stored}"))
+            weights = make_weights(self.cfg, seed=ord(name), matrix_dtype=dt)
+            P.write_model(folder, dict(self.cfg, torch_dtype=stored), weights)
+            refs = {rid: P.forward(weights, self.cfg, toks, torch.float64).numpy()
+                    for rid, toks in self.requests.items()}
+            self.folder[stored], self.refs[stored] = folder, refs
+            # what storing activations in this 16-bit type between the kernels costs
+            self.own_error[stored] = max(
+                np.abs(P.forward(weights, self.cfg, toks, torch.float64, dt).numpy() - refs[rid]).max()
+                for rid, toks in self.requests.items())
+            if stored == STORED["float32"]:
+                # what 32-bit arithmetic itself costs on this model: the plain implementation in float32
+                self.own_error["float32"] = max(
+                    np.abs(P.forward(weights, self.cfg, toks, torch.float32).numpy() - refs[rid]).max()
+                    for rid, toks in self.requests.items())
+
+
 @pytest.fixture(scope="module", params=list(ALL))
 def model(request, tmp_path_factory):
-    name = request.param
-    cfg = ALL[name]
-    folder = str(tmp_path_factory.mktemp(f"tiny_{name}"))
-    weights = make_weights(cfg, seed=ord(name))
-    P.write_model(folder, cfg, weights)
-    g = torch.Generator().manual_seed(7)
-    requests = {f"r{i}": torch.randint(0, cfg["vocab_size"], (n,), generator=g).tolist()
-                for i, n in enumerate(LENGTHS[name])}
-    refs = {rid: P.forward(weights, cfg, toks, torch.float64).numpy() for rid, toks in requests.items()}
-    # what 32-bit arithmetic itself costs on this model: the plain implementation in float32
-    FP32_ERROR[name] = max(np.abs(P.forward(weights, cfg, toks, torch.float32).numpy() - refs[rid]).max()
-                           for rid, toks in requests.items())
-    # and what storing activations in bfloat16 between the kernels costs
-    BF16_ERROR[name] = max(np.abs(P.forward(weights, cfg, toks, torch.float64, torch.bfloat16).numpy()
-                                  - refs[rid]).max() for rid, toks in requests.items())
-    return name, cfg, folder, requests, refs
+    return Model(request.param, tmp_path_factory)
 
 
-FP32_ERROR = {}
-BF16_ERROR = {}
-
-
-def check(got, refs, dtype, what):
+def check(got, model, dtype, what):
     """Within three times the error that the plain implementation itself has against float64 on
-    the same model and requests: in float32 arithmetic, or with its activations rounded to
-    bfloat16 at the places where a 16-bit engine stores them."""
+    the same model and requests: in float32 arithmetic, or with its activations rounded to the
+    16-bit type at the places where a 16-bit engine stores them."""
+    refs = model.refs[STORED[dtype]]
     scale = np.mean([r.std() for r in refs.values()])
-    own = FP32_ERROR if dtype == "float32" else BF16_ERROR
-    tol = 3 * own[what.split()[0]] + 1e-6 * scale
+    tol = 3 * model.own_error[dtype] + 1e-6 * scale
     worst, worst_key = 0.0, None
     for (rid, p), row in got.items():
         e = np.abs(row.astype(np.float64) - refs[rid][p]).max()
         if e > worst:
             worst, worst_key = e, (rid, p)
-    assert worst < tol, f"{what} {dtype}: first look at {worst_key}: error {worst:.3e}, allowed {tol:.3e}"
+    assert worst < tol, f"{model.name} {what} {dtype}: first look at {worst_key}: error {worst:.3e}, allowed {tol:.3e}"
     return worst
 
 
-@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("dtype", DTYPES)
 def test_replay_three_schedules(model, dtype, tmp_path):
-    name, cfg, folder, requests, refs = model
+    cfg, requests = model.cfg, model.requests
     vocab = cfg["vocab_size"]
     s1, w1 = TU.steps_whole(requests)
     s2, w2 = TU.steps_tail(requests, 32, first_step=1000)
@@ -78,7 +92,8 @@ def test_replay_three_schedules(model, dtype, tmp_path):
     s3, w3 = TU.steps_batches(requests, 3, decoded, first_step=5000)
     need = sum(-(-len(t) // 64) * 64 for t in list(requests.values())[:3])
     max_tokens = max(need, max(-(-len(t) // 64) * 64 for t in requests.values()) * 3)
-    got = TU.run_trace(folder, dtype, s1 + s2 + s3, {**w1, **w2, **w3}, vocab, max_tokens, str(tmp_path))
+    got = TU.run_trace(model.folder[STORED[dtype]], dtype, s1 + s2 + s3, {**w1, **w2, **w3}, vocab, max_tokens,
+                       str(tmp_path))
     assert got
     all_keys = set()
     for where, what in ((w1, "whole"), (w2, "tail"), (w3, "batches")):
@@ -88,24 +103,24 @@ def test_replay_three_schedules(model, dtype, tmp_path):
             for k, row in zip(keys, data):
                 sub[k] = row
         assert set(sub) == {(r, p) for r, t in requests.items() for p in range(len(t))}, what
-        check(sub, refs, dtype, f"{name} {what}")
+        check(sub, model, dtype, what)
         all_keys |= set(sub)
     assert len(all_keys) == sum(len(t) for t in requests.values())
 
 
-@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("dtype", DTYPES)
 def test_step_direct_and_generate(model, dtype):
     """Through the Python entry point: logits of a ragged batch, then greedy generation compared
     with the plain implementation token by token (where the plain logits leave no near tie)."""
     import llm_infer_amd
-    name, cfg, folder, requests, refs = model
+    cfg, requests, folder = model.cfg, model.requests, model.folder[STORED[dtype]]
     weights = P.load_weights(folder)
     eng = llm_infer_amd.load(folder, dtype=dtype, max_tokens=4096)
     ids = list(requests)[:4]
     slots = [eng.alloc_slot() for _ in ids]
     logits = eng.step(slots, [requests[r] for r in ids]).cpu().numpy()
     got = {(r, len(requests[r]) - 1): logits[i] for i, r in enumerate(ids)}
-    check(got, refs, dtype, f"{name} step")
+    check(got, model, dtype, "step")
     for s in slots:
         eng.free_slot(s)
     prompts = [requests[r][:20] for r in ids]
@@ -121,5 +136,20 @@ def test_step_direct_and_generate(model, dtype):
                 margin = (top2[0] - top2[1]).item()
                 if margin < (1e-4 if dtype == "float32" else 5e-2) * ref.std().item():
                     break                                     # a near tie: either token is right
-                assert t == int(ref.argmax()), (name, dtype, use_graph)
+                assert t == int(ref.argmax()), (model.name, dtype, use_graph)
                 toks.append(t)
+
+
+def test_a_model_runs_in_its_own_dtype_unless_told_otherwise(model, capfd):
+    """A folder opened with no dtype runs in the type its files say; a dtype that narrows or swaps the
+    stored 16-bit type is said in one line."""
+    import llm_infer_amd
+    for stored, dt in TORCH.items():
+        eng = llm_infer_amd.load(model.folder[stored], max_tokens=256)
+        assert eng.dtype == dt and eng.model.layers[0].mixer.wo.dtype == dt
+        assert eng.model.final_norm.weight.dtype == torch.float32
+        assert "stored" not in capfd.readouterr().err
+    eng = llm_infer_amd.load(model.folder["float16"], dtype="bfloat16", max_tokens=256)
+    assert eng.dtype == torch.bfloat16 and "three bits" in capfd.readouterr().err
+    eng = llm_infer_amd.load(model.folder["float16"], dtype="float32", max_tokens=256)
+    assert eng.dtype == torch.float32 and "stored" not in capfd.readouterr().err

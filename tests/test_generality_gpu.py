@@ -19,8 +19,8 @@ DEV = "cuda"
 ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 
 
-def sharp_weights(cfg, seed):
-    w = P.random_weights(cfg, seed, std=0.05)
+def sharp_weights(cfg, seed, matrix_dtype=torch.bfloat16):
+    w = P.random_weights(cfg, seed, std=0.05, matrix_dtype=matrix_dtype)
     for name in w:
         if "q_proj" in name or "k_proj" in name:
             w[name] = (w[name].float() * 2).to(w[name].dtype)
@@ -40,7 +40,19 @@ def folders(tmp_path_factory):
         d = str(tmp_path_factory.mktemp(f"gen_{name}"))
         P.write_model(d, cfg, sharp_weights(cfg, 11 + ord(name)))
         out[name] = d
+        d = str(tmp_path_factory.mktemp(f"gen_{name}_float16"))          # the same model stored in float16
+        P.write_model(d, dict(cfg, torch_dtype="float16"), sharp_weights(cfg, 11 + ord(name), torch.float16))
+        out[name, "float16"] = d
     return out
+
+
+DTYPES = ["float32", "bfloat16", "float16"]
+ACT = {"bfloat16": torch.bfloat16, "float16": torch.float16}
+
+
+def folder_for(folders, name, dtype):
+    """The folder a run in ``dtype`` opens: matrices stored in float16 for float16, in bfloat16 otherwise."""
+    return folders[name, "float16"] if dtype == "float16" else folders[name]
 
 
 def _ctx(lens_before, tokens):
@@ -154,15 +166,15 @@ def test_parts_alone(lib, dt):
 # ---------------------------------------------------------------------------
 # long decoding, the first tokens, graph replay
 # ---------------------------------------------------------------------------
-@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("dtype", DTYPES)
 def test_long_decoding_and_first_tokens(lib, folders, dtype):
-    cfg, folder = TINY_C, folders["C"]
+    cfg, folder = TINY_C, folder_for(folders, "C", dtype)
     weights = P.load_weights(folder)
     n = 700
     toks = torch.randint(0, cfg["vocab_size"], (n,), generator=torch.Generator().manual_seed(2)).tolist()
     ref = P.forward(weights, cfg, toks, torch.float64)
     own = (P.forward(weights, cfg, toks, torch.float32) if dtype == "float32"
-           else P.forward(weights, cfg, toks, torch.float64, torch.bfloat16))
+           else P.forward(weights, cfg, toks, torch.float64, ACT[dtype]))
     tol = 3 * (own.double() - ref).abs().max().item() + 1e-6
     eng = lib.load(folder, dtype=dtype, max_tokens=2048)
     s = eng.alloc_slot()
@@ -224,11 +236,11 @@ def test_float32_with_the_references_float16_cache(lib, folders, name, cfg):
         lib.load(folder, dtype="bfloat16", max_tokens=256, kv_round="float16")
 
 
-@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("dtype", DTYPES)
 def test_recorded_steps_replay_like_eager_steps(lib, folders, dtype):
     """Greedy generation of 150 tokens for a ragged batch whose sequences end at different times:
     the recorded (graph) runner and the eager runner must give the same tokens, replay after replay."""
-    eng = lib.load(folders["C"], dtype=dtype, max_tokens=8192)
+    eng = lib.load(folder_for(folders, "C", dtype), dtype=dtype, max_tokens=8192)
     g = torch.Generator().manual_seed(3)
     prompts = [torch.randint(0, 331, (n,), generator=g).tolist() for n in (5, 90, 33, 64)]
     plain_tokens = eng.generate(prompts, max_new_tokens=150, temperature=0.0, use_graph=False)
@@ -248,9 +260,9 @@ def test_recorded_steps_replay_like_eager_steps(lib, folders, dtype):
 # ---------------------------------------------------------------------------
 # slots and pages used again, batch composition
 # ---------------------------------------------------------------------------
-@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("dtype", DTYPES)
 def test_reused_slots_and_batch_composition(lib, folders, dtype):
-    cfg, folder = TINY_B, folders["B"]
+    cfg, folder = TINY_B, folder_for(folders, "B", dtype)
     eng = lib.load(folder, dtype=dtype, max_tokens=64 * 6, n_slots=3)
     g = torch.Generator().manual_seed(9)
     reqs = [torch.randint(0, cfg["vocab_size"], (n,), generator=g).tolist() for n in (100, 17, 64, 65, 1, 30)]
@@ -310,11 +322,11 @@ def test_many_sequences_in_one_batch(lib, folders):
         one.free_slot(s)
 
 
-@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("dtype", DTYPES)
 def test_prompt_in_several_chunks(lib, folders, dtype):
     """A prompt fed in chunks of several tokens (each chunk attends to the cache of the chunks before
     it and causally to itself), next to a sequence that is decoding: same logits as the whole prompt."""
-    cfg, folder = TINY_A, folders["A"]
+    cfg, folder = TINY_A, folder_for(folders, "A", dtype)
     weights = P.load_weights(folder)
     eng = lib.load(folder, dtype=dtype, max_tokens=1024)
     g = torch.Generator().manual_seed(4)
@@ -322,7 +334,7 @@ def test_prompt_in_several_chunks(lib, folders, dtype):
     b = torch.randint(0, 256, (90,), generator=g).tolist()
     ref_a, ref_b = (P.forward(weights, cfg, t, torch.float64) for t in (a, b))
     own = (P.forward(weights, cfg, a, torch.float32) if dtype == "float32"
-           else P.forward(weights, cfg, a, torch.float64, torch.bfloat16))
+           else P.forward(weights, cfg, a, torch.float64, ACT[dtype]))
     tol = 3 * (own.double() - ref_a).abs().max().item() + 1e-6
     sa, sb = eng.alloc_slot(), eng.alloc_slot()
     eng.step([sb], [b[:60]])
