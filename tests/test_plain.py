@@ -165,6 +165,87 @@ def test_block_is_identity_without_output_matrices(name):
     assert torch.equal(P.block(x, w, 0, s, torch.arange(5)), x)
 
 
+def _block_weights(cfg, seed):
+    return {k: v.double() for k, v in P.random_weights(cfg, seed, std=0.3).items()}
+
+
+@pytest.mark.parametrize("name", list(ALL))
+def test_block_arrangement_norm_before_each_part_and_sequential_residuals(name):
+    """block.cpp:113-119, 170-183, 220-222: a norm feeds the mixer, its result is added, a second norm
+    reads the sum, the feed-forward's result is added.  Each line fails for one plausible mistake: a
+    missing norm, a norm after the part, a feed-forward that reads x instead of x + attention."""
+    cfg = ALL[name]
+    s = P.sizes(cfg)
+    w = _block_weights(cfg, 4)
+    p = "model.layers.0."
+    pos = torch.arange(6)
+    x = torch.randn(6, s["d"], dtype=F64)
+    n1 = P.rmsnorm(x, w[p + "input_layernorm.weight"], s["eps"])
+    a = P.attention_part(n1, w, p + "self_attn.", s, pos)
+    # without the feed-forward's output matrix exactly x + attention(norm1(x)) is left
+    w0 = dict(w)
+    w0[p + "mlp.down_proj.weight"] = torch.zeros_like(w[p + "mlp.down_proj.weight"])
+    assert torch.allclose(P.block(x, w0, 0, s, pos), x + a, atol=1e-12)
+    assert not torch.allclose(P.block(x, w0, 0, s, pos), x + P.attention_part(x, w, p + "self_attn.", s, pos), atol=1e-3)
+    # the feed-forward reads norm2(x + attention), not norm2(x) (a parallel residual) and not x + attention
+    y = P.block(x, w, 0, s, pos)
+    gate, up, down = (w[p + f"mlp.{m}_proj.weight"] for m in ("gate", "up", "down"))
+    n2 = P.rmsnorm(x + a, w[p + "post_attention_layernorm.weight"], s["eps"])
+    assert torch.allclose(y - x - a, P.swiglu(n2, gate, up, down, act=s["act"]), atol=1e-10)
+    parallel = P.swiglu(P.rmsnorm(x, w[p + "post_attention_layernorm.weight"], s["eps"]), gate, up, down, act=s["act"])
+    assert not torch.allclose(y - x - a, parallel, atol=1e-3)
+    assert not torch.allclose(y - x - a, P.swiglu(x + a, gate, up, down, act=s["act"]), atol=1e-3)
+    # what a layer adds does not depend on the scale of a large input: both parts see it only through a
+    # norm (and norm2(c x + a) = norm2(x + a / c) -> norm2(x) as x grows).  Without either norm it does.
+    big = 1e6 * x
+    u1 = P.block(big, w, 0, s, pos) - big
+    u3 = P.block(3 * big, w, 0, s, pos) - 3 * big
+    assert (u1 - u3).abs().max() < 1e-3 * u1.abs().max()
+    # and the norms' weights are the layer's own two vectors, each in its place
+    w2 = dict(w)
+    w2[p + "input_layernorm.weight"] = 2 * w[p + "input_layernorm.weight"]
+    a2 = P.attention_part(2 * n1, w, p + "self_attn.", s, pos)
+    assert torch.allclose(P.block(x, {**w2, p + "mlp.down_proj.weight": w0[p + "mlp.down_proj.weight"]}, 0, s, pos),
+                          x + a2, atol=1e-12)
+
+
+@pytest.mark.parametrize("name", list(ALL))
+def test_final_norm_and_unscaled_embedding(name):
+    """model.cpp:79-98, 101-118: the last layer's output goes through the final norm before the head, and a
+    token's row of the table enters unscaled."""
+    cfg = dict(ALL[name], num_hidden_layers=1)
+    s = P.sizes(cfg)
+    w = _block_weights(cfg, 6)
+    toks = [3, 1, 4, 1, 5]
+    full = P.forward(w, cfg, toks, F64)
+    # the logits scale with the final norm's weight and vanish with it
+    w2 = dict(w)
+    w2["model.norm.weight"] = 2 * w["model.norm.weight"]
+    assert torch.allclose(P.forward(w2, cfg, toks, F64), 2 * full, atol=1e-9)
+    w2["model.norm.weight"] = torch.zeros_like(w["model.norm.weight"])
+    assert P.forward(w2, cfg, toks, F64).abs().max() == 0
+    # a weight that picks one channel: the logits see that channel of the normalised state alone
+    e0 = torch.zeros_like(w["model.norm.weight"])
+    e0[2] = 1.0
+    w2["model.norm.weight"] = e0
+    head = w["model.embed_tokens.weight"] if s["tied"] else w["lm_head.weight"]
+    one = P.forward(w2, cfg, toks, F64)
+    assert torch.allclose(one / head[:, 2][None, :], (one / head[:, 2][None, :])[:, :1].expand_as(one), atol=1e-9)
+    # with a layer that adds nothing the logits are norm(E[token]) W^T, the norm taken from the library:
+    # no factor on the embedding (sqrt(d) or any other would change what eps does to a small row)
+    wz = dict(w)
+    wz["model.layers.0.self_attn.o_proj.weight"] = torch.zeros_like(w["model.layers.0.self_attn.o_proj.weight"])
+    wz["model.layers.0.mlp.down_proj.weight"] = torch.zeros_like(w["model.layers.0.mlp.down_proj.weight"])
+    wz["model.embed_tokens.weight"] = w["model.embed_tokens.weight"] * 1e-2      # rows near sqrt(eps): a scale would show
+    rows = wz["model.embed_tokens.weight"][torch.tensor(toks)]
+    normed = torch.nn.functional.rms_norm(rows, (s["d"],), w["model.norm.weight"], s["eps"])
+    headz = wz["model.embed_tokens.weight"] if s["tied"] else wz["lm_head.weight"]
+    got = P.forward(wz, cfg, toks, F64)
+    assert torch.allclose(got, normed @ headz.t(), atol=1e-12)
+    scaled = torch.nn.functional.rms_norm(rows * s["d"] ** 0.5, (s["d"],), w["model.norm.weight"], s["eps"])
+    assert not torch.allclose(got, scaled @ headz.t(), rtol=1e-3, atol=0)
+
+
 def test_attention_part_shift_invariance():
     s = P.sizes(TINY_A)
     w = {k: v.double() for k, v in P.random_weights(TINY_A, 1, std=0.3).items()}
