@@ -64,6 +64,7 @@ class KVGroup:
         self.table_host = np.zeros((n_slots, self.max_pages), dtype=np.int32)
         self.pages_of = [dict() for _ in range(n_slots)]            # slot -> {page index in sequence: page}
         self.device, self.dtype = device, dtype
+        self._views = {}
         if device is not None:
             self.storage = torch.zeros((n_pages, self.page_elems), dtype=dtype, device=device)
             self.page_table = torch.zeros((n_slots, self.max_pages), dtype=torch.int32, device=device)
@@ -74,11 +75,14 @@ class KVGroup:
         return self.page_elems // PAGE * torch.empty((), dtype=self.dtype).element_size()
 
     def view(self, entry: int) -> KVView:
-        i = self.entries.index(entry)
-        flat = self.storage.view(-1)
-        k = flat[i * self.layer_elems:]
-        v = flat[i * self.layer_elems + self.k_elems:]
-        return KVView(k, v, self.page_elems, self.page_table, self.spec, self.round_to)
+        view = self._views.get(entry)
+        if view is None:                # the storage never moves: a view is made once
+            i = self.entries.index(entry)
+            flat = self.storage.view(-1)
+            k = flat[i * self.layer_elems:]
+            v = flat[i * self.layer_elems + self.k_elems:]
+            view = self._views[entry] = KVView(k, v, self.page_elems, self.page_table, self.spec, self.round_to)
+        return view
 
     def first_needed_page(self, length: int) -> int:
         """First page that a token at position ``length`` (the next one) still reads."""
@@ -152,7 +156,8 @@ class StateGroup:
 
 
 class Cache:
-    """``specs[i]`` is what schedule entry i asks for (None: it keeps no cache of its own).
+    """``specs[i]`` is what unit i asks for (a unit: one mixer of one run of a layer; None: it keeps no
+    cache of its own).
     ``max_tokens`` bounds the tokens all live sequences hold together, each sequence's count
     rounded up to a whole page."""
 

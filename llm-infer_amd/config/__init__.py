@@ -1,4 +1,4 @@
-from .spec import PartSpec, LayerSpec, ScheduleEntry, ModelSpec, ConfigError
+from .spec import PartSpec, SubLayerSpec, LayerSpec, ScheduleEntry, ModelSpec, ConfigError
 from .llama import LlamaConfig
 
-__all__ = ["PartSpec", "LayerSpec", "ScheduleEntry", "ModelSpec", "ConfigError", "LlamaConfig"]
+__all__ = ["PartSpec", "SubLayerSpec", "LayerSpec", "ScheduleEntry", "ModelSpec", "ConfigError", "LlamaConfig"]

@@ -18,7 +18,7 @@ import os
 import sys
 from dataclasses import dataclass
 
-from .spec import ConfigError, LayerSpec, ModelSpec, PartSpec, ScheduleEntry
+from .spec import ConfigError, LayerSpec, ModelSpec, PartSpec, ScheduleEntry, SubLayerSpec
 
 _REQUIRED = ("num_hidden_layers", "hidden_size", "intermediate_size", "num_attention_heads",
              "vocab_size", "max_position_embeddings")          # config.cpp:77-85 (.at() throws)
@@ -223,10 +223,10 @@ class LlamaConfig:
             p = f"model.layers.{i}."
             layers.append(LayerSpec(
                 block="pre_norm",
-                mixer=mixer.with_prefix(p + "self_attn."),
-                feed_forward=ffn.with_prefix(p + "mlp."),
-                mixer_norm=norm.with_prefix(p + "input_layernorm."),
-                feed_forward_norm=norm.with_prefix(p + "post_attention_layernorm."),
+                sublayers=(SubLayerSpec("mixer", mixer.with_prefix(p + "self_attn."),
+                                        norm=norm.with_prefix(p + "input_layernorm.")),
+                           SubLayerSpec("feed_forward", ffn.with_prefix(p + "mlp."),
+                                        norm=norm.with_prefix(p + "post_attention_layernorm."))),
                 position=position))
         spec = ModelSpec(
             hidden_size=self.hidden_size, vocab_size=self.vocab_size,

@@ -28,14 +28,31 @@ class PartSpec:
 
 
 @dataclass(frozen=True)
+class SubLayerSpec:
+    """One sub-layer: a part that reads the residual stream and adds to it, with the norm on its input
+    and, if the arrangement has one, a norm on its output.  ``role`` says what the part is to the
+    engine: a "mixer" looks at other tokens and may keep a cache, a "feed_forward" does not."""
+    role: str
+    part: PartSpec
+    norm: PartSpec | None = None
+    post_norm: PartSpec | None = None
+
+
+@dataclass(frozen=True)
 class LayerSpec:
-    """One layer: how its parts are arranged (``block``) and the parts themselves."""
+    """One layer: its sub-layers in the order in which they run (any number of mixers and
+    feed-forwards, each with its norms), how they are arranged (``block``), and the position encoding
+    that its mixers are handed."""
     block: str
-    mixer: PartSpec
-    feed_forward: PartSpec
-    mixer_norm: PartSpec
-    feed_forward_norm: PartSpec
+    sublayers: tuple
     position: PartSpec | None = None
+
+    @classmethod
+    def mixer_then_feed_forward(cls, block: str, mixer: PartSpec, feed_forward: PartSpec, mixer_norm: PartSpec,
+                                feed_forward_norm: PartSpec, position: PartSpec | None = None) -> "LayerSpec":
+        """The common layer of two sub-layers, each with a norm on its input."""
+        return cls(block, (SubLayerSpec("mixer", mixer, mixer_norm),
+                           SubLayerSpec("feed_forward", feed_forward, feed_forward_norm)), position)
 
 
 @dataclass(frozen=True)
@@ -61,6 +78,12 @@ class ModelSpec:
     def validate(self) -> None:
         if not self.layers:
             raise ConfigError("a model needs at least one layer")
+        for i, layer in enumerate(self.layers):
+            if not layer.sublayers:
+                raise ConfigError(f"layer {i} has no sub-layer")
+            for sub in layer.sublayers:
+                if sub.role not in ("mixer", "feed_forward"):
+                    raise ConfigError(f"layer {i}: a sub-layer is a 'mixer' or a 'feed_forward', not {sub.role!r}")
         for i, e in enumerate(self.schedule):
             if not 0 <= e.layer < len(self.layers):
                 raise ConfigError(f"schedule entry {i} names layer {e.layer}, there are {len(self.layers)}")

@@ -96,8 +96,13 @@ __device__ __forceinline__ float wave_inclusive_scan(float v, int lane) {
 }
 
 // workspace per row and chunk: [0] maximum, [1] sum, [2 .. 2 + steps) step sums; steps = chunk / 64
+// (temperature_dev, if not null, holds the temperature on the device and wins: a recorded step then
+// serves every temperature)
 __global__ __launch_bounds__(256) void sample_chunks_kernel(const float* __restrict__ logits, int V, int chunk,
-                                                            float temperature, float* __restrict__ ws) {
+                                                            float temperature,
+                                                            const float* __restrict__ temperature_dev,
+                                                            float* __restrict__ ws) {
+    if (temperature_dev) temperature = *temperature_dev;
     __shared__ float scratch[16];
     __shared__ float wave_tot[4];
     const float* row = logits + (int64_t)blockIdx.x * V;
@@ -127,11 +132,13 @@ __global__ __launch_bounds__(256) void sample_chunks_kernel(const float* __restr
 
 __global__ __launch_bounds__(64) void sample_final_kernel(const float* __restrict__ logits, int V, int chunk,
                                                           int n_chunks, float temperature,
+                                                          const float* __restrict__ temperature_dev,
                                                           const float* __restrict__ ws,
                                                           const int* __restrict__ seq_slot,
                                                           unsigned long long* __restrict__ state,
                                                           const float* __restrict__ forced_r,
                                                           int* __restrict__ out) {
+    if (temperature_dev) temperature = *temperature_dev;
     const int lane = threadIdx.x;
     const float* row = logits + (int64_t)blockIdx.x * V;
     const int steps = chunk >> 6;
@@ -277,16 +284,18 @@ extern "C" int li_sample_ws_floats(int V) {
     return ((V + chunk - 1) / chunk) * (2 + chunk / 64);
 }
 
-extern "C" int li_sample(const float* logits, int n_rows, int V, float temperature, const int* seq_slot,
-                         void* state, const float* forced_r, float* ws, int* out, hipStream_t stream) {
+// temperature_dev (may be null): one float on the device that replaces `temperature`; it must be positive
+extern "C" int li_sample(const float* logits, int n_rows, int V, float temperature, const float* temperature_dev,
+                         const int* seq_slot, void* state, const float* forced_r, float* ws, int* out,
+                         hipStream_t stream) {
     if (n_rows <= 0) return LI_OK;
-    if (V <= 0 || temperature <= 0.f || !ws) return LI_BAD_ARG;      // greedy goes through li_argmax
+    if (V <= 0 || (!temperature_dev && temperature <= 0.f) || !ws) return LI_BAD_ARG;      // greedy goes through li_argmax
     if (!forced_r && (!seq_slot || !state)) return LI_BAD_ARG;
     const int chunk = li_sample_chunk(V), n_chunks = (V + chunk - 1) / chunk;
-    sample_chunks_kernel<<<dim3(n_rows, n_chunks), 256, 0, stream>>>(logits, V, chunk, temperature, ws);
+    sample_chunks_kernel<<<dim3(n_rows, n_chunks), 256, 0, stream>>>(logits, V, chunk, temperature, temperature_dev, ws);
     LI_CHECK_LAUNCH();
-    sample_final_kernel<<<n_rows, 64, 0, stream>>>(logits, V, chunk, n_chunks, temperature, ws, seq_slot,
-                                                   (unsigned long long*)state, forced_r, out);
+    sample_final_kernel<<<n_rows, 64, 0, stream>>>(logits, V, chunk, n_chunks, temperature, temperature_dev, ws,
+                                                   seq_slot, (unsigned long long*)state, forced_r, out);
     LI_CHECK_LAUNCH();
     return LI_OK;
 }
@@ -297,7 +306,7 @@ extern "C" int li_token_prob(const float* logits, int n_rows, int V, const int* 
     if (n_rows <= 0) return LI_OK;
     if (V <= 0 || !logits || !tokens || !ws || !out) return LI_BAD_ARG;
     const int chunk = li_sample_chunk(V), n_chunks = (V + chunk - 1) / chunk;
-    sample_chunks_kernel<<<dim3(n_rows, n_chunks), 256, 0, stream>>>(logits, V, chunk, 1.0f, ws);
+    sample_chunks_kernel<<<dim3(n_rows, n_chunks), 256, 0, stream>>>(logits, V, chunk, 1.0f, nullptr, ws);
     LI_CHECK_LAUNCH();
     token_prob_kernel<<<n_rows, 64, 0, stream>>>(logits, V, chunk, n_chunks, ws, tokens, out);
     LI_CHECK_LAUNCH();

@@ -12,7 +12,7 @@ from __future__ import annotations
 import torch
 
 from ..kernels import ops
-from .step import decode_splits
+from .step import StepShared, decode_splits, split_bucket
 
 
 class PlainDecodeRunner:
@@ -28,29 +28,33 @@ class PlainDecodeRunner:
         pass
 
 
-class _GraphContext:
-    """The step description of a recorded decode step: fixed device buffers."""
+class _GraphContext(StepShared):
+    """The step description of a recorded decode step: fixed device buffers.  The lengths of the
+    sequences are known to it only as a bucket (``split_bucket``), which is what the split count of a
+    decode attention depends on."""
     is_decode = True
 
-    def __init__(self, bufs, n, splits):
+    def __init__(self, bufs, n, bucket):
         self.n_seqs = self.n_tokens = self.n_want = n
         self.token_ids, self.pos, self.seq_ctx = bufs["tokens"][:n], bufs["pos"][:n], bufs["ctx"][:n]
         self.tok_slot = self.seq_slot = bufs["slots"][:n]
         self.want_rows = bufs["rows"][:n]
-        self._splits = splits
+        self.device = self.token_ids.device
+        self._bucket = bucket
 
     def decode_splits(self, n_kv_heads, n_heads):
-        return self._splits
+        return decode_splits(self.n_seqs, n_kv_heads, n_heads, self._bucket)
 
-    def prefill_meta(self):
-        raise RuntimeError("a recorded decode step has no prompt")
+
+MAX_RECORDED_STEPS = 48        # recorded steps an engine keeps; the least recently used goes first
 
 
 class GraphDecodeRunner:
     """Replays a recorded step while the set of live sequences stays the same; when it
     changes, the slots and tokens are uploaded anew and the graph of the new size is used.
-    A step is run eagerly the first time its (batch size, split) is seen and recorded the
-    second time."""
+    A step is run eagerly the first time its (batch size, bucket of context lengths, sampling mode)
+    is seen and recorded the second time; the temperature is read from the device, so it is no part
+    of the key.  An engine keeps at most MAX_RECORDED_STEPS recorded steps."""
 
     def __init__(self, engine, sampler):
         self.engine, self.sampler = engine, sampler
@@ -62,6 +66,7 @@ class GraphDecodeRunner:
             self.bufs = {k: torch.zeros((n,), dtype=torch.int32, device=dev)
                          for k in ("tokens", "slots", "pos", "ctx", "next")}
             self.bufs["rows"] = torch.arange(n, dtype=torch.int32, device=dev)
+            self.bufs["temperature"] = torch.ones((1,), dtype=torch.float32, device=dev)
             # where the tokens of the steps in flight arrive on the host
             self.bufs["host"] = [torch.zeros((n,), dtype=torch.int32, pin_memory=True) for _ in range(3)]
             self.bufs["done"] = [torch.cuda.Event() for _ in range(3)]
@@ -72,24 +77,12 @@ class GraphDecodeRunner:
         self._host, self._done = self.bufs["host"], self.bufs["done"]
         self._turn = 0
 
-    def _splits(self, n, max_ctx):
-        spec = None
-        for s in self.engine.model.cache_specs():
-            if s is not None and hasattr(s, "n_kv_heads"):
-                spec = s
-                break
-        if spec is None:
-            return 1
-        mixer = self.engine.model.layers[0].mixer
-        n_heads = getattr(mixer, "n_heads", spec.n_kv_heads)
-        return decode_splits(n, spec.n_kv_heads, n_heads, max_ctx)
-
-    def _body(self, n, splits):
+    def _body(self, n, bucket):
         eng, b = self.engine, self.bufs
         ops.decode_prepare(b["slots"], eng.cache.lens_dev, b["pos"], b["ctx"], n)
-        ctx = _GraphContext(b, n, splits)
+        ctx = _GraphContext(b, n, bucket)
         logits = eng.model.forward(ctx, eng.cache)
-        self.sampler.sample(logits, b["slots"][:n], eng.cache, out=b["next"])
+        self.sampler.sample(logits, b["slots"][:n], eng.cache, out=b["next"], temperature_dev=b["temperature"])
         b["tokens"][:n].copy_(b["next"][:n])
 
     def _launch(self, slots, tokens):
@@ -105,20 +98,31 @@ class GraphDecodeRunner:
             b["slots"][:n].copy_(torch.tensor(slots, dtype=torch.int32))
             b["tokens"][:n].copy_(torch.tensor(tokens, dtype=torch.int32))
             self.current = list(slots)
-        splits = self._splits(n, max(new_lens))
-        key = (n, splits, self.sampler.temperature > 0.0, self.sampler.temperature)
-        entry = eng._graphs.get(key)
+        bucket = split_bucket(max(new_lens))
+        hot = self.sampler.temperature > 0.0
+        if hot and b.get("temperature_value") != self.sampler.temperature:
+            b["temperature"].fill_(self.sampler.temperature)
+            b["temperature_value"] = self.sampler.temperature
+        key = (n, bucket, hot)
+        graphs = eng._graphs
+        entry = graphs.pop(key, None)            # taken out and put back: the dict is in order of last use
         if entry is None:
-            self._body(n, splits)
-            eng._graphs[key] = "seen"
+            self._body(n, bucket)
+            entry = "seen"
         else:
             if entry == "seen":
                 g = torch.cuda.CUDAGraph()
                 torch.cuda.synchronize()
                 with torch.cuda.graph(g):
-                    self._body(n, splits)
-                eng._graphs[key] = entry = g
+                    self._body(n, bucket)
+                entry = g
             entry.replay()
+        graphs[key] = entry
+        while len(graphs) > MAX_RECORDED_STEPS:
+            old = next(iter(graphs))
+            if graphs[old] != "seen":
+                torch.cuda.synchronize()         # a recorded step may still be running: let it finish first
+            del graphs[old]
         self._turn = (self._turn + 1) % len(self._host)
         host, done = self._host[self._turn], self._done[self._turn]
         host[:n].copy_(b["next"][:n], non_blocking=True)

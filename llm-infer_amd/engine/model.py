@@ -8,6 +8,7 @@ import torch
 from .. import parts as _parts  # noqa: F401  (registers the built-in parts)
 from ..config.spec import ModelSpec
 from ..parts.base import Part, collect_params
+from ..parts.block import SubLayer
 from ..registry import lookup
 
 
@@ -22,24 +23,49 @@ class DecoderModel(Part):
         self.device = device if allocate else None
         dev = self.device
         self.embedding = _make("embedding", spec.embedding, dtype, dev)
+        self.positions = {}            # layers whose position specs are equal share one part
         self.layers = []
+        self.layer_mixers = []         # for each layer its mixers, in the order in which they run
         for ls in spec.layers:
-            position = None
-            if ls.position is not None:
-                position = lookup("position", ls.position.kind)(**ls.position.params, dtype=dtype, device=dev)
-            mixer = _make("mixer", ls.mixer, dtype, dev, position=position)
-            ffn = _make("feed_forward", ls.feed_forward, dtype, dev)
-            n1 = _make("norm", ls.mixer_norm, dtype, dev)
-            n2 = _make("norm", ls.feed_forward_norm, dtype, dev)
-            self.layers.append(lookup("block", ls.block)(n1, mixer, n2, ffn))
+            position = self._position(ls.position, dtype, dev)
+            subs, mixers = [], []
+            for sub in ls.sublayers:
+                if sub.role == "mixer":
+                    part = _make("mixer", sub.part, dtype, dev, position=position)
+                    mixers.append(part)
+                else:
+                    part = _make("feed_forward", sub.part, dtype, dev)
+                subs.append(SubLayer(sub.role, part,
+                                     None if sub.norm is None else _make("norm", sub.norm, dtype, dev),
+                                     None if sub.post_norm is None else _make("norm", sub.post_norm, dtype, dev)))
+            self.layers.append(lookup("block", ls.block)(subs))
+            self.layer_mixers.append(mixers)
         self.final_norm = _make("norm", spec.final_norm, dtype, dev)
         self.head = _make("head", spec.head, dtype, dev)
         self.schedule = list(spec.schedule)
+        # what the cache keeps is counted in units: one for each mixer of each run of a layer
+        self._unit, n = {}, 0
+        for i, e in enumerate(self.schedule):
+            if e.cache_from is not None and (len(self.layer_mixers[e.layer]) !=
+                                             len(self.layer_mixers[self.schedule[e.cache_from].layer])):
+                raise ValueError(f"schedule entry {i} reads the cache of entry {e.cache_from}, whose layer has "
+                                 "another number of mixers")
+            for k in range(len(self.layer_mixers[e.layer])):
+                self._unit[i, k] = n
+                n += 1
         self._table = collect_params(self)
+
+    def _position(self, spec, dtype, dev):
+        if spec is None:
+            return None
+        key = (spec.kind, spec.prefix, repr(sorted(spec.params.items())))
+        if key not in self.positions:
+            self.positions[key] = _make("position", spec, dtype, dev)
+        return self.positions[key]
 
     # -- weights -----------------------------------------------------------
     def children(self):
-        return [self.embedding, *self.layers, self.final_norm, self.head]
+        return [self.embedding, *self.positions.values(), *self.layers, self.final_norm, self.head]
 
     def recordable(self) -> bool:
         """True if every part's forward pass can be recorded into a graph."""
@@ -78,17 +104,19 @@ class DecoderModel(Part):
 
     # -- cache -------------------------------------------------------------
     def cache_specs(self) -> list:
-        """For each schedule entry what its mixer asks of the cache (None: reads another's)."""
-        return [None if e.cache_from is not None else self.layers[e.layer].mixer.cache_spec()
-                for e in self.schedule]
+        """For each unit (each mixer of each schedule entry, in order) what it asks of the cache
+        (None: it reads another's)."""
+        return [None if e.cache_from is not None else m.cache_spec()
+                for e in self.schedule for m in self.layer_mixers[e.layer]]
 
     # -- the forward pass of one step ---------------------------------------
     def forward(self, ctx, cache) -> torch.Tensor:
         """Runs the step's tokens through the schedule; returns float32 logits [n_want, vocab]."""
-        x = self.embedding.forward(ctx.token_ids)
+        x = self.embedding.forward(ctx)
         for i, e in enumerate(self.schedule):
             owner = i if e.cache_from is None else e.cache_from
-            self.layers[e.layer].forward(x, ctx, cache.view(owner), e.cache_from is None)
+            views = [cache.view(self._unit[owner, k]) for k in range(len(self.layer_mixers[e.layer]))]
+            self.layers[e.layer].forward(x, ctx, views, e.cache_from is None)
         if ctx.n_want == 0:
             return torch.empty((0, self.spec.vocab_size), dtype=torch.float32, device=x.device)
         h = self.final_norm.forward(x, ctx.want_rows)

@@ -6,16 +6,28 @@ import numpy as np
 import torch
 
 PAGE = 64
-Q_TILE = 128            # tokens of one workgroup of the prefill attention kernel
 
 
-class StepContext:
+class StepShared:
+    """What the parts of a step share: a value that depends on the step alone (a table of angles, the
+    index arrays of a kernel's grid) is made by the first part that asks for it under its key and
+    found by the others."""
+
+    def shared(self, key, make):
+        store = self.__dict__.setdefault("_shared", {})
+        if key not in store:
+            store[key] = make()
+        return store[key]
+
+
+class StepContext(StepShared):
     """All index arrays are int32 on the device, uploaded with one copy.
 
     per token   : token_ids, pos (position in its sequence), tok_slot (its sequence's slot)
     per sequence: seq_slot, seq_qstart (first token of the sequence in this step),
                   seq_qlen (tokens in this step), seq_ctx (context length after the step)
     want_rows   : rows of the step whose logits are asked for
+    The host keeps ``host_slots``, ``host_qlens`` and ``host_lens_before`` for parts that plan on the host.
     """
 
     def __init__(self, device, slots, tokens, lens_before, want):
@@ -31,16 +43,11 @@ class StepContext:
         tok_slot = [s for s, q in zip(slots, qlens) for _ in range(q)]
         want_rows = [int(qstart[i]) + w for i, ws in enumerate(want) for w in ws]
         self.n_want = len(want_rows)
-        tile_seq, tile_q0 = [], []
-        for i, q in enumerate(qlens):
-            for q0 in range(0, q, Q_TILE):
-                tile_seq.append(i)
-                tile_q0.append(q0)
-        self.n_tiles = len(tile_seq)
+        self.device = device
         fields = [("token_ids", flat), ("pos", pos), ("tok_slot", tok_slot), ("seq_slot", slots),
                   ("seq_qstart", qstart), ("seq_qlen", qlens),
                   ("seq_ctx", [l + q for l, q in zip(lens_before, qlens)]),
-                  ("want_rows", want_rows), ("tile_seq", tile_seq), ("tile_q0", tile_q0)]
+                  ("want_rows", want_rows)]
         sizes = [len(v) for _, v in fields]
         offs = np.concatenate([[0], np.cumsum([(s + 3) // 4 * 4 for s in sizes])])
         packed = np.zeros(int(offs[-1]) + 4, dtype=np.int32)
@@ -51,24 +58,26 @@ class StepContext:
             setattr(self, name, dev[int(o):int(o) + s])
         self._packed = dev
 
-    def prefill_meta(self) -> dict:
-        return {"tile_seq": self.tile_seq, "tile_q0": self.tile_q0, "n_tiles": self.n_tiles,
-                "seq_slot": self.seq_slot, "seq_qstart": self.seq_qstart, "seq_qlen": self.seq_qlen,
-                "seq_ctx": self.seq_ctx}
-
     def decode_splits(self, n_kv_heads: int, n_heads: int) -> int:
-        """How many ways the decode attention cuts each sequence's context so that the chip is filled."""
-        return decode_splits(self.n_seqs, n_kv_heads, n_heads, self.max_ctx)
+        """How many ways the decode attention of a mixer with these heads cuts each sequence's context."""
+        return decode_splits(self.n_seqs, n_kv_heads, n_heads, split_bucket(self.max_ctx))
 
 
-def decode_splits(n_seqs: int, n_kv_heads: int, n_heads: int, max_ctx: int) -> int:
-    waves = n_seqs * n_kv_heads * ((n_heads // n_kv_heads + 31) // 32)
+def split_bucket(max_ctx: int) -> int:
+    """The most splits that a context of this length is worth (a power of two up to 64): at least two
+    pages a split.  It is all that the split count needs to know of the lengths, so a recorded step
+    serves every length of one bucket."""
     pages = (max_ctx + PAGE - 1) // PAGE
+    s = max(1, min(pages // 2, 64))
+    return 1 << (s.bit_length() - 1)
+
+
+def decode_splits(n_seqs: int, n_kv_heads: int, n_heads: int, bucket: int) -> int:
+    """Splits of the context for a decode attention of ``n_seqs`` sequences (a power of two, at most
+    ``bucket``), so that the chip is filled."""
+    waves = n_seqs * n_kv_heads * ((n_heads // n_kv_heads + 31) // 32)
     # measured on MI355X: 1,024 waves fill the chip best, but from 512 waves on one pass without the
     # merge kernel is faster than two halves with it
     want = 1 if waves >= 512 else max(1, 1024 // max(1, waves))
-    s = max(1, min(want, pages // 2, 64))
-    p = 1
-    while p * 2 <= s:                 # powers of two, so that a captured step is reused for many lengths
-        p *= 2
-    return p
+    s = max(1, min(want, bucket))
+    return 1 << (s.bit_length() - 1)

@@ -455,6 +455,25 @@ def _check_pages(k_pages, v_pages, page_table, n_kv_heads, head_dim, dtype):
     _need(page_table.dtype == torch.int32 and page_table.dim() == 2, "page_table: int32 [slots, pages]")
 
 
+Q_TILE = 128            # tokens of one workgroup of the prefill attention kernel
+
+
+def prefill_meta(ctx) -> dict:
+    """The index arrays of attention_prefill for a step: the per-sequence arrays of the step and the
+    kernel's own list of tiles (one for every Q_TILE tokens of every sequence), which is made and
+    uploaded once per step, by the first attention layer that runs."""
+    def tiles():
+        tile_seq, tile_q0 = [], []
+        for i, n in enumerate(ctx.host_qlens):
+            for q0 in range(0, n, Q_TILE):
+                tile_seq.append(i)
+                tile_q0.append(q0)
+        both = torch.tensor([tile_seq, tile_q0], dtype=torch.int32).to(ctx.device)
+        return {"tile_seq": both[0], "tile_q0": both[1], "n_tiles": len(tile_seq)}
+    return dict(ctx.shared(("attention_prefill_tiles", Q_TILE), tiles), seq_slot=ctx.seq_slot,
+                seq_qstart=ctx.seq_qstart, seq_qlen=ctx.seq_qlen, seq_ctx=ctx.seq_ctx)
+
+
 def attention_prefill(q, kv, meta, n_heads, n_kv_heads, head_dim, scale, window) -> torch.Tensor:
     """16-bit attention for a step with whole prompts.  ``kv``: (k_pages, v_pages, page_stride,
     page_table); ``meta``: dict of int32 device arrays tile_seq, tile_q0, seq_slot, seq_qstart,
@@ -524,10 +543,14 @@ def argmax(logits: torch.Tensor, out: torch.Tensor | None = None) -> torch.Tenso
     return out
 
 
-def sample(logits, temperature: float, seq_slot=None, state=None, forced_r=None, out=None) -> torch.Tensor:
+def sample(logits, temperature: float, seq_slot=None, state=None, forced_r=None, out=None,
+           temperature_dev=None) -> torch.Tensor:
     """Temperature sampling; ``state`` is the [slots, 2] int64 (key, counter) table, ``forced_r``
-    (float32 [B]) replaces the generator for tests."""
-    _dev(logits, seq_slot, state, forced_r, out)
+    (float32 [B]) replaces the generator for tests.  ``temperature_dev`` (float32 [1] on the device, holding
+    the same positive value) is what the kernels read if given, so that a recorded step serves any temperature."""
+    _dev(logits, seq_slot, state, forced_r, out, temperature_dev)
+    if temperature_dev is not None:
+        _need(temperature_dev.dtype == torch.float32 and temperature_dev.numel() >= 1, "temperature_dev: float32 [1]")
     _need(logits.dtype == torch.float32 and logits.dim() == 2, "logits: float32 [B, V]")
     b = logits.shape[0]
     if temperature <= 0:
@@ -541,8 +564,8 @@ def sample(logits, temperature: float, seq_slot=None, state=None, forced_r=None,
     if forced_r is not None:
         _need(forced_r.dtype == torch.float32 and forced_r.numel() >= b, "forced_r: float32 [B]")
     ws = torch.empty((b * core().li_sample_ws_floats(logits.shape[1]),), dtype=torch.float32, device=logits.device)
-    _check(core().li_sample(_ptr(logits), b, logits.shape[1], c_float(temperature), _ptr(seq_slot), _ptr(state),
-                            _ptr(forced_r), _ptr(ws), _ptr(out), _stream()), "sample")
+    _check(core().li_sample(_ptr(logits), b, logits.shape[1], c_float(temperature), _ptr(temperature_dev),
+                            _ptr(seq_slot), _ptr(state), _ptr(forced_r), _ptr(ws), _ptr(out), _stream()), "sample")
     return out
 
 

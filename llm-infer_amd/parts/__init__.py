@@ -4,7 +4,7 @@ from .position import RotaryPosition, NoPosition
 from .attention import Attention
 from .feed_forward import GatedMLP
 from .embedding import Embedding, LMHead
-from .block import PreNormBlock
+from .block import Block, PreNormBlock, SubLayer
 
 __all__ = ["Part", "collect_params", "RMSNorm", "RotaryPosition", "NoPosition", "Attention", "GatedMLP",
-           "Embedding", "LMHead", "PreNormBlock"]
+           "Embedding", "LMHead", "Block", "PreNormBlock", "SubLayer"]

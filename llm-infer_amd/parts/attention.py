@@ -59,5 +59,5 @@ class Attention(Part):
             a = ops.attention_decode(q, kv, ctx.seq_slot, ctx.seq_ctx, ctx.n_seqs, H, K, hd, self.scale,
                                      self.window, ctx.decode_splits(K, H))
         else:
-            a = ops.attention_prefill(q, kv, ctx.prefill_meta(), H, K, hd, self.scale, self.window)
+            a = ops.attention_prefill(q, kv, ops.prefill_meta(ctx), H, K, hd, self.scale, self.window)
         ops.linear(a.view(a.shape[0], H * hd), self.wo, ops.EPI_ADD, out=residual)

@@ -4,17 +4,72 @@ from ..registry import register_block
 from .base import Part
 
 
-@register_block("pre_norm")
-class PreNormBlock(Part):
-    """x += mixer(norm(x)); x += feed_forward(norm(x))   (src/model/block.cpp:106-224)."""
+class SubLayer:
+    """A built sub-layer: its part, what the part is to the engine ("mixer" or "feed_forward"), the norm
+    on its input and the norm on its output (either may be None)."""
 
-    def __init__(self, mixer_norm, mixer, feed_forward_norm, feed_forward):
-        self.mixer_norm, self.mixer = mixer_norm, mixer
-        self.feed_forward_norm, self.feed_forward = feed_forward_norm, feed_forward
+    def __init__(self, role: str, part, norm=None, post_norm=None):
+        self.role, self.part, self.norm, self.post_norm = role, part, norm, post_norm
+
+    def parts(self) -> list:
+        return [p for p in (self.norm, self.part, self.post_norm) if p is not None]
+
+
+class Block(Part):
+    """An arrangement of sub-layers.  A block class is built from the list of its ``SubLayer``s and runs
+    them on the float32 residual stream ``x`` [T, hidden] in place: ``forward(x, ctx, cache_views,
+    owns_cache)``, where ``cache_views`` holds one view for each mixer of the layer, in their order."""
+
+    def __init__(self, sublayers):
+        self.sublayers = list(sublayers)
 
     def children(self):
-        return [self.mixer_norm, self.mixer, self.feed_forward_norm, self.feed_forward]
+        return [p for s in self.sublayers for p in s.parts()]
 
-    def forward(self, x, ctx, cache_view, owns_cache=True):
-        self.mixer.forward(self.mixer_norm.forward(x), ctx, cache_view, x, owns_cache)
-        self.feed_forward.forward(self.feed_forward_norm.forward(x), x)
+    # the first of each kind, for layers of the common shape
+    def _first(self, role):
+        for s in self.sublayers:
+            if s.role == role:
+                return s
+        return None
+
+    @property
+    def mixer(self):
+        s = self._first("mixer")
+        return s.part if s else None
+
+    @property
+    def mixer_norm(self):
+        s = self._first("mixer")
+        return s.norm if s else None
+
+    @property
+    def feed_forward(self):
+        s = self._first("feed_forward")
+        return s.part if s else None
+
+    @property
+    def feed_forward_norm(self):
+        s = self._first("feed_forward")
+        return s.norm if s else None
+
+
+@register_block("pre_norm")
+class PreNormBlock(Block):
+    """x += part(norm(x)) for each sub-layer in turn; for the Llama layer: x += mixer(norm(x));
+    x += feed_forward(norm(x))   (src/model/block.cpp:106-224)."""
+
+    def __init__(self, sublayers):
+        super().__init__(sublayers)
+        for s in self.sublayers:
+            if s.norm is None or s.post_norm is not None:
+                raise ValueError("a pre_norm block has one norm before each part and none after it")
+
+    def forward(self, x, ctx, cache_views, owns_cache=True):
+        views = iter(cache_views)
+        for s in self.sublayers:
+            h = s.norm.forward(x)
+            if s.role == "mixer":
+                s.part.forward(h, ctx, next(views), x, owns_cache)
+            else:
+                s.part.forward(h, x)

@@ -23,8 +23,10 @@ class Embedding(Part):
     def bind(self, tensors):
         self.weight = tensors["weight"]
 
-    def forward(self, tokens):
-        return ops.embed(self.weight, tokens)
+    def forward(self, ctx):
+        """The residual stream's first value for the step's tokens, float32 [T, hidden].  ``ctx`` is the
+        step (``token_ids``, and ``pos`` for an embedding that adds positions)."""
+        return ops.embed(self.weight, ctx.token_ids)
 
 
 @register_head("lm_head")

@@ -4,22 +4,27 @@ import torch
 
 from ..kernels import ops
 from ..registry import register_position
+from .base import Part
 
 
 @register_position("rope")
-class RotaryPosition:
+class RotaryPosition(Part):
     """Rotation of q and k by position: angle = pos * theta^(-i / rotary_dim) for the pair
     that starts at dimension i (include/kernels_cpu.hpp:82-100).  ``pairing`` "adjacent"
     rotates (i, i+1) as the reference does; "half" rotates (i/2, i/2 + rotary_dim/2).
 
-    A position encoding owns a table of one frequency per rotated pair; another
-    encoding of this family (scaled, interpolated) only fills the table differently.
-    Its one duty towards a mixer is ``rotate_store``: rotate q and k of the step's
-    tokens, write k and v into the layer's pages, and return q.
+    A position encoding is a part like the others: it may own tensors (``params`` under its
+    ``prefix``, handed over by ``bind``); this one owns none.  It keeps a table of one frequency per
+    rotated pair; another encoding of this family (scaled, interpolated, with learned factors) only
+    fills the table differently.  Layers whose position specs are equal share one instance.  Its one
+    duty towards a mixer is ``rotate_store``: rotate q and k of the step's tokens, write k and v into
+    the layer's pages, and return q.
     """
 
-    def __init__(self, *, theta: float, rotary_dim: int, head_dim: int, pairing: str = "adjacent", dtype, device):
+    def __init__(self, *, theta: float, rotary_dim: int, head_dim: int, pairing: str = "adjacent", prefix: str = "",
+                 dtype, device):
         self.rotary_dim, self.head_dim, self.pairing, self.theta = rotary_dim, head_dim, pairing, float(theta)
+        self.prefix = prefix
         i = torch.arange(0, rotary_dim, 2, dtype=torch.float32)
         # 1 / powf(theta, i / rotary_dim) in float32, as kernels_cpu.hpp:87
         inv = 1.0 / torch.pow(torch.tensor(float(theta), dtype=torch.float32), i / float(rotary_dim))
@@ -45,13 +50,9 @@ class RotaryPosition:
         rotate with the same frequencies."""
         if self.rotary_dim == 0 or self.pairing != "adjacent" or self.dtype == torch.float32:
             return None
-        cache = getattr(ctx, "_rope_tables", None)
-        if cache is None:
-            cache = ctx._rope_tables = {}
-        key = (self.theta, self.rotary_dim)
-        if key not in cache:
-            cache[key] = ops.rope_table(self.inv_freq, ctx.pos, ctx.n_tokens)
-        return cache[key]
+        # keyed by the frequencies themselves: two encodings that fill them differently never share a table
+        return ctx.shared(("rope_table", self.inv_freq.data_ptr(), self.rotary_dim),
+                          lambda: ops.rope_table(self.inv_freq, ctx.pos, ctx.n_tokens))
 
 
 def _project(part, h, w, ctx, kv_view, n_heads, n_kv_heads, head_dim, inv_freq, rotary_dim, fusable, table=None):
@@ -66,11 +67,11 @@ def _project(part, h, w, ctx, kv_view, n_heads, n_kv_heads, head_dim, inv_freq, 
 
 
 @register_position("none")
-class NoPosition:
+class NoPosition(Part):
     """No position encoding: q passes unrotated, k and v are written as they are."""
 
-    def __init__(self, *, dtype, device, **_):
-        self.dtype = dtype
+    def __init__(self, *, prefix: str = "", dtype, device, **_):
+        self.dtype, self.prefix = dtype, prefix
 
     def rotate_store(self, qkv, ctx, kv_view, n_heads, n_kv_heads, head_dim):
         k = v = table = stride = None

@@ -33,11 +33,13 @@ class Sampler:
         idx = torch.tensor(list(slots), dtype=torch.int64, device=cache.device)
         cache.seq_state.index_copy_(0, idx, rows)
 
-    def sample(self, logits: torch.Tensor, seq_slot: torch.Tensor, cache, out=None) -> torch.Tensor:
-        """logits float32 [B, V], seq_slot int32 [B] -> token ids int32 [B] on the device."""
+    def sample(self, logits: torch.Tensor, seq_slot: torch.Tensor, cache, out=None, temperature_dev=None) -> torch.Tensor:
+        """logits float32 [B, V], seq_slot int32 [B] -> token ids int32 [B] on the device.
+        ``temperature_dev``: this sampler's (positive) temperature as a float32 on the device, read by
+        the kernels instead of the host's value."""
         if self.temperature <= 0.0:
             return ops.argmax(logits, out)
-        return ops.sample(logits, self.temperature, seq_slot, cache.seq_state, out=out)
+        return ops.sample(logits, self.temperature, seq_slot, cache.seq_state, out=out, temperature_dev=temperature_dev)
 
     @staticmethod
     def token_prob(logits: torch.Tensor, tokens: torch.Tensor) -> torch.Tensor:

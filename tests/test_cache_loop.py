@@ -8,7 +8,7 @@ import torch
 from llm_infer_amd.cache import Cache, CacheError, KVSpec, PagePool, SlotAllocator, StateSpec
 from llm_infer_amd.config.spec import ConfigError, ModelSpec, PartSpec, ScheduleEntry
 from llm_infer_amd.engine.generate import BatchTracker, RequestError, plan_batches
-from llm_infer_amd.engine.step import decode_splits
+from llm_infer_amd.engine.step import decode_splits, split_bucket
 from llm_infer_amd.cli import parse_args
 from llm_infer_amd.tokenizer import Tokenizer
 
@@ -127,7 +127,7 @@ def test_schedule_validation():
     def spec(schedule, n_layers=2):
         ps = PartSpec("x")
         from llm_infer_amd.config.spec import LayerSpec
-        layer = LayerSpec("pre_norm", ps, ps, ps, ps)
+        layer = LayerSpec.mixer_then_feed_forward("pre_norm", ps, ps, ps, ps)
         return ModelSpec(8, 8, 8, ps, tuple([layer] * n_layers), tuple(schedule), ps, ps)
     spec([ScheduleEntry(0), ScheduleEntry(1), ScheduleEntry(0), ScheduleEntry(1, cache_from=1)]).validate()
     with pytest.raises(ConfigError, match="names layer 5"):
@@ -136,6 +136,15 @@ def test_schedule_validation():
         spec([ScheduleEntry(0, cache_from=1), ScheduleEntry(1)]).validate()
     with pytest.raises(ConfigError, match="keeps none of its own"):
         spec([ScheduleEntry(0), ScheduleEntry(1, cache_from=0), ScheduleEntry(0, cache_from=1)]).validate()
+    # a layer is a list of sub-layers, each a mixer or a feed-forward
+    from llm_infer_amd.config.spec import LayerSpec, SubLayerSpec
+    ps = PartSpec("x")
+    layer = LayerSpec("pre_norm", (SubLayerSpec("mixer", ps, ps), SubLayerSpec("mixer", ps, ps, ps), SubLayerSpec("feed_forward", ps)))
+    ModelSpec(8, 8, 8, ps, (layer,), (ScheduleEntry(0),), ps, ps).validate()
+    with pytest.raises(ConfigError, match="no sub-layer"):
+        ModelSpec(8, 8, 8, ps, (LayerSpec("pre_norm", ()),), (ScheduleEntry(0),), ps, ps).validate()
+    with pytest.raises(ConfigError, match="'mixer' or a 'feed_forward'"):
+        ModelSpec(8, 8, 8, ps, (LayerSpec("pre_norm", (SubLayerSpec("norm", ps),)),), (ScheduleEntry(0),), ps, ps).validate()
 
 
 def test_plan_batches():
@@ -182,11 +191,20 @@ def test_the_loop_knows_beforehand_whether_all_go_on():
 
 
 def test_decode_splits_fill_the_chip_and_are_powers_of_two():
-    assert decode_splits(1, 8, 32, 8192) == 64
-    assert decode_splits(8, 8, 32, 8192) == 16
-    assert decode_splits(64, 8, 32, 8192) == 1 and decode_splits(32, 8, 32, 8192) == 4
-    assert decode_splits(64, 32, 32, 4096) == 1
-    assert decode_splits(1, 8, 32, 100) == 1 and decode_splits(1, 1, 64, 640) == 4
+    def splits(n, k, h, ctx):
+        return decode_splits(n, k, h, split_bucket(ctx))
+    assert splits(1, 8, 32, 8192) == 64
+    assert splits(8, 8, 32, 8192) == 16
+    assert splits(64, 8, 32, 8192) == 1 and splits(32, 8, 32, 8192) == 4
+    assert splits(64, 32, 32, 4096) == 1
+    assert splits(1, 8, 32, 100) == 1 and splits(1, 1, 64, 640) == 4
+    # the bucket is all that the count knows of the lengths: at least two pages a split, at most 64 splits
+    assert [split_bucket(c) for c in (1, 64, 128, 192, 193, 256, 4096, 8192, 100_000)] == [1, 1, 1, 1, 2, 2, 32, 64, 64]
+    for ctx in range(1, 9000, 37):
+        pages = (ctx + 63) // 64
+        for n, k, h in ((1, 8, 32), (3, 1, 4), (8, 2, 2)):
+            s = splits(n, k, h, ctx)
+            assert s & (s - 1) == 0 and 1 <= s <= max(1, pages // 2)
 
 
 def test_launch_plans_cover_every_product_once():

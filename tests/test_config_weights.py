@@ -68,9 +68,13 @@ def test_model_spec_is_data():
     spec = llm_infer_amd.config_from_dict(TINY_B).model_spec()
     assert len(spec.layers) == 3 and [e.layer for e in spec.schedule] == [0, 1, 2]
     l1 = spec.layers[1]
-    assert l1.block == "pre_norm" and l1.mixer.kind == "attention" and l1.feed_forward.kind == "gated_mlp"
-    assert l1.mixer.params["n_kv_heads"] == 1 and l1.mixer.params["scale"] == 32 ** -0.5
-    assert l1.mixer.prefix == "model.layers.1.self_attn." and l1.position.params["theta"] == 500000.0
+    mix, ffn = l1.sublayers                                   # the sub-layers in the order in which they run
+    assert l1.block == "pre_norm" and (mix.role, ffn.role) == ("mixer", "feed_forward")
+    assert mix.part.kind == "attention" and ffn.part.kind == "gated_mlp"
+    assert mix.part.params["n_kv_heads"] == 1 and mix.part.params["scale"] == 32 ** -0.5
+    assert mix.part.prefix == "model.layers.1.self_attn." and l1.position.params["theta"] == 500000.0
+    assert mix.norm.prefix == "model.layers.1.input_layernorm." and mix.post_norm is None
+    assert ffn.norm.prefix == "model.layers.1.post_attention_layernorm." and ffn.norm.kind == "rmsnorm"
     assert spec.head.params["tied"] and spec.final_norm.params["eps"] == 1e-6
 
 

@@ -66,7 +66,7 @@ def _ctx(lens_before, tokens):
 @pytest.mark.parametrize("dt", [torch.float32, torch.bfloat16])
 def test_parts_alone(lib, dt):
     from llm_infer_amd.cache import Cache
-    from llm_infer_amd.parts import Attention, Embedding, GatedMLP, LMHead, PreNormBlock, RMSNorm, RotaryPosition
+    from llm_infer_amd.parts import Attention, Embedding, GatedMLP, LMHead, PreNormBlock, RMSNorm, RotaryPosition, SubLayer
     d, H, K, hd, F, V, eps, theta, rot = 112, 6, 3, 32, 200, 77, 1e-3, 777.0, 16
     g = torch.Generator().manual_seed(4)
     tol = 2e-5 if dt == torch.float32 else 3e-2
@@ -98,7 +98,7 @@ def test_parts_alone(lib, dt):
     toks = [torch.randint(0, V, (n,), generator=g).tolist() for n in lens]
     ctx = _ctx([0, 0], toks)
     # embedding
-    x = emb.forward(ctx.token_ids)
+    x = emb.forward(ctx)
     x_ref = torch.cat([w64["e.weight"][t] for t in toks])
     assert torch.equal(x.double().cpu(), x_ref)
     # norm
@@ -140,9 +140,9 @@ def test_parts_alone(lib, dt):
         cache.free_slot(sl)
     slots = [cache.alloc_slot(), cache.alloc_slot()]
     cache.grow(slots, lens)
-    blk = PreNormBlock(norm1, attn, norm2, ffn)
+    blk = PreNormBlock([SubLayer("mixer", attn, norm1), SubLayer("feed_forward", ffn, norm2)])
     xb = x.clone()
-    blk.forward(xb, ctx, cache.view(0))
+    blk.forward(xb, ctx, [cache.view(0)])
     wb = {"model.layers.0.input_layernorm.weight": w64["n1.weight"],
           "model.layers.0.post_attention_layernorm.weight": w64["n2.weight"]}
     for k in ("q_proj", "k_proj", "v_proj", "o_proj"):
@@ -509,10 +509,10 @@ def test_toy_architecture_with_a_stateful_mixer(lib):
             d, hd = r["width"], r["head"]
             norm = PartSpec("rmsnorm", {"size": d, "eps": r["eps"]})
             ffn = PartSpec("gated_mlp", {"hidden_size": d, "intermediate_size": r["ffn"]})
-            toy = LayerSpec("pre_norm", PartSpec("toy_decay", {"hidden_size": d, "state_size": r["state"],
+            toy = LayerSpec.mixer_then_feed_forward("pre_norm", PartSpec("toy_decay", {"hidden_size": d, "state_size": r["state"],
                                                                "decay": r["decay"]}, "l0.mix."),
                             ffn.with_prefix("l0.ffn."), norm.with_prefix("l0.n1."), norm.with_prefix("l0.n2."))
-            att = LayerSpec("pre_norm", PartSpec("attention", {"hidden_size": d, "n_heads": 2, "n_kv_heads": 1,
+            att = LayerSpec.mixer_then_feed_forward("pre_norm", PartSpec("attention", {"hidden_size": d, "n_heads": 2, "n_kv_heads": 1,
                                                                "head_dim": hd, "scale": hd ** -0.5}, "l1.mix."),
                             ffn.with_prefix("l1.ffn."), norm.with_prefix("l1.n1."), norm.with_prefix("l1.n2."),
                             PartSpec("rope", {"theta": 100.0, "rotary_dim": hd, "head_dim": hd}))
@@ -615,7 +615,7 @@ def test_toy_architecture_with_a_window_group(lib, dtype):
             for i, window in enumerate((None, 70)):
                 att = PartSpec("attention", {"hidden_size": d, "n_heads": 2, "n_kv_heads": 2, "head_dim": hd,
                                              "scale": hd ** -0.5, "window": window}, f"l{i}.mix.")
-                layers.append(LayerSpec("pre_norm", att, ffn.with_prefix(f"l{i}.ffn."), norm.with_prefix(f"l{i}.n1."),
+                layers.append(LayerSpec.mixer_then_feed_forward("pre_norm", att, ffn.with_prefix(f"l{i}.ffn."), norm.with_prefix(f"l{i}.n1."),
                                         norm.with_prefix(f"l{i}.n2."), rope))
             return ModelSpec(d, 40, 512, PartSpec("embedding", {"vocab_size": 40, "hidden_size": d}, "emb."),
                              tuple(layers), (ScheduleEntry(0), ScheduleEntry(1)), norm.with_prefix("final."),
@@ -724,7 +724,6 @@ def test_toy_routed_feed_forward_and_another_position_encoding(lib, dtype):
         def __init__(self, *, slowdown, **kw):
             super().__init__(**kw)
             self.inv_freq = self.inv_freq / float(slowdown)
-            self.theta = (self.theta, float(slowdown))          # the per-step table is keyed by it
 
     class RoutedConfig:
         def __init__(self, raw):
@@ -744,7 +743,7 @@ def test_toy_routed_feed_forward_and_another_position_encoding(lib, dtype):
                                              "scale": hd ** -0.5}, f"l{i}.mix.")
                 ffn = PartSpec("toy_top1", {"hidden_size": d, "expert_size": r["expert"], "n_experts": 3}, f"l{i}.moe.")
                 pos = PartSpec("toy_slow_rope", {"theta": 50.0, "rotary_dim": hd, "head_dim": hd, "slowdown": 4.0})
-                layers.append(LayerSpec("pre_norm", mix, ffn, norm.with_prefix(f"l{i}.n1."),
+                layers.append(LayerSpec.mixer_then_feed_forward("pre_norm", mix, ffn, norm.with_prefix(f"l{i}.n1."),
                                         norm.with_prefix(f"l{i}.n2."), pos))
             return ModelSpec(d, r["vocab"], r["positions"],
                              PartSpec("embedding", {"vocab_size": r["vocab"], "hidden_size": d}, "emb."),
@@ -857,15 +856,16 @@ def test_toy_norm_and_parallel_block(lib, dtype):
     class ParallelBlock(Part):
         """x += mixer(n(x)) + feed_forward(n(x)) with one norm; the second norm of the spec is unused."""
 
-        def __init__(self, mixer_norm, mixer, feed_forward_norm, feed_forward):
-            self.norm, self.mixer, self.feed_forward = mixer_norm, mixer, feed_forward
+        def __init__(self, sublayers):
+            mix, ffn = sublayers
+            self.norm, self.mixer, self.feed_forward = mix.norm, mix.part, ffn.part
 
         def children(self):
             return [self.norm, self.mixer, self.feed_forward]
 
-        def forward(self, x, ctx, cache_view, owns_cache=True):
+        def forward(self, x, ctx, cache_views, owns_cache=True):
             h = self.norm.forward(x)
-            self.mixer.forward(h, ctx, cache_view, x, owns_cache)
+            self.mixer.forward(h, ctx, cache_views[0], x, owns_cache)
             self.feed_forward.forward(h, x)
 
     class ParallelConfig:
@@ -886,7 +886,7 @@ def test_toy_norm_and_parallel_block(lib, dtype):
                                              "scale": hd ** -0.5}, f"h.{i}.attn.")
                 ffn = PartSpec("gated_mlp", {"hidden_size": d, "intermediate_size": r["ffn"]}, f"h.{i}.mlp.")
                 pos = PartSpec("rope", {"theta": 777.0, "rotary_dim": hd // 2, "head_dim": hd})
-                layers.append(LayerSpec("toy_parallel", mix, ffn, norm, norm, pos))
+                layers.append(LayerSpec.mixer_then_feed_forward("toy_parallel", mix, ffn, norm, norm, pos))
             return ModelSpec(d, r["vocab"], r["positions"],
                              PartSpec("embedding", {"vocab_size": r["vocab"], "hidden_size": d}, "wte."),
                              tuple(layers), tuple(ScheduleEntry(i) for i in range(r["layers"])),
@@ -949,3 +949,149 @@ def test_toy_norm_and_parallel_block(lib, dtype):
     assert a == b
     if dtype == "float32":
         assert a[1][0] == int(refs[1][-1].argmax())
+
+
+# ---------------------------------------------------------------------------
+# layers of other shapes: norms after the parts, three sub-layers, no feed-forward; a position
+# encoding that owns a tensor
+# ---------------------------------------------------------------------------
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_toy_layers_of_other_shapes_and_a_position_part_with_a_tensor(lib, dtype):
+    """A block with a norm before and after each part (four norms a layer), a layer of three sub-layers
+    (two attention mixers with caches of their own, then a feed-forward), a layer without feed-forward,
+    and a rotation whose frequencies are divided by factors that it owns as a tensor, shared by all
+    layers: all registered from here, described by a configuration, built and stepped by the engine
+    whole, cut and through generation, against a float64 reference of the same toy model."""
+    from llm_infer_amd.config.spec import LayerSpec, ModelSpec, PartSpec, ScheduleEntry, SubLayerSpec
+    from llm_infer_amd.engine import Engine
+    from llm_infer_amd.parts.block import Block
+    from llm_infer_amd.parts.position import RotaryPosition
+    from llm_infer_amd.weights.loader import ParamSpec
+
+    @lib.register_block("toy_sandwich")
+    class SandwichBlock(Block):
+        """x += post_norm(part(norm(x))) for each sub-layer; a sub-layer without a post norm adds directly."""
+
+        def forward(self, x, ctx, cache_views, owns_cache=True):
+            views = iter(cache_views)
+            for s in self.sublayers:
+                h = s.norm.forward(x)
+                out = x if s.post_norm is None else torch.zeros_like(x)
+                if s.role == "mixer":
+                    s.part.forward(h, ctx, next(views), out, owns_cache)
+                else:
+                    s.part.forward(h, out)
+                if s.post_norm is not None:
+                    x += s.post_norm.forward(out).float()
+
+    @lib.register_position("toy_factor_rope")
+    class FactorRotary(RotaryPosition):
+        """Rotation with each frequency divided by a factor; the factors are a tensor of the model."""
+
+        def params(self):
+            return {"weight": ParamSpec((self.rotary_dim // 2,), "vector", "ones")}
+
+        def bind(self, tensors):
+            self.factors = tensors["weight"]
+            self.inv_freq = self.inv_freq / self.factors
+
+    D, HD, F, V = 64, 16, 72, 60
+
+    class ShapesConfig:
+        def __init__(self, raw):
+            self.raw = raw
+
+        @classmethod
+        def from_dict(cls, raw):
+            return cls(raw)
+
+        def model_spec(self):
+            norm = PartSpec("rmsnorm", {"size": D, "eps": 1e-5})
+            pos = PartSpec("toy_factor_rope", {"theta": 300.0, "rotary_dim": HD, "head_dim": HD}, "rope_freqs.")
+
+            def att(prefix, n_heads, n_kv):
+                return PartSpec("attention", {"hidden_size": D, "n_heads": n_heads, "n_kv_heads": n_kv, "head_dim": HD,
+                                              "scale": HD ** -0.5}, prefix)
+            ffn = PartSpec("gated_mlp", {"hidden_size": D, "intermediate_size": F})
+            l0 = LayerSpec("toy_sandwich", (
+                SubLayerSpec("mixer", att("l0.a.", 4, 2), norm.with_prefix("l0.n1."), norm.with_prefix("l0.p1.")),
+                SubLayerSpec("feed_forward", ffn.with_prefix("l0.f."), norm.with_prefix("l0.n2."), norm.with_prefix("l0.p2."))), pos)
+            l1 = LayerSpec("pre_norm", (
+                SubLayerSpec("mixer", att("l1.a.", 4, 2), norm.with_prefix("l1.n1.")),
+                SubLayerSpec("mixer", att("l1.b.", 2, 1), norm.with_prefix("l1.n2.")),
+                SubLayerSpec("feed_forward", ffn.with_prefix("l1.f."), norm.with_prefix("l1.n3."))), pos)
+            l2 = LayerSpec("pre_norm", (SubLayerSpec("mixer", att("l2.a.", 2, 1), norm.with_prefix("l2.n1.")),), pos)
+            return ModelSpec(D, V, 256, PartSpec("embedding", {"vocab_size": V, "hidden_size": D}, "emb."),
+                             (l0, l1, l2), (ScheduleEntry(0), ScheduleEntry(1), ScheduleEntry(2)),
+                             norm.with_prefix("final."),
+                             PartSpec("lm_head", {"vocab_size": V, "hidden_size": D, "tied": True}, "head."))
+
+    lib.register_architecture("ShapesToyForCausalLM", ShapesConfig)
+    cfg = lib.config_from_dict({"architectures": ["ShapesToyForCausalLM"]})
+    eng = Engine.from_random(cfg, seed=6, dtype=dtype, max_tokens=1024)
+    model = Engine.from_random(cfg, seed=6, dtype="float32", max_tokens=64).model      # the same values as plain tensors
+    # one position part for all three layers, and its tensor is in the model's table once
+    assert len(eng.model.positions) == 1 and "rope_freqs.weight" in eng.model.params()
+    assert all(m.position is next(iter(eng.model.positions.values())) for ms in eng.model.layer_mixers for m in ms)
+    # four units of cache: two groups (2 KV heads: l0.a and l1.a; 1 KV head: l1.b and l2.a)
+    assert len(eng.model.cache_specs()) == 4 and len(eng.cache.groups) == 2
+    assert sorted(len(g.entries) for g in eng.cache.groups) == [2, 2]
+    factors = next(iter(model.positions.values())).factors.double().cpu()
+    assert (factors - 1).abs().max() > 1e-3              # they matter: angles differ by a radian at position 100
+
+    def dbl(t):
+        return t.double().cpu()
+
+    def rotate(v, posn):
+        i = torch.arange(0, HD, 2, dtype=torch.float64)
+        ang = posn.double()[:, None] * (1.0 / torch.pow(torch.tensor(300.0, dtype=torch.float64), i / HD) / factors)[None, :]
+        cos, sin = torch.cos(ang)[:, None, :], torch.sin(ang)[:, None, :]
+        out = v.clone()
+        out[..., 0::2] = v[..., 0::2] * cos - v[..., 1::2] * sin
+        out[..., 1::2] = v[..., 0::2] * sin + v[..., 1::2] * cos
+        return out
+
+    def ref_forward(toks):
+        n = len(toks)
+        x = dbl(model.embedding.weight)[toks]
+        posn = torch.arange(n)
+        for layer in model.layers:
+            for s in layer.sublayers:
+                h = P.rmsnorm(x, dbl(s.norm.weight), 1e-5)
+                if s.role == "mixer":
+                    a = s.part
+                    wq, wk, wv = dbl(a.wqkv).split([a.n_heads * HD, a.n_kv_heads * HD, a.n_kv_heads * HD])
+                    q = rotate((h @ wq.t()).view(n, a.n_heads, HD), posn)
+                    k = rotate((h @ wk.t()).view(n, a.n_kv_heads, HD), posn)
+                    y = P.attention(q, k, (h @ wv.t()).view(n, a.n_kv_heads, HD)).reshape(n, -1) @ dbl(a.wo).t()
+                else:
+                    gu = dbl(s.part.w_gate_up)
+                    y = P.swiglu(h, gu[0::2], gu[1::2], dbl(s.part.w_down))
+                if s.post_norm is not None:
+                    y = P.rmsnorm(y, dbl(s.post_norm.weight), 1e-5)
+                x = x + y
+        return P.rmsnorm(x, dbl(model.final_norm.weight), 1e-5) @ dbl(model.embedding.weight).t()
+
+    g = torch.Generator().manual_seed(12)
+    seqs = [torch.randint(0, V, (n,), generator=g).tolist() for n in (130, 4, 70)]
+    refs = [ref_forward(t) for t in seqs]
+    tol = 3e-5 if dtype == "float32" else 4e-2
+    scale = 1 + max(r.abs().max().item() for r in refs)
+    slots = [eng.alloc_slot() for _ in seqs]
+    whole = eng.step(slots, seqs, [list(range(len(t))) for t in seqs]).double().cpu()
+    assert (whole - torch.cat(refs)).abs().max().item() < tol * scale
+    for s in slots:
+        eng.free_slot(s)
+    slots = [eng.alloc_slot() for _ in seqs]
+    heads = [len(t) - 3 for t in seqs]
+    eng.step(slots, [t[:h] for t, h in zip(seqs, heads)])
+    for kk in range(3):
+        out = eng.step(slots, [[t[h + kk]] for t, h in zip(seqs, heads)]).double().cpu()
+        for i, (r, h) in enumerate(zip(refs, heads)):
+            assert (out[i] - r[h + kk]).abs().max().item() < tol * scale
+    for s in slots:
+        eng.free_slot(s)
+    a = eng.generate(seqs, max_new_tokens=5, temperature=0.0, use_graph=True)
+    b = eng.generate(seqs, max_new_tokens=5, temperature=0.0, use_graph=False)
+    assert a == b
+    assert eng.cache.slots.n_free == eng.cache.n_slots and eng.cache.tokens_free() == (eng.cache.n_pages - 1) * 64

@@ -269,7 +269,7 @@ def test_attention_whole_prompts_and_decode(ops, H, K, hd, lens, dt):
     if dt == torch.float32:
         out = ops.attention_f32(q_all, view.as_tuple(), ctx.pos, ctx.tok_slot, H, K, hd, scale, None)
     else:
-        out = ops.attention_prefill(q_all, view.as_tuple(), ctx.prefill_meta(), H, K, hd, scale, None)
+        out = ops.attention_prefill(q_all, view.as_tuple(), ops.prefill_meta(ctx), H, K, hd, scale, None)
     ref_all = torch.cat(refs)
     err = (out.double().cpu() - ref_all).abs().max().item()
     assert err < tol, err
@@ -314,7 +314,7 @@ def test_attention_window_and_far_key(ops, dt):
         if dt == torch.float32:
             out = ops.attention_f32(qd, view.as_tuple(), ctx.pos, ctx.tok_slot, H, K, hd, scale, window)
         else:
-            out = ops.attention_prefill(qd, view.as_tuple(), ctx.prefill_meta(), H, K, hd, scale, window)
+            out = ops.attention_prefill(qd, view.as_tuple(), ops.prefill_meta(ctx), H, K, hd, scale, window)
         assert (out.double().cpu() - ref).abs().max().item() < tol, window
         if window == 100:
             # position far+99 still sees the far key, far+100 does not
@@ -327,6 +327,60 @@ def test_attention_window_and_far_key(ops, dt):
                                         torch.tensor([n], dtype=torch.int32, device=DEV), 1, H, K, hd, scale,
                                         window, 2)
             assert (out1.double().cpu()[0] - ref[-1]).abs().max().item() < tol
+
+
+@pytest.mark.parametrize("dt", F16S)
+@pytest.mark.parametrize("window", [100, 64])
+def test_decode_attention_at_the_window_edge(ops, dt, window):
+    """The 16-bit decode kernel cuts the window exactly: a far key that outweighs all others is seen by
+    the last position that may see it and not by the next, with every count of splits; and with the
+    pages below the window given back and everything free filled with NaN."""
+    H, K, hd, n = 2, 1, 32, 300
+    scale = hd ** -0.5
+    tol = 3e-3 if dt == torch.float16 else 2.5e-2
+
+    def make(far):
+        g = torch.Generator().manual_seed(far)
+        k = torch.randn(n, K, hd, generator=g) * 0.1
+        v = torch.randn(n, K, hd, generator=g)
+        q = torch.randn(n, H, hd, generator=g) * 0.1
+        k[far, 0, :] = 0
+        k[far, 0, 3] = 12.0
+        q[:, :, 3] = 6.0
+        return k.to(dt), v.to(dt), q.to(dt)
+
+    def decode(view, q_row, ctx_len, splits):
+        return ops.attention_decode(q_row.to(DEV).contiguous(), view.as_tuple(), torch.zeros(1, dtype=torch.int32, device=DEV),
+                                    torch.tensor([ctx_len], dtype=torch.int32, device=DEV), 1, H, K, hd, scale,
+                                    window, splits).float().cpu()[0]
+
+    # a cache that keeps everything; the context length moves over the edge
+    far = 37
+    k, v, q = make(far)
+    cache, view = _fill_cache(ops, dt, K, hd, [(0, k, v)])
+    ref = _attn_ref(q.float(), k.float(), v.float(), window)
+    for splits in (1, 2, 8):
+        for ctx_len, sees in ((far + window, True), (far + window + 1, False)):
+            out = decode(view, q[ctx_len - 1:ctx_len], ctx_len, splits)
+            assert (out.double() - ref[ctx_len - 1]).abs().max().item() < tol, (splits, ctx_len)
+            assert ((out[0] - v[far, 0].float()).abs().max() < 0.05) == sees, (splits, ctx_len)
+    # a cache of a window group: pages that lie wholly below the window are given back, and whatever is
+    # free (the page that free table entries point at included) holds NaN
+    for far, sees in ((n - window, True), (n - window - 1, False)):
+        k, v, q = make(far)
+        cache, view = _fill_cache(ops, dt, K, hd, [(0, k, v)], window=window)
+        cache.trim_windows([0])
+        group = cache.groups[0]
+        first = group.first_needed_page(n)
+        assert first >= 3 and sorted(group.pages_of[0]) == list(range(first, (n + 63) // 64))
+        free = [p for p in range(group.n_pages) if p not in group.pool.held()]
+        group.storage[torch.tensor(free, device=DEV)] = float("nan")
+        ref = _attn_ref(q.float(), k.float(), v.float(), window)[-1]
+        for splits in (1, 2, 8):
+            out = decode(view, q[-1:], n, splits)
+            assert torch.isfinite(out).all(), (far, splits)
+            assert (out.double() - ref).abs().max().item() < tol, (far, splits)
+            assert ((out[0] - v[far, 0].float()).abs().max() < 0.05) == sees, (far, splits)
 
 
 def test_rope_store_rotation_and_cache_layout(ops):
