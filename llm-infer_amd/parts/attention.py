@@ -18,15 +18,22 @@ class Attention(Part):
 
     The three projections are one matrix product against the rows [Wq; Wk; Wv]; the sum
     for each row is unchanged by that.
+
+    The attention kernels take head sizes in steps of 16 up to 256.  Any other head size (the reference's
+    CPU path takes any, include/kernels_cpu.hpp:140-167) runs as the next multiple of 16: when the
+    weights are bound every head gets zero rows in Wq, Wk and Wv and zero columns in Wo, so the
+    dimensions added hold zeros in q, k and v, add nothing to a score and nothing to the output;
+    ``scale`` and the rotated dimensions stay those of the true head size.
     """
 
     def __init__(self, *, hidden_size, n_heads, n_kv_heads, head_dim, scale, window=None, position=None,
                  prefix, dtype, device):
         if n_heads % n_kv_heads != 0:
             raise ValueError("n_heads must be a multiple of n_kv_heads")
-        if head_dim % 16 != 0 or not 16 <= head_dim <= 256:
-            raise ValueError(f"head size {head_dim}: the attention kernels take multiples of 16 up to 256")
+        if not 1 <= head_dim <= 256:
+            raise ValueError(f"head size {head_dim}: the attention kernels take head sizes up to 256")
         self.hidden_size, self.n_heads, self.n_kv_heads, self.head_dim = hidden_size, n_heads, n_kv_heads, head_dim
+        self.padded_head_dim = (head_dim + 15) // 16 * 16        # what the kernels and the cache see
         self.scale, self.window, self.position = float(scale), window, position
         self.prefix, self.dtype, self.device = prefix, dtype, device
         self.wqkv = self.wo = None
@@ -36,18 +43,33 @@ class Attention(Part):
         return {"q_proj.weight": ParamSpec((h * hd, d)), "k_proj.weight": ParamSpec((k * hd, d)),
                 "v_proj.weight": ParamSpec((k * hd, d)), "o_proj.weight": ParamSpec((d, h * hd))}
 
+    def _pad_rows(self, w, heads):
+        """[heads * hd, d] -> [heads * padded, d]: zero rows after each head's own."""
+        hd, pad = self.head_dim, self.padded_head_dim
+        if pad == hd:
+            return w
+        out = torch.zeros((heads, pad, w.shape[1]), dtype=w.dtype, device=w.device)
+        out[:, :hd] = w.view(heads, hd, w.shape[1])
+        return out.view(heads * pad, w.shape[1])
+
     def bind(self, tensors):
-        wqkv = torch.cat([tensors["q_proj.weight"], tensors["k_proj.weight"], tensors["v_proj.weight"]], 0)
+        H, K, hd, pad = self.n_heads, self.n_kv_heads, self.head_dim, self.padded_head_dim
+        wqkv = torch.cat([self._pad_rows(tensors["q_proj.weight"], H), self._pad_rows(tensors["k_proj.weight"], K),
+                          self._pad_rows(tensors["v_proj.weight"], K)], 0)
         self.wqkv = ops.prepare_weight(wqkv)
-        self.wq = self.wqkv.prefix(self.n_heads * self.head_dim) if isinstance(self.wqkv, ops.TiledWeight) \
-            else self.wqkv[:self.n_heads * self.head_dim]
-        self.wo = ops.prepare_weight(tensors["o_proj.weight"])
+        self.wq = self.wqkv.prefix(H * pad) if isinstance(self.wqkv, ops.TiledWeight) else self.wqkv[:H * pad]
+        wo = tensors["o_proj.weight"]
+        if pad != hd:                               # zero columns after each head's own
+            full = torch.zeros((wo.shape[0], H, pad), dtype=wo.dtype, device=wo.device)
+            full[:, :, :hd] = wo.view(wo.shape[0], H, hd)
+            wo = full.view(wo.shape[0], H * pad)
+        self.wo = ops.prepare_weight(wo)
 
     def cache_spec(self):
-        return KVSpec(self.n_kv_heads, self.head_dim, self.window)
+        return KVSpec(self.n_kv_heads, self.padded_head_dim, self.window)
 
     def forward(self, h, ctx, cache_view, residual, owns_cache=True):
-        H, K, hd = self.n_heads, self.n_kv_heads, self.head_dim
+        H, K, hd = self.n_heads, self.n_kv_heads, self.padded_head_dim
         if owns_cache:
             q = self.position.project_rotate_store(h, self.wqkv, ctx, cache_view, H, K, hd)
         else:                                   # reads another layer's keys and values

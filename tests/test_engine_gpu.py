@@ -14,7 +14,8 @@ from tiny_configs import ALL
 
 pytestmark = pytest.mark.gpu
 
-LENGTHS = {"A": [40, 7, 100, 1, 64, 65, 33, 127], "B": [200, 1, 4, 9, 16, 31, 130, 255], "C": [300, 70, 5, 640, 129]}
+LENGTHS = {"A": [40, 7, 100, 1, 64, 65, 33, 127], "B": [200, 1, 4, 9, 16, 31, 130, 255], "C": [300, 70, 5, 640, 129],
+           "D": [150, 2, 64, 33, 190], "E": [90, 1, 65, 300]}
 
 
 def make_weights(cfg, seed, matrix_dtype=torch.bfloat16):

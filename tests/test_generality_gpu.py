@@ -163,6 +163,60 @@ def test_parts_alone(lib, dt):
     assert logits.dtype == torch.float32 and (logits.double().cpu() - l_ref).abs().max() < tol * (1 + l_ref.abs().max())
 
 
+@pytest.mark.parametrize("dt", [torch.float32, torch.float16])
+@pytest.mark.parametrize("hd,H,K,rot", [(72, 3, 1, 72), (20, 4, 2, 10), (100, 2, 2, 50), (250, 1, 1, 250)])
+def test_attention_part_with_head_sizes_that_are_no_multiple_of_16(dt, hd, H, K, rot):
+    """The attention part alone at head sizes that the kernels do not take as they are: it runs them as
+    the next multiple of 16 with zero rows and columns in its matrices, and the plain implementation at
+    the true head size (scale 1/sqrt(hd), rotation of the first ``rot`` dimensions) is what it must match,
+    for whole prompts and for decoded tokens.  Above 256 it refuses."""
+    from llm_infer_amd.cache import Cache
+    from llm_infer_amd.parts import Attention, RotaryPosition
+    d, theta = 64, 3000.0
+    g = torch.Generator().manual_seed(hd)
+    w = {n: (torch.randn(*shape, generator=g) * s).to(torch.float16) for n, shape, s in (
+        ("q_proj.weight", (H * hd, d), 0.3), ("k_proj.weight", (K * hd, d), 0.3), ("v_proj.weight", (K * hd, d), 0.2),
+        ("o_proj.weight", (d, H * hd), 0.1))}
+    pos = RotaryPosition(theta=theta, rotary_dim=rot, head_dim=hd, dtype=dt, device=DEV)
+    attn = Attention(hidden_size=d, n_heads=H, n_kv_heads=K, head_dim=hd, scale=hd ** -0.5, position=pos,
+                     prefix="a.", dtype=dt, device=DEV)
+    assert attn.padded_head_dim == -(-hd // 16) * 16 and attn.cache_spec().head_dim == attn.padded_head_dim
+    attn.bind({n: t.to(DEV).to(dt if dt != torch.float32 else torch.float32) for n, t in w.items()})
+    lens = [70, 3]
+    x = (torch.randn(sum(lens), d, generator=g)).to(dt)
+    w64 = {"a." + n: t.double() for n, t in w.items()}
+    s = dict(n_heads=H, n_kv=K, hd=hd, theta=theta, rotary=rot)
+    ref, off = [], 0
+    for n in lens:
+        ref.append(P.attention_part(x.double()[off:off + n], w64, "a.", s, torch.arange(n)))
+        off += n
+    ref = torch.cat(ref)
+    tol = (2e-5 if dt == torch.float32 else 6e-3) * (1 + ref.abs().max().item())
+    cache = Cache([attn.cache_spec()], 256, 128, dt, DEV, 2)
+    slots = [cache.alloc_slot(), cache.alloc_slot()]
+    # whole prompts
+    cache.grow(slots, lens)
+    res = torch.zeros((sum(lens), d), dtype=torch.float32, device=DEV)
+    attn.forward(x.to(DEV), _ctx([0, 0], [[0] * n for n in lens]), cache.view(0), res)
+    assert (res.double().cpu() - ref).abs().max().item() < tol
+    # the last token of each again, as a decode step over what the prompts left (positions n - 1 rewritten)
+    for sl in slots:
+        cache.free_slot(sl)
+    slots = [cache.alloc_slot(), cache.alloc_slot()]
+    cache.grow(slots, [n - 1 for n in lens])
+    head = torch.cat([x[:lens[0] - 1], x[lens[0]:lens[0] + lens[1] - 1]])
+    attn.forward(head.to(DEV), _ctx([0, 0], [[0] * (n - 1) for n in lens]), cache.view(0),
+                 torch.zeros((head.shape[0], d), dtype=torch.float32, device=DEV))
+    cache.grow(slots, lens)
+    last = torch.stack([x[lens[0] - 1], x[-1]])
+    res = torch.zeros((2, d), dtype=torch.float32, device=DEV)
+    attn.forward(last.to(DEV), _ctx([n - 1 for n in lens], [[0], [0]]), cache.view(0), res)
+    assert (res.double().cpu() - torch.stack([ref[lens[0] - 1], ref[-1]])).abs().max().item() < tol
+    with pytest.raises(ValueError, match="up to 256"):
+        Attention(hidden_size=d, n_heads=1, n_kv_heads=1, head_dim=272, scale=1.0, position=pos, prefix="a.",
+                  dtype=dt, device=DEV)
+
+
 # ---------------------------------------------------------------------------
 # long decoding, the first tokens, graph replay
 # ---------------------------------------------------------------------------

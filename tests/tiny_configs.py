@@ -26,4 +26,19 @@ TINY_C = {
     "max_position_embeddings": 1024, "tie_word_embeddings": False, "hidden_act": "gelu",
 }
 
-ALL = {"A": TINY_A, "B": TINY_B, "C": TINY_C}
+# head sizes that are no multiple of 16: 40 (GQA 6/2, 24 of the 40 dimensions rotated, tied head) and 100 (MHA)
+TINY_D = {
+    "architectures": ["LlamaForCausalLM"], "model_type": "llama",
+    "num_hidden_layers": 2, "hidden_size": 72, "num_attention_heads": 6, "num_key_value_heads": 2, "head_dim": 40,
+    "intermediate_size": 100, "vocab_size": 210, "rope_theta": 20000.0, "rms_norm_eps": 1e-5,
+    "partial_rotary_factor": 0.6,
+    "max_position_embeddings": 192, "tie_word_embeddings": True, "hidden_act": "silu",
+}
+TINY_E = {
+    "architectures": ["LlamaForCausalLM"], "model_type": "llama",
+    "num_hidden_layers": 1, "hidden_size": 200, "num_attention_heads": 2, "num_key_value_heads": 2,
+    "intermediate_size": 152, "vocab_size": 129, "rope_theta": 10000.0, "rms_norm_eps": 1e-6,
+    "max_position_embeddings": 320, "tie_word_embeddings": False, "hidden_act": "silu",
+}
+
+ALL = {"A": TINY_A, "B": TINY_B, "C": TINY_C, "D": TINY_D, "E": TINY_E}
