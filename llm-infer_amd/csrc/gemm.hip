@@ -291,14 +291,36 @@ __global__ void tile_weight_kernel(const T* __restrict__ W, T* __restrict__ out,
     *(v8*)(out + i * 8) = n < N ? *(const v8*)(W + (int64_t)n * K + k) : z;
 }
 
+// A norm split over two products of a decode step (up to 16 rows), so that no norm kernel runs between
+// them.  The product that adds into the residual stream (EPI_ADD) also leaves, for the rows x it has
+// just completed, (a) the sums of squares as one partial sum per workgroup and row, `ss` [blocks, 16], and
+// (b) x * w * scale rounded to the 16-bit type, `xw` [M, N], w being the weight of the norm that reads
+// x next (RowsOut).  The next product takes `xw` as its X and multiplies its sums by
+// 1 / (scale * sqrt(mean(x^2) + eps)) from the partial sums (RowScale): together  W . (x / rms * w),
+// the norm of include/kernels_cpu.hpp:43-54 in another order of rounding.  `scale` keeps x * w inside
+// float16's range.
+struct RowsOut {
+    float* ss;               // [gridDim.x, 16]
+    void* xw;                // [M, N] in the product's 16-bit type
+    const float* w;          // [N] weight of the next norm
+    float scale;
+};
+struct RowScale {
+    const float* ss;         // [P, 16]
+    int P;
+    float eps;               // of the norm
+    float inv_scale;         // 1 / RowsOut.scale
+};
+
 template <class T, int NT, int MT, int KW>
 __global__ __launch_bounds__(64 * KW) void gemv_tiled_kernel(const T* __restrict__ X, const T* __restrict__ Wt,
-                                                             int K, Epilogue e) {
+                                                             int K, Epilogue e, RowsOut ro, RowScale rsc) {
     // NT tiles of 16 rows of W and MT tiles of 16 rows of X per wave; W comes from HBM once, the
     // rows of X from the caches (they are few)
     typedef typename Vec<T>::v8 v8;
     constexpr int U = (NT + MT) <= 2 ? 8 : ((NT + MT) <= 4 ? 4 : 2);   // 32-element steps of K in flight
     __shared__ float part[KW][NT * MT][64][4];
+    __shared__ float ss_wave[KW][16];
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int r = lane & 15, g = lane >> 4;
     const int tile0 = blockIdx.x * NT;
@@ -321,6 +343,22 @@ __global__ __launch_bounds__(64 * KW) void gemv_tiled_kernel(const T* __restrict
     for (int t = 0; t < NT; ++t)
 #pragma unroll
         for (int j = 0; j < MT; ++j) acc[t][j] = f32x4{0.f, 0.f, 0.f, 0.f};
+    // RowScale (rows 0..15 only): the partial sums of squares of row r are dealt to the waves, and within a
+    // wave to the four lanes of the row; the loads are issued here and used after the main loop
+    float ss_mine = 0.f;
+    if (MT == 1 && rsc.ss) {
+        // partial sum p of row r lies at ss[p * 16 + r]: the 16 lanes of a group read 64 contiguous bytes
+        const float* p = rsc.ss + r;
+        const int share = (rsc.P + 4 * KW - 1) / (4 * KW);
+        const int lo = (wave * 4 + g) * share, hi = min(rsc.P, lo + share);
+        for (int i = lo; i < hi; i += 8) {
+            float v[8];
+#pragma unroll
+            for (int c = 0; c < 8; ++c) v[c] = p[min(i + c, hi - 1) * 16];
+#pragma unroll
+            for (int c = 0; c < 8; ++c) ss_mine += (i + c < hi) ? v[c] : 0.f;
+        }
+    }
     for (int s0 = s_begin; s0 < s_end; s0 += U) {
         v8 a[U][NT], b[U][MT];
 #pragma unroll
@@ -338,6 +376,11 @@ __global__ __launch_bounds__(64 * KW) void gemv_tiled_kernel(const T* __restrict
             for (int t = 0; t < NT; ++t)
 #pragma unroll
                 for (int j = 0; j < MT; ++j) acc[t][j] = mfma16(a[u][t], b[u][j], acc[t][j]);
+    }
+    if (MT == 1 && rsc.ss) {
+        ss_mine += __shfl_xor(ss_mine, 16, WAVE);
+        ss_mine += __shfl_xor(ss_mine, 32, WAVE);
+        if (g == 0) ss_wave[wave][r] = ss_mine;
     }
     if (KW > 1) {
 #pragma unroll
@@ -358,6 +401,47 @@ __global__ __launch_bounds__(64 * KW) void gemv_tiled_kernel(const T* __restrict
                     for (int w = 1; w < KW; ++w) v += part[w][t * MT + j][lane][q];
                     acc[t][j][q] = v;
                 }
+    }
+    if (MT == 1 && rsc.ss) {
+        // this lane's row: the waves' sums in wave order, then 1 / (scale * rms)
+        float ss = ss_wave[0][r];
+        for (int w = 1; w < KW; ++w) ss += ss_wave[w][r];
+        const float f = rsc.inv_scale / sqrtf(ss / (float)K + rsc.eps);
+#pragma unroll
+        for (int t = 0; t < NT; ++t)
+#pragma unroll
+            for (int q = 0; q < 4; ++q) acc[t][0][q] *= f;
+    }
+    if (ro.ss) {
+        // EPI_ADD, and what RowsOut asks for (the host has checked: N a multiple of 4, at most 16 rows)
+        float sq[MT];
+#pragma unroll
+        for (int j = 0; j < MT; ++j) {
+            sq[j] = 0.f;
+            const int m = 16 * j + r;
+#pragma unroll
+            for (int t = 0; t < NT; ++t) {
+                const int n = (tile0 + t) * 16 + 4 * g;
+                if (m < e.M && n < e.N) {
+                    float* c = (float*)e.C + (int64_t)m * e.N + n;
+                    f32x4 o = *(f32x4*)c;
+                    const f32x4 wv = *(const f32x4*)(ro.w + n);
+                    typename Vec<T>::v4 xw;
+#pragma unroll
+                    for (int q = 0; q < 4; ++q) {
+                        o[q] += acc[t][j][q];
+                        sq[j] = fmaf(o[q], o[q], sq[j]);
+                        xw[q] = from_f32<T>(o[q] * wv[q] * ro.scale);
+                    }
+                    *(f32x4*)c = o;
+                    *(typename Vec<T>::v4*)((T*)ro.xw + (int64_t)m * e.N + n) = xw;
+                }
+            }
+            sq[j] += __shfl_xor(sq[j], 16, WAVE);
+            sq[j] += __shfl_xor(sq[j], 32, WAVE);
+            if (g == 0) ro.ss[(int64_t)blockIdx.x * 16 + m] = sq[j];      // (rows beyond M: zeros)
+        }
+        return;
     }
 #pragma unroll
     for (int t = 0; t < NT; ++t)
@@ -596,27 +680,50 @@ extern "C" int li_tile_weight(const void* W, void* out, int dt, int N, int K, hi
     return LI_OK;
 }
 
+// ro (may be null; mode EPI_ADD, at most 16 rows): RowsOut, with li_gemv_tiled_blocks(...) partial sums a
+// row.  rsc (may be null; at most 16 rows): RowScale.
+static void gemv_tiled_shape(int M, int N, int K, int& nt, int& kw, int& blocks) {
+    const int n_tiles = (N + 15) / 16;
+    const int mt = (M + 15) / 16;
+    if (nt <= 0) nt = (mt >= 2 || (M > 12 && N >= 16384)) ? 2 : 1;           // measured on MI355X
+    if (mt >= 3) nt = 2;
+    blocks = (n_tiles + nt - 1) / nt;
+    if (kw <= 0) kw = (K >= 8192 || blocks < 320 || blocks > 4096) ? 8 : 4;   // measured on MI355X
+    while (kw * nt * (mt == 3 ? 4 : mt) > 64) kw >>= 1;                       // the partial sums fit 64 KiB of LDS
+}
+
+// workgroups of li_gemv_tiled for this product (= partial sums a row that ss_out receives)
+extern "C" int li_gemv_tiled_blocks(int M, int N, int K, int nt, int kw) {
+    int blocks = 0;
+    gemv_tiled_shape(M, N, K, nt, kw, blocks);
+    return blocks;
+}
+
 extern "C" int li_gemv_tiled(const void* X, const void* Wt, int dt, void* C, int out_dt, int mode,
-                             int M, int N, int K, int nt, int kw, const RopeStore* rs, hipStream_t stream) {
+                             int M, int N, int K, int nt, int kw, const RopeStore* rs, const RowsOut* ro,
+                             const RowScale* rsc, hipStream_t stream) {
     int rc = check_common(X, Wt, C, M, N, K, mode, out_dt);
     if (rc) return rc;
     if (dt != DT_F16 && dt != DT_BF16) return LI_BAD_ARG;
     if (M > 64) return LI_BAD_ARG;
     if (K % 32 != 0 || ((uintptr_t)X & 15) || ((uintptr_t)Wt & 15)) return LI_UNSUPPORTED;
+    if (ro && (mode != EPI_ADD || M > 16 || (N & 3) || !ro->ss || !ro->xw || !ro->w || !(ro->scale > 0.f) ||
+               (((uintptr_t)C | (uintptr_t)ro->w) & 15) || ((uintptr_t)ro->xw & 7)))
+        return LI_BAD_ARG;
+    if (rsc && (M > 16 || !rsc->ss || rsc->P <= 0 || !(rsc->inv_scale > 0.f))) return LI_BAD_ARG;
     if (M == 0) return LI_OK;
     Epilogue e;
     rc = make_epilogue(e, C, mode, out_dt, M, N, rs);
     if (rc) return rc;
-    const int n_tiles = (N + 15) / 16;
     const int mt = (M + 15) / 16;
-    if (nt <= 0) nt = (mt >= 2 || (M > 12 && N >= 16384)) ? 2 : 1;           // measured on MI355X
-    if (mt >= 3) nt = 2;
-    const int blocks = (n_tiles + nt - 1) / nt;
-    if (kw <= 0) kw = (K >= 8192 || blocks < 320 || blocks > 4096) ? 8 : 4;   // measured on MI355X
-    while (kw * nt * (mt == 3 ? 4 : mt) > 64) kw >>= 1;                       // the partial sums fit 64 KiB of LDS
+    int blocks = 0;
+    gemv_tiled_shape(M, N, K, nt, kw, blocks);
     if (kw < 2) return LI_BAD_ARG;
+    const RowsOut no_out{};
+    const RowScale no_scale{};
 #define LAUNCH(T, NT, MT, KW) \
-    gemv_tiled_kernel<T, NT, MT, KW><<<blocks, 64 * KW, 0, stream>>>((const T*)X, (const T*)Wt, K, e)
+    gemv_tiled_kernel<T, NT, MT, KW><<<blocks, 64 * KW, 0, stream>>>((const T*)X, (const T*)Wt, K, e, \
+                                                                     ro ? *ro : no_out, rsc ? *rsc : no_scale)
 #define PICK_KW(T, NT, MT)                                \
     do {                                                  \
         if (kw == 4) LAUNCH(T, NT, MT, 4);                \

@@ -116,7 +116,14 @@ class DecoderModel(Part):
         for i, e in enumerate(self.schedule):
             owner = i if e.cache_from is None else e.cache_from
             views = [cache.view(self._unit[owner, k]) for k in range(len(self.layer_mixers[e.layer]))]
-            self.layers[e.layer].forward(x, ctx, views, e.cache_from is None)
+            layer = self.layers[e.layer]
+            if getattr(layer, "takes_next_norm", False):
+                # the norm that reads the residual stream after this layer: the next layer's first
+                nxt = self.layers[self.schedule[i + 1].layer] if i + 1 < len(self.schedule) else None
+                first = getattr(nxt, "first_norm", None)
+                layer.forward(x, ctx, views, e.cache_from is None, next_norm=first() if first else None)
+            else:
+                layer.forward(x, ctx, views, e.cache_from is None)
         if ctx.n_want == 0:
             return torch.empty((0, self.spec.vocab_size), dtype=torch.float32, device=x.device)
         h = self.final_norm.forward(x, ctx.want_rows)

@@ -78,6 +78,7 @@ def embed(table: torch.Tensor, tokens: torch.Tensor, out: torch.Tensor | None = 
     if out is None:
         out = torch.empty((n, d), dtype=torch.float32, device=table.device)
     _need(out.dtype == torch.float32 and out.shape == (n, d), "out: float32 [T, d]")
+    _drop_row_stats(out)
     _check(core().li_embed(_ptr(table), DT[table.dtype], _ptr(tokens), _ptr(out), n, d, vocab, _stream()), "embed")
     return out
 
@@ -97,6 +98,59 @@ def rmsnorm(x: torch.Tensor, w: torch.Tensor, eps: float, out_dtype, rows: torch
     _check(core().li_rmsnorm(_ptr(x), _ptr(w), _ptr(rows), _ptr(out), DT[out_dtype], n, x.shape[1],
                              c_float(eps), _stream()), "rmsnorm")
     return out
+
+
+class _RowsOut(ctypes.Structure):
+    _fields_ = [("ss", c_void_p), ("xw", c_void_p), ("w", c_void_p), ("scale", c_float)]
+
+
+class _RowScale(ctypes.Structure):
+    _fields_ = [("ss", c_void_p), ("P", c_int), ("eps", c_float), ("inv_scale", c_float)]
+
+
+class LazyNorm:
+    """A norm whose last step has not been taken yet, for the few rows of a decode step.  The product that
+    last added into the float32 rows ``x`` also left ``xw`` = x * weight * scale in the 16-bit type and
+    the rows' sums of squares as partial sums ``ss`` [P, 16]; the product that reads the norm takes
+    ``xw`` as its X and multiplies its sums by 1 / (scale * rms).  ``linear`` does that where its kernel
+    can (up to 16 rows against a tiled weight); everywhere else ``tensor()`` runs the norm kernel."""
+
+    def __init__(self, x, weight, eps, dtype, xw, ss, scale):
+        self.x, self.weight, self.eps, self.dtype = x, weight, float(eps), dtype
+        self.xw, self.ss, self.scale = xw, ss, float(scale)
+        self.shape, self.device = x.shape, x.device
+
+    def dim(self):
+        return 2
+
+    def tensor(self) -> torch.Tensor:
+        return rmsnorm(self.x, self.weight, self.eps, self.dtype)
+
+
+def expect_norm(x: torch.Tensor, weight) -> None:
+    """Says which norm weight (float32 [width], or None) will read the rows of ``x`` next.  A product
+    that adds into ``x`` may then prepare that norm (``LazyNorm``).  Only a hint: a norm with another
+    weight, or rows that something else has written to since, get the norm kernel."""
+    x._li_next_norm = weight
+
+
+def _drop_row_stats(x) -> None:
+    if x is not None and getattr(x, "_li_rows", None) is not None:
+        x._li_rows = None
+
+
+def lazy_rmsnorm(x: torch.Tensor, w: torch.Tensor, eps: float, out_dtype):
+    """A ``LazyNorm`` of ``x`` if the product that last added into ``x`` prepared this very norm (same
+    weight tensor, same 16-bit type) and nothing has written to ``x`` since (torch counts its own
+    in-place writes in ``_version``; every kernel of this library that writes into a tensor drops the
+    record first); else None."""
+    rec = getattr(x, "_li_rows", None)
+    if rec is None:
+        return None
+    xw, ss, scale, weight, version = rec
+    if weight is not w or version != x._version or xw.dtype != out_dtype or xw.shape != x.shape:
+        return None
+    return LazyNorm(x, w, eps, out_dtype, xw, ss, scale)
 
 
 class _RopeStore(ctypes.Structure):
@@ -154,6 +208,15 @@ def linear(x: torch.Tensor, w, mode: int = EPI_STORE, out: torch.Tensor | None =
     interleaved gate/up rows of W (C has N/2 columns; EPI_SWIGLU: silu, EPI_GEGLU: gelu).  ``force`` picks a kernel for tests."""
     tiled = isinstance(w, TiledWeight)
     wd = w.data if tiled else w
+    _drop_row_stats(out)                   # whatever this call writes into `out`, an older record is void
+    lazy = None
+    if isinstance(x, LazyNorm):
+        # the kernel that finishes the norm: gemv_tiled, for up to 16 rows
+        if tiled and force is None and x.dtype == w.dtype and x.shape[0] <= 16 and wd.data_ptr() % 16 == 0:
+            lazy = x
+            x = lazy.xw
+        else:
+            x = x.tensor()
     _dev(x, wd, out)
     _need(x.dim() == 2 and len(w.shape) == 2 and x.shape[1] == w.shape[1], f"linear: x {tuple(x.shape)} w {tuple(w.shape)}")
     m, k = x.shape
@@ -183,9 +246,25 @@ def linear(x: torch.Tensor, w, mode: int = EPI_STORE, out: torch.Tensor | None =
         # rows (128 against a matrix of many rows) they go through LDS once per workgroup; beyond
         # that the tiled GEMM is faster
         if kind == "gemv_mfma" or (force is None and (m <= 16 or (m <= 32 and n * k <= (1 << 25)))):
-            _check(lib.li_gemv_tiled(_ptr(x), _ptr(wd), DT[x.dtype], _ptr(out), out_dt, mode, m, n, k, 0, 0,
-                                     rs, _stream()), "gemv_tiled")
+            ro = rsc = None
+            nxt = getattr(out, "_li_next_norm", None) if mode == EPI_ADD else None
+            if (nxt is not None and m <= 16 and n % 32 == 0 and out.data_ptr() % 16 == 0 and nxt.dtype == torch.float32
+                    and nxt.shape == (n,) and nxt.is_cuda and nxt.data_ptr() % 16 == 0):
+                # the rows of `out` are about to be complete rows of a residual stream that this norm reads
+                # next: leave x * weight in 16 bits and the sums of squares for the product behind the norm
+                ss = torch.empty((lib.li_gemv_tiled_blocks(m, n, k, 0, 0), 16), dtype=torch.float32, device=x.device)
+                xw = torch.empty((m, n), dtype=x.dtype, device=x.device)
+                scale = 0.125 if x.dtype == torch.float16 else 1.0        # x * w stays inside float16's range
+                ro = _RowsOut(ss.data_ptr(), xw.data_ptr(), nxt.data_ptr(), scale)
+            if lazy is not None:
+                rsc = _RowScale(lazy.ss.data_ptr(), lazy.ss.shape[0], lazy.eps, 1.0 / lazy.scale)
+            _check(lib.li_gemv_tiled(_ptr(x), _ptr(wd), DT[x.dtype], _ptr(out), out_dt, mode, m, n, k, 0, 0, rs,
+                                     ctypes.byref(ro) if ro is not None else None,
+                                     ctypes.byref(rsc) if rsc is not None else None, _stream()), "gemv_tiled")
+            if ro is not None:
+                out._li_rows = (xw, ss, scale, nxt, out._version)
             return out
+        _need(lazy is None, "a norm is finished by gemv_tiled alone")
         if force is None and (m <= 96 or (m <= 128 and n >= 16384)):
             kind = "stream"
         elif force is None and m * k * 2 < (1 << 32):
@@ -395,6 +474,7 @@ def rope_table(inv_freq: torch.Tensor, pos: torch.Tensor, n_tokens: int) -> torc
 
 def linear_rope_store(x, w, inv_freq, rotary_dim, pos, tok_slot, page_table, page_stride, k_pages, v_pages,
                       n_heads, n_kv_heads, head_dim, out_dtype, force=None, cos_sin=None) -> torch.Tensor:
+    # (x may be a LazyNorm: linear sorts that out)
     """q, k, v = x W^T with the rotation (adjacent pairs) and the cache write done in the product's
     epilogue, on the float32 accumulators: the same result as linear (float32) followed by
     rope_store, without the round trip.  Returns q [T, H, hd]."""
@@ -604,5 +684,5 @@ def gemv_tiled(x, w: TiledWeight, mode=EPI_STORE, out_dtype=None, nt=0, kw=0):
     n_out = w.n // 2 if mode in GATED else w.n
     out = torch.empty((m, n_out), dtype=out_dtype or x.dtype, device=x.device)
     _check(core().li_gemv_tiled(_ptr(x), _ptr(w.data), DT[x.dtype], _ptr(out), DT[out.dtype], mode, m, w.n, k,
-                                nt, kw, None, _stream()), "gemv_tiled")
+                                nt, kw, None, None, None, _stream()), "gemv_tiled")
     return out

@@ -26,6 +26,8 @@ class Attention(Part):
     ``scale`` and the rotated dimensions stay those of the true head size.
     """
 
+    takes_lazy_norm = True      # the normed input goes to ops.linear as it comes
+
     def __init__(self, *, hidden_size, n_heads, n_kv_heads, head_dim, scale, window=None, position=None,
                  prefix, dtype, device):
         if n_heads % n_kv_heads != 0:

@@ -1,5 +1,6 @@
 from __future__ import annotations
 
+from ..kernels import ops
 from ..registry import register_block
 from .base import Part
 
@@ -25,6 +26,10 @@ class Block(Part):
 
     def children(self):
         return [p for s in self.sublayers for p in s.parts()]
+
+    def first_norm(self):
+        """The norm that reads the residual stream first in this layer (None: the first part takes it raw)."""
+        return self.sublayers[0].norm
 
     # the first of each kind, for layers of the common shape
     def _first(self, role):
@@ -58,6 +63,7 @@ class Block(Part):
 class PreNormBlock(Block):
     """x += part(norm(x)) for each sub-layer in turn; for the Llama layer: x += mixer(norm(x));
     x += feed_forward(norm(x))   (src/model/block.cpp:106-224)."""
+    takes_next_norm = True          # forward accepts ``next_norm``
 
     def __init__(self, sublayers):
         super().__init__(sublayers)
@@ -65,10 +71,19 @@ class PreNormBlock(Block):
             if s.norm is None or s.post_norm is not None:
                 raise ValueError("a pre_norm block has one norm before each part and none after it")
 
-    def forward(self, x, ctx, cache_views, owns_cache=True):
+    def forward(self, x, ctx, cache_views, owns_cache=True, next_norm=None):
+        """``next_norm``: the norm that reads ``x`` after this layer, if the caller knows it."""
         views = iter(cache_views)
-        for s in self.sublayers:
-            h = s.norm.forward(x)
+        for i, s in enumerate(self.sublayers):
+            # a part that only passes its input on to ops.linear may get a norm whose last step is taken
+            # inside that product (ops.LazyNorm)
+            if getattr(s.part, "takes_lazy_norm", False) and getattr(s.norm, "can_be_lazy", False):
+                h = s.norm.forward(x, lazy=True)
+            else:
+                h = s.norm.forward(x)
+            # and the product that completes the rows of x may prepare the norm that reads them next
+            after = self.sublayers[i + 1].norm if i + 1 < len(self.sublayers) else next_norm
+            ops.expect_norm(x, after.weight if getattr(after, "can_be_lazy", False) else None)
             if s.role == "mixer":
                 s.part.forward(h, ctx, next(views), x, owns_cache)
             else:

@@ -19,6 +19,8 @@ class GatedMLP(Part):
     anything is written; each row's sum is what it would be alone.
     """
 
+    takes_lazy_norm = True      # the normed input goes to ops.linear as it comes
+
     def __init__(self, *, hidden_size, intermediate_size, activation="silu", prefix, dtype, device):
         if activation not in ("silu", "gelu"):
             raise ValueError(f"gated_mlp: activation {activation!r} is not built (silu and gelu are)")

@@ -156,6 +156,68 @@ def test_linear_tiled_weights(ops, M, N, K, dt):
         ops.tile_weight(w[:, :K - 8].contiguous())
 
 
+@pytest.mark.parametrize("dt", F16S)
+@pytest.mark.parametrize("M,d,K2,N2", [(1, 4096, 4096, 6144), (8, 4096, 14336, 28672), (16, 96, 160, 200), (5, 2048, 64, 128256)])
+def test_norm_split_over_two_products(ops, M, d, K2, N2, dt):
+    """A decode step's product that adds into the residual stream prepares the norm that reads the rows
+    next (x * weight in 16 bits, sums of squares), and the product behind the norm finishes it: the same
+    result as norm kernel + product, without the kernel.  The preparation is void as soon as anything
+    else writes to the rows, and for any other norm."""
+    g = torch.Generator().manual_seed(M + d)
+    x0 = torch.randn(M, d, generator=g) * 3
+    a = (torch.randn(M, K2, generator=g) * 0.5).to(dt)
+    wo = (torch.randn(d, K2, generator=g) * 0.05).to(dt)
+    wn = (1 + 0.1 * torch.randn(d, generator=g)).to(DEV)
+    w2 = (torch.randn(N2, d, generator=g) * 0.05).to(dt)
+    eps = 1e-5
+    wot = ops.tile_weight(wo.to(DEV))
+    x = x0.to(DEV)
+    ops.linear(a.to(DEV), wot, ops.EPI_ADD, out=x)
+    assert ops.lazy_rmsnorm(x, wn, eps, dt) is None                         # nobody said which norm comes next
+    x = x0.to(DEV)
+    ops.expect_norm(x, wn)
+    ops.linear(a.to(DEV), wot, ops.EPI_ADD, out=x)
+    x_ref = x0.double() + a.double() @ wo.double().t()
+    assert (x.double().cpu() - x_ref).abs().max().item() < 1e-3 * (1 + x_ref.abs().max().item())
+    ln = ops.lazy_rmsnorm(x, wn, eps, dt)
+    assert isinstance(ln, ops.LazyNorm) and ln.dtype == dt and tuple(ln.shape) == (M, d)
+    assert torch.allclose(ln.ss.double().sum(0).cpu()[:M], (x.double().cpu() ** 2).sum(1), rtol=1e-5)
+    assert torch.allclose(ln.xw.double().cpu(), x.double().cpu() * wn.double().cpu() * ln.scale, rtol=2.0 ** -8)
+    w2t = ops.tile_weight(w2.to(DEV))
+    fused = ops.linear(ln, w2t, out_dtype=torch.float32)
+    h = ops.rmsnorm(x, wn, eps, dt)
+    assert torch.equal(ln.tensor(), h)
+    plain = ops.linear(h, w2t, out_dtype=torch.float32)
+    xd = x.double().cpu()
+    ref = (xd / torch.sqrt((xd ** 2).mean(1, keepdim=True) + eps) * wn.double().cpu()) @ w2.double().t()
+    own = (plain.double().cpu() - ref).abs().max().item()                   # what rounding the normed rows to 16 bits costs
+    assert (fused.double().cpu() - ref).abs().max().item() < 1.5 * own + 1e-6
+    # the gated epilogue, and a weight that is not tiled (the norm is then taken by its kernel)
+    if N2 % 2 == 0:
+        gated = ops.linear(ln, w2t, ops.EPI_SWIGLU, out_dtype=torch.float32)
+        g_ref = torch.nn.functional.silu(ref[:, 0::2]) * ref[:, 1::2]
+        g_own = (ops.linear(h, w2t, ops.EPI_SWIGLU, out_dtype=torch.float32).double().cpu() - g_ref).abs().max().item()
+        assert (gated.double().cpu() - g_ref).abs().max().item() < 1.5 * g_own + 1e-6
+    assert torch.equal(ops.linear(ln, w2.to(DEV)[:64].contiguous(), out_dtype=torch.float32),
+                       ops.linear(h, w2.to(DEV)[:64].contiguous(), out_dtype=torch.float32))
+    # anything else that writes to the rows voids the preparation; so does another norm's weight
+    assert ops.lazy_rmsnorm(x, wn.clone(), eps, dt) is None
+    assert ops.lazy_rmsnorm(x, wn, eps, torch.float32) is None              # a 32-bit norm is never deferred
+    x += 1.0
+    assert ops.lazy_rmsnorm(x, wn, eps, dt) is None
+    ops.linear(a.to(DEV), wot, ops.EPI_ADD, out=x)
+    assert ops.lazy_rmsnorm(x, wn, eps, dt) is not None
+    ops.linear(a.to(DEV), wo.to(DEV), ops.EPI_ADD, out=x)                   # a kernel that prepares nothing
+    assert ops.lazy_rmsnorm(x, wn, eps, dt) is None
+    ops.linear(a.to(DEV), wot, ops.EPI_ADD, out=x)
+    assert ops.lazy_rmsnorm(x.view(M, d), wn, eps, dt) is None              # another tensor object, no record
+    if M < 16:
+        big = torch.zeros(17, d, device=DEV)
+        ops.expect_norm(big, wn)
+        ops.linear(torch.zeros(17, K2, device=DEV, dtype=dt), wot, ops.EPI_ADD, out=big)
+        assert ops.lazy_rmsnorm(big, wn, eps, dt) is None                   # more than 16 rows: the norm kernel
+
+
 def test_gate_activation_alone(ops):
     """act(gate) * up on interleaved columns, for a product that was stored unactivated."""
     g = torch.Generator().manual_seed(3)
