@@ -50,10 +50,42 @@ def main() -> int:
     ap.add_argument("--dtype", default="fp16", choices=["fp16", "bf16"])
     ap.add_argument("--prefill-tokens", type=int, default=2048)
     ap.add_argument("--points", default="1,64", help="further decode batch sizes, comma separated ('' for none)")
+    ap.add_argument("--no-other-shapes", action="store_true",
+                    help="leave out the 1B ragged step and the 7B batch-64 decode that the default run adds to points")
     args = ap.parse_args()
     if args.gpus != 1:
         print(f"bench.py: this library runs on one GPU; --gpus {args.gpus} is not supported")
         return 2
+
+    line = measure(args)
+    if args.shape == "llama-3.1-8b" and not args.no_other_shapes and not args.ragged_prefill:
+        # the other two benchmark shapes, each in an engine of its own, into the same line
+        import copy
+        a1 = copy.copy(args)
+        a1.shape, a1.batch, a1.points, a1.ragged_prefill, a1.context, a1.layers = "llama-3.2-1b", 8, "", 32, 0, 0
+        a1.steps, a1.warmup, a1.prefill_tokens = 8, 2, 0
+        r1 = measure(a1)["ragged_prefill"]
+        a7 = copy.copy(args)
+        a7.shape, a7.batch, a7.points, a7.ragged_prefill, a7.context, a7.layers = "llama-2-7b", 64, "", 0, 0, 0
+        a7.steps, a7.warmup, a7.prefill_tokens = 24, 4, 0
+        r7 = measure(a7)
+        line["points"].update({
+            "ragged_1b_32prompts_ms": r1["ms"], "ragged_1b_32prompts_tokens": r1["tokens"],
+            "ragged_1b_32prompts_frac_of_peak": r1["frac"],
+            "decode_7b_b64_ctx4096_ms": r7["ms_per_step"], "decode_7b_b64_ctx4096_tokens_s": r7["value"],
+            "decode_7b_b64_ctx4096_frac_of_hbm": r7["roofline"]["frac"]})
+        line["config"]["also_in_points"] = ("llama-3.2-1b shape (16 layers, hidden 2048, 32/8 heads of 64, intermediate "
+                                            "8192, tied): one step of 32 prompts of 16..2048 tokens; llama-2-7b shape (32 "
+                                            "layers, hidden 4096, 32/32 heads of 128, intermediate 11008, vocab 32000): "
+                                            "decode batch 64 at context 4096")
+    print(json.dumps(line))
+    return 0
+
+
+def measure(args) -> dict:
+    """One engine of one shape: decode at the given batch sizes, the prefill of one prompt, optionally a
+    ragged step of many prompts; returns the benchmark line."""
+    import gc
 
     import torch
 
@@ -189,8 +221,10 @@ def main() -> int:
     }
     if ragged:
         line["ragged_prefill"] = ragged
-    print(json.dumps(line))
-    return 0
+    del engine, model, cache
+    gc.collect()
+    torch.cuda.empty_cache()
+    return line
 
 
 if __name__ == "__main__":

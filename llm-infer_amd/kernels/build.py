@@ -24,7 +24,9 @@ CSRC = os.path.join(os.path.dirname(os.path.dirname(os.path.abspath(__file__))),
 ARCH = "gfx950"
 CORE_SOURCES = ("elementwise.hip", "gemm.hip", "gemm_prefill.hip", "sampling.hip")
 ATTN_SOURCE = "attention.hip"
-HEADERS = ("common.h", "gemm_common.h", "no_alloc.h")
+# the headers a library's sources include (its stamp covers them)
+HEADERS = {"libli_core.so": ("common.h", "gemm_common.h", "no_alloc.h")}
+DEFAULT_HEADERS = ("common.h",)
 FLAGS = ["--offload-arch=" + ARCH, "-O3", "-std=c++17", "-fPIC",
          "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops", "-Wno-unused-command-line-argument"]
 
@@ -67,9 +69,9 @@ def _hipcc() -> str:
     raise BuildError("hipcc not found: the HIP kernels cannot be built and there is no other implementation")
 
 
-def _stamp(sources, defines) -> str:
+def _stamp(sources, defines, lib_name="") -> str:
     h = hashlib.sha256()
-    for name in tuple(sources) + HEADERS:
+    for name in tuple(sources) + HEADERS.get(lib_name, DEFAULT_HEADERS):
         with open(os.path.join(CSRC, name), "rb") as f:
             h.update(name.encode() + b"\0" + f.read())
     h.update(" ".join(FLAGS + list(defines)).encode())
@@ -95,7 +97,7 @@ def _run(cmd, what):
 
 
 def _build_library(lib_name: str, sources, defines=(), force=False) -> str:
-    stamp = _stamp(sources, defines)
+    stamp = _stamp(sources, defines, lib_name)
     if not force:
         # a library built from these very sources is taken where it lies, also from a folder that
         # cannot be written
