@@ -4,6 +4,7 @@
     new_tokens = engine.generate([[1, 2, 3], [4, 5]], max_new_tokens=16, temperature=0.0)
 """
 from .config import ConfigError, LlamaConfig
+from .tensor import Tensor
 from .registry import (config_from_dict, config_from_folder, register_architecture, register_block,
                        register_embedding, register_feed_forward, register_head, register_mixer,
                        register_norm, register_position)

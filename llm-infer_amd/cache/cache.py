@@ -20,6 +20,7 @@ from dataclasses import dataclass
 import numpy as np
 import torch
 
+from ..tensor import Tensor
 from .slots import CacheError, PagePool, SlotAllocator
 from .specs import KVSpec, StateSpec
 
@@ -66,8 +67,8 @@ class KVGroup:
         self.device, self.dtype = device, dtype
         self._views = {}
         if device is not None:
-            self.storage = torch.zeros((n_pages, self.page_elems), dtype=dtype, device=device)
-            self.page_table = torch.zeros((n_slots, self.max_pages), dtype=torch.int32, device=device)
+            self.storage = Tensor.zeros((n_pages, self.page_elems), dtype, device)
+            self.page_table = Tensor.zeros((n_slots, self.max_pages), torch.int32, device)
         else:
             self.storage = self.page_table = None
 
@@ -144,7 +145,7 @@ class StateGroup:
         dtype = getattr(torch, spec.dtype)
         self.storage = None
         if device is not None:
-            self.storage = torch.zeros((len(self.entries), n_slots) + tuple(spec.shape), dtype=dtype, device=device)
+            self.storage = Tensor.zeros((len(self.entries), n_slots) + tuple(spec.shape), dtype, device)
 
     def view(self, entry: int) -> StateView:
         return StateView(self.storage[self.entries.index(entry)], self.spec)
@@ -188,9 +189,9 @@ class Cache:
             for e in entries:
                 self._group_of[e] = g
         if device is not None:
-            self.lens_dev = torch.zeros((self.n_slots,), dtype=torch.int32, device=device)
+            self.lens_dev = Tensor.zeros((self.n_slots,), torch.int32, device)
             # fixed-size state of every sequence: key and counter of its sampling generator
-            self.seq_state = torch.zeros((self.n_slots, 2), dtype=torch.int64, device=device)
+            self.seq_state = Tensor.zeros((self.n_slots, 2), torch.int64, device)
         else:
             self.lens_dev = self.seq_state = None
 

@@ -12,6 +12,7 @@ from __future__ import annotations
 import torch
 
 from ..kernels import ops
+from ..tensor import Tensor
 from .step import StepShared, decode_splits, split_bucket
 
 
@@ -68,7 +69,7 @@ class GraphDecodeRunner:
             self.bufs["rows"] = torch.arange(n, dtype=torch.int32, device=dev)
             self.bufs["temperature"] = torch.ones((1,), dtype=torch.float32, device=dev)
             # where the tokens of the steps in flight arrive on the host
-            self.bufs["host"] = [torch.zeros((n,), dtype=torch.int32, pin_memory=True) for _ in range(3)]
+            self.bufs["host"] = [Tensor.pinned((n,), torch.int32) for _ in range(3)]
             self.bufs["done"] = [torch.cuda.Event() for _ in range(3)]
             engine._graph_bufs = self.bufs
         self.current = None            # the slots now in the buffers

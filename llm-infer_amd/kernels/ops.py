@@ -11,6 +11,7 @@ from ctypes import c_float, c_int, c_int64, c_uint64, c_void_p
 import torch
 
 from . import build
+from ..tensor import Tensor
 
 PAGE = 64
 DT = {torch.float32: 0, torch.float16: 1, torch.bfloat16: 2}
@@ -160,28 +161,27 @@ class _RopeStore(ctypes.Structure):
                 ("dt", c_int)]
 
 
-class TiledWeight:
-    """A 16-bit matrix [n, k] kept in the order in which the matrix cores take it (csrc/gemm.hip,
-    "Tiled weights"); rows are padded to a multiple of 16.  ``prefix(rows)`` is the matrix of the
-    first rows (a multiple of 16), sharing the storage."""
+def is_tiled(w) -> bool:
+    """True for a ``Tensor`` in tiled layout: a 16-bit matrix [n, k] kept in the order in which the matrix
+    cores take it (csrc/gemm.hip, "Tiled weights"; rows padded to a multiple of 16)."""
+    return getattr(w, "layout", "rows") == "tiled"
 
-    def __init__(self, data: torch.Tensor, n: int, k: int):
-        self.data, self.n, self.k = data, n, k
-        self.dtype, self.device, self.shape = data.dtype, data.device, (n, k)
 
-    def prefix(self, rows: int) -> "TiledWeight":
-        _need(rows % 16 == 0 and 0 < rows <= self.n, "a tiled weight is cut at multiples of 16 rows")
-        return TiledWeight(self.data[: rows * self.k], rows, self.k)
+def matrix_shape(w) -> tuple:
+    """(n, k) of a matrix operand, whatever its layout."""
+    return tuple(w.logical) if is_tiled(w) else tuple(w.shape)
 
 
 def can_tile(w: torch.Tensor) -> bool:
-    return w.dim() == 2 and w.dtype in (torch.float16, torch.bfloat16) and w.shape[1] % 32 == 0 and w.is_cuda
+    return not is_tiled(w) and w.dim() == 2 and w.dtype in (torch.float16, torch.bfloat16) and w.shape[1] % 32 == 0 and w.is_cuda
 
 
 def prepare_weight(w: torch.Tensor):
     """The form in which a linear layer keeps its matrix: tiled where the kernels can use that
     (16-bit, K a multiple of 32), else as it is."""
-    return tile_weight(w) if can_tile(w) else w
+    if can_tile(w):
+        return tile_weight(w)
+    return w if isinstance(w, Tensor) else Tensor.wrap(w)
 
 
 _ws_cache: dict = {}
@@ -206,8 +206,9 @@ def linear(x: torch.Tensor, w, mode: int = EPI_STORE, out: torch.Tensor | None =
            out_dtype=None, force: str | None = None, _rope=None) -> torch.Tensor:
     """C = X W^T with the epilogue ``mode``: store, add into ``out`` (float32), or act(gate) * up over
     interleaved gate/up rows of W (C has N/2 columns; EPI_SWIGLU: silu, EPI_GEGLU: gelu).  ``force`` picks a kernel for tests."""
-    tiled = isinstance(w, TiledWeight)
-    wd = w.data if tiled else w
+    tiled = is_tiled(w)
+    wd = w
+    w_shape = matrix_shape(w)
     _drop_row_stats(out)                   # whatever this call writes into `out`, an older record is void
     lazy = None
     if isinstance(x, LazyNorm):
@@ -218,9 +219,9 @@ def linear(x: torch.Tensor, w, mode: int = EPI_STORE, out: torch.Tensor | None =
         else:
             x = x.tensor()
     _dev(x, wd, out)
-    _need(x.dim() == 2 and len(w.shape) == 2 and x.shape[1] == w.shape[1], f"linear: x {tuple(x.shape)} w {tuple(w.shape)}")
+    _need(x.dim() == 2 and len(w_shape) == 2 and x.shape[1] == w_shape[1], f"linear: x {tuple(x.shape)} w {w_shape}")
     m, k = x.shape
-    n = w.shape[0]
+    n = w_shape[0]
     n_out = n // 2 if mode in GATED else n
     if mode == EPI_ADD:
         _need(out is not None and out.dtype == torch.float32, "add epilogue needs a float32 output")
@@ -480,7 +481,7 @@ def linear_rope_store(x, w, inv_freq, rotary_dim, pos, tok_slot, page_table, pag
     rope_store, without the round trip.  Returns q [T, H, hd]."""
     _dev(inv_freq, pos, tok_slot, page_table, k_pages, v_pages)
     t = x.shape[0]
-    _need(w.shape[0] == (n_heads + 2 * n_kv_heads) * head_dim, "linear_rope_store: rows of W are not (H + 2K) hd")
+    _need(matrix_shape(w)[0] == (n_heads + 2 * n_kv_heads) * head_dim, "linear_rope_store: rows of W are not (H + 2K) hd")
     _need(head_dim % 16 == 0, "head size must be a multiple of 16")
     _need(pos.dtype == torch.int32 and pos.numel() >= t, "pos: int32 [T]")
     if rotary_dim > 0:
@@ -668,21 +669,32 @@ def uniform01(key: int, counter: int) -> float:
     return float(core().li_uniform01(c_uint64(key & (2 ** 64 - 1)), c_uint64(counter & (2 ** 64 - 1))))
 
 
-def tile_weight(w: torch.Tensor) -> TiledWeight:
-    """A 16-bit matrix [N, K] (K a multiple of 32) in tiled order."""
+def tile_weight(w: torch.Tensor) -> Tensor:
+    """A 16-bit matrix [N, K] (K a multiple of 32) as a device-owned ``Tensor`` in tiled layout."""
     _dev(w)
     _need(can_tile(w), "tile_weight: 16-bit [N, K] on the GPU with K a multiple of 32")
     n, k = w.shape
     out = torch.empty(((n + 15) // 16 * 16 * k,), dtype=w.dtype, device=w.device)
     _check(core().li_tile_weight(_ptr(w), _ptr(out), DT[w.dtype], n, k, _stream()), "tile_weight")
-    return TiledWeight(out, n, k)
+    return Tensor.wrap(out, "tiled", (n, k))
 
 
-def gemv_tiled(x, w: TiledWeight, mode=EPI_STORE, out_dtype=None, nt=0, kw=0):
+def untile(w: Tensor) -> torch.Tensor:
+    """The matrix [N, K] that a tiled ``Tensor`` holds, in rows (for inspection and tests; on the device)."""
+    _need(is_tiled(w), "untile: a tiled Tensor")
+    n, k = w.logical
+    flat = w.as_subclass(torch.Tensor)
+    # [n/16][k/32][lane = 16 * ((k % 32) / 8) + n % 16][k % 8]  ->  [n][k]
+    t = flat.view((n + 15) // 16, k // 32, 4, 16, 8).permute(0, 3, 1, 2, 4).reshape(-1, k)
+    return t[:n].contiguous()
+
+
+def gemv_tiled(x, w: Tensor, mode=EPI_STORE, out_dtype=None, nt=0, kw=0):
     """gemv_tiled with a chosen shape of workgroup (for tuning and tests)."""
     m, k = x.shape
-    n_out = w.n // 2 if mode in GATED else w.n
+    n = w.logical[0]
+    n_out = n // 2 if mode in GATED else n
     out = torch.empty((m, n_out), dtype=out_dtype or x.dtype, device=x.device)
-    _check(core().li_gemv_tiled(_ptr(x), _ptr(w.data), DT[x.dtype], _ptr(out), DT[out.dtype], mode, m, w.n, k,
+    _check(core().li_gemv_tiled(_ptr(x), _ptr(w), DT[x.dtype], _ptr(out), DT[out.dtype], mode, m, n, k,
                                 nt, kw, None, None, None, _stream()), "gemv_tiled")
     return out

@@ -59,7 +59,7 @@ class Attention(Part):
         wqkv = torch.cat([self._pad_rows(tensors["q_proj.weight"], H), self._pad_rows(tensors["k_proj.weight"], K),
                           self._pad_rows(tensors["v_proj.weight"], K)], 0)
         self.wqkv = ops.prepare_weight(wqkv)
-        self.wq = self.wqkv.prefix(H * pad) if isinstance(self.wqkv, ops.TiledWeight) else self.wqkv[:H * pad]
+        self.wq = self.wqkv.prefix(H * pad) if ops.is_tiled(self.wqkv) else self.wqkv[:H * pad]
         wo = tensors["o_proj.weight"]
         if pad != hd:                               # zero columns after each head's own
             full = torch.zeros((wo.shape[0], H, pad), dtype=wo.dtype, device=wo.device)

@@ -22,6 +22,8 @@ import struct
 import numpy as np
 import torch
 
+from ..tensor import Tensor
+
 MAGIC = b"GGUF"
 _SCALARS = {0: "<B", 1: "<b", 2: "<H", 3: "<h", 4: "<I", 5: "<i", 6: "<f", 7: "<?", 10: "<Q", 11: "<q", 12: "<d"}
 T_STRING, T_ARRAY = 8, 9
@@ -129,7 +131,7 @@ class GGUFFile:
                             "are read (quantized weights are not supported)")
         return _TENSOR_TYPES[ttype][0], shape
 
-    def tensor(self, name: str) -> torch.Tensor:
+    def tensor(self, name: str) -> Tensor:
         dtype, shape = self.info(name)
         _, _, offset = self._info[name]
         count = 1
@@ -137,7 +139,7 @@ class GGUFFile:
             count *= s
         raw = np.frombuffer(self._map, dtype=np.uint8, count=count * _TENSOR_TYPES[self._info[name][0]][1],
                             offset=self._data_start + offset)
-        return torch.from_numpy(raw).view(dtype).reshape(shape)
+        return Tensor.borrow(torch.from_numpy(raw).view(dtype).reshape(shape), keeps=self._map)
 
 
 # ---------------------------------------------------------------------------

@@ -18,6 +18,7 @@ from dataclasses import dataclass
 
 import torch
 
+from ..tensor import Tensor
 from .safetensors_io import SafetensorsFile
 
 
@@ -137,9 +138,12 @@ def kept_dtype(stored: torch.dtype, kind: str, compute: torch.dtype) -> torch.dt
     return compute
 
 
-def place_tensor(t: torch.Tensor, kind: str, compute: torch.dtype, device) -> torch.Tensor:
-    """Move one tensor to the device in the dtype the engine keeps it in."""
-    return t.to(device=device, dtype=kept_dtype(t.dtype, kind, compute)).contiguous()
+def place_tensor(t: torch.Tensor, kind: str, compute: torch.dtype, device) -> Tensor:
+    """One tensor as the engine keeps it: a device-owned copy in its kept dtype (a borrowed view of a file's
+    mapping is read once on the way)."""
+    if not isinstance(t, Tensor):
+        t = Tensor.wrap(t)
+    return t.on_device(device, kept_dtype(t.dtype, kind, compute))
 
 
 _DTYPE_NAMES = {"float32": torch.float32, "float16": torch.float16, "bfloat16": torch.bfloat16}

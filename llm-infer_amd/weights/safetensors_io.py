@@ -16,6 +16,8 @@ import struct
 
 import torch
 
+from ..tensor import Tensor
+
 MAX_HEADER = 100_000_000            # src/safetensors.cpp:11
 
 _DTYPES = {
@@ -94,15 +96,16 @@ class SafetensorsFile:
         dtype, shape, _, _ = self._info[name]
         return dtype, shape
 
-    def tensor(self, name: str) -> torch.Tensor:
+    def tensor(self, name: str) -> Tensor:
+        """The tensor as a view into the file's mapping (owner "borrowed": nothing is copied)."""
         if name not in self._info:
             raise SafetensorsError(f"{self.path}: Tensor not found: {name}")
         dtype, shape, lo, hi = self._info[name]
         count = (hi - lo) // _itemsize(dtype)
         if count == 0:
-            return torch.empty(shape, dtype=dtype)
+            return Tensor.wrap(torch.empty(shape, dtype=dtype))
         flat = torch.frombuffer(self._map, dtype=dtype, count=count, offset=self._data_start + lo)
-        return flat.view(shape)
+        return Tensor.borrow(flat.view(shape), keeps=self._map)
 
 
 def write_safetensors(path: str, tensors: dict, metadata: dict | None = None) -> None:

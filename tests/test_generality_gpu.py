@@ -687,8 +687,8 @@ def test_toy_architecture_with_a_window_group(lib, dtype):
 
     def rows(w):                                     # a weight back in plain row order, whatever its layout
         from llm_infer_amd.kernels import ops
-        if isinstance(w, ops.TiledWeight):
-            eye = torch.eye(w.k, dtype=w.dtype, device=DEV)
+        if ops.is_tiled(w):
+            eye = torch.eye(w.logical[1], dtype=w.dtype, device=DEV)
             return ops.linear(eye, w, out_dtype=torch.float32).t().double().cpu()
         return w.double().cpu()
 

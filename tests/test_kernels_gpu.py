@@ -120,7 +120,8 @@ def test_linear_tiled_weights(ops, M, N, K, dt):
     w = (torch.randn(N, K, generator=g) / math.sqrt(K)).to(dt).to(DEV)
     res = torch.randn(M, N, generator=g).to(DEV)
     wt = ops.tile_weight(w)
-    assert wt.shape == (N, K) and wt.data.numel() == (N + 15) // 16 * 16 * K
+    assert ops.is_tiled(wt) and wt.logical == (N, K) and wt.numel() == (N + 15) // 16 * 16 * K and wt.owner == "device"
+    assert torch.equal(ops.untile(wt), w.to(DEV))
     kinds = [None, "mfma:0:1", "mfma:1:2", "mfma:2:1", "big:0", "big:1", "big:0:2", "big:1:5"] + (["gemv_mfma"] if M <= 16 else [])
     kinds += ["dma", "dma:0", "dma:1", "dma:2", "dma:0:2", "dma:1:5", "dma:2:3"]
     # the first columns with one tile, the rest with another (the first count a multiple of the first tile)
