@@ -317,15 +317,21 @@ __global__ __launch_bounds__(256, HD <= 128 ? 2 : 1) void attn_prefill_kernel(
 // ---------------------------------------------------------------------------
 // decode: one new token per sequence, q [B, H, HD]
 // ---------------------------------------------------------------------------
-template <class T>
-__global__ __launch_bounds__(64) void attn_decode_kernel(
+// A workgroup is W waves that take W consecutive splits of one (sequence, KV head) and merge their
+// states through LDS, in wave order; the grid's z extent times W is the number of splits.  With all
+// splits inside one workgroup the result is written as it is and no merge kernel runs.
+template <class T, int W>
+__global__ __launch_bounds__(64 * W) void attn_decode_kernel(
     const T* __restrict__ q, T* __restrict__ out, float* __restrict__ part_o, float* __restrict__ part_ml,
     CachePtrs c, const int* __restrict__ seq_slot, const int* __restrict__ seq_ctx, int H, int K, float scale,
     int window) {
-    const int lane = threadIdx.x & 63;
+    constexpr int OLD = 33;                                   // floats from one output dim to the next in LDS
+    extern __shared__ __attribute__((aligned(16))) unsigned char smem_raw[];
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int b = blockIdx.x, G = H / K, gchunks = (G + 31) / 32;
     const int kvh = blockIdx.y / gchunks, gc = blockIdx.y % gchunks;
-    const int S = gridDim.z, split = blockIdx.z;
+    const int S = gridDim.z * W, split = blockIdx.z * W + wave;
+    const int grid_splits = gridDim.z, grid_split = blockIdx.z;
     const int hg = gc * 32 + (lane & 31);
     const bool live = hg < G;
     const int h = kvh * G + hg;
@@ -352,9 +358,53 @@ __global__ __launch_bounds__(64) void attn_decode_kernel(
         if (p + 1 < p1) a.load_k(kbase + (int64_t)table[p + 1] * c.page_stride, kf);
         a.mix(vf, s);
     }
-    const float total = a.total();
+    float total = a.total();
+    if (W > 1) {
+        // waves 1..W-1 lay their states down as [wave - 1][dim][row] (+ m and l per row); wave 0 adds them
+        // to its own in wave order:  M = max m,  o = sum o_w 2^(m_w - M),  l = sum l_w 2^(m_w - M)
+        float* sm = (float*)smem_raw;
+        constexpr int PER = HD * OLD + 64;
+        const int row = lane & 31;
+        if (wave > 0) {
+            float* mine = sm + (wave - 1) * PER;
+#pragma unroll
+            for (int blk = 0; blk < DB; ++blk)
+#pragma unroll
+                for (int r = 0; r < 16; ++r) {
+                    const int d = 32 * blk + 8 * (r >> 2) + 4 * (lane >> 5) + (r & 3);
+                    if (d < HD) mine[d * OLD + row] = a.o[blk][r];
+                }
+            if (lane < 32) { mine[HD * OLD + row] = a.m; mine[HD * OLD + 32 + row] = total; }
+        }
+        __syncthreads();
+        if (wave > 0) return;
+        float M = a.m;
+#pragma unroll
+        for (int w = 1; w < W; ++w) M = fmaxf(M, sm[(w - 1) * PER + HD * OLD + row]);
+        const float f0 = (a.m == -INFINITY) ? 0.f : exp2f(a.m - M);
+#pragma unroll
+        for (int blk = 0; blk < DB; ++blk)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) a.o[blk][r] *= f0;
+        total *= f0;
+#pragma unroll
+        for (int w = 1; w < W; ++w) {
+            const float* theirs = sm + (w - 1) * PER;
+            const float mw = theirs[HD * OLD + row];
+            const float fw = (mw == -INFINITY) ? 0.f : exp2f(mw - M);
+            total += theirs[HD * OLD + 32 + row] * fw;
+#pragma unroll
+            for (int blk = 0; blk < DB; ++blk)
+#pragma unroll
+                for (int r = 0; r < 16; ++r) {
+                    const int d = 32 * blk + 8 * (r >> 2) + 4 * (lane >> 5) + (r & 3);
+                    if (d < HD) a.o[blk][r] += theirs[d * OLD + row] * fw;
+                }
+        }
+        a.m = M;
+    }
     if (!live) return;
-    if (S == 1) {
+    if (grid_splits == 1) {
         const float inv = 1.f / total;
         T* orow = out + ((int64_t)b * H + h) * HD;
 #pragma unroll
@@ -369,7 +419,7 @@ __global__ __launch_bounds__(64) void attn_decode_kernel(
             }
         return;
     }
-    const int64_t slot = ((int64_t)b * H + h) * S + split;
+    const int64_t slot = ((int64_t)b * H + h) * grid_splits + grid_split;
     float* po = part_o + slot * HD;
 #pragma unroll
     for (int blk = 0; blk < DB; ++blk)
@@ -494,29 +544,51 @@ extern "C" int li_attn_prefill(const void* q, void* out, int dt, const void* k, 
     return LI_OK;
 }
 
-// part_o: [B, H, splits, HD] float32, part_ml: [B, H, splits, 2] float32 (needed when splits > 1)
+// How the splits of the context are dealt: waves of a workgroup (merged inside) times workgroups (merged by
+// the merge kernel).  li_attn_decode_parts(splits) is the number of partial states per
+// (sequence, head) that the caller's workspace must hold: part_o [B, H, parts, HD], part_ml [B, H, parts, 2]
+// float32 (needed when parts > 1).
+// (measured on MI355X: workgroups of several waves pay where they save the merge kernel altogether, that
+// is for two and four splits; with more splits, one wave a workgroup and one merge over all of them is faster)
+static int waves_per_group(int splits) { return (splits == 2 || splits == 4) ? splits : 1; }
+extern "C" int li_attn_decode_parts(int splits) { return splits < 1 ? 0 : splits / waves_per_group(splits); }
+
+template <class T, int W>
+static int launch_decode(const void* q, void* out, float* part_o, float* part_ml, CachePtrs c, const int* seq_slot,
+                         const int* seq_ctx, int n_seqs, int H, int K, float scale, int window, int parts,
+                         hipStream_t stream) {
+    const int G = H / K;
+    dim3 grid(n_seqs, K * ((G + 31) / 32), parts), block(64 * W);
+    const size_t lds = W > 1 ? (size_t)(W - 1) * (HD * 33 + 64) * sizeof(float) : 0;
+    auto kfn = attn_decode_kernel<T, W>;
+    if (lds > 48 * 1024 &&
+        hipFuncSetAttribute((const void*)kfn, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds) != hipSuccess)
+        return LI_HIP_ERROR;
+    kfn<<<grid, block, lds, stream>>>((const T*)q, (T*)out, part_o, part_ml, c, seq_slot, seq_ctx, H, K, scale, window);
+    LI_CHECK_LAUNCH();
+    if (parts > 1) {
+        attn_merge_kernel<T><<<n_seqs * H, 128, 0, stream>>>(part_o, part_ml, (T*)out, parts);
+        LI_CHECK_LAUNCH();
+    }
+    return LI_OK;
+}
+
 extern "C" int li_attn_decode(const void* q, void* out, int dt, const void* k, const void* v, int64_t page_stride,
                               const int* page_table, int max_pages, const int* seq_slot, const int* seq_ctx,
                               int n_seqs, int H, int K, float scale, int window, int splits, float* part_o,
                               float* part_ml, hipStream_t stream) {
-    if (check_heads(H, K) || splits < 1 || splits > 64 || (splits > 1 && (!part_o || !part_ml))) return LI_BAD_ARG;
+    if (check_heads(H, K) || splits < 1 || splits > 64) return LI_BAD_ARG;
+    const int w = waves_per_group(splits), parts = splits / w;
+    if (parts > 64 || (parts > 1 && (!part_o || !part_ml))) return LI_BAD_ARG;
+    if (dt != DT_F16 && dt != DT_BF16) return LI_BAD_ARG;
     if (n_seqs <= 0) return LI_OK;
     CachePtrs c{k, v, page_stride, page_table, max_pages};
-    const int G = H / K;
-    dim3 grid(n_seqs, K * ((G + 31) / 32), splits), block(64);
-    if (dt == DT_F16) {
-        attn_decode_kernel<f16><<<grid, block, 0, stream>>>((const f16*)q, (f16*)out, part_o, part_ml, c, seq_slot,
-                                                            seq_ctx, H, K, scale, window);
-        LI_CHECK_LAUNCH();
-        if (splits > 1) attn_merge_kernel<f16><<<n_seqs * H, 128, 0, stream>>>(part_o, part_ml, (f16*)out, splits);
-    } else if (dt == DT_BF16) {
-        attn_decode_kernel<bf16><<<grid, block, 0, stream>>>((const bf16*)q, (bf16*)out, part_o, part_ml, c,
-                                                             seq_slot, seq_ctx, H, K, scale, window);
-        LI_CHECK_LAUNCH();
-        if (splits > 1) attn_merge_kernel<bf16><<<n_seqs * H, 128, 0, stream>>>(part_o, part_ml, (bf16*)out, splits);
-    } else return LI_BAD_ARG;
-    LI_CHECK_LAUNCH();
-    return LI_OK;
+#define GO(T)                                                                                                      \
+    (w == 4 ? launch_decode<T, 4>(q, out, part_o, part_ml, c, seq_slot, seq_ctx, n_seqs, H, K, scale, window, parts, stream) \
+     : w == 2 ? launch_decode<T, 2>(q, out, part_o, part_ml, c, seq_slot, seq_ctx, n_seqs, H, K, scale, window, parts, stream) \
+              : launch_decode<T, 1>(q, out, part_o, part_ml, c, seq_slot, seq_ctx, n_seqs, H, K, scale, window, parts, stream))
+    return dt == DT_F16 ? GO(f16) : GO(bf16);
+#undef GO
 }
 
 extern "C" int li_attn_f32(const float* q, float* out, const void* k, const void* v, int64_t page_stride,

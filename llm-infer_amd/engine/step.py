@@ -76,8 +76,8 @@ def decode_splits(n_seqs: int, n_kv_heads: int, n_heads: int, bucket: int) -> in
     """Splits of the context for a decode attention of ``n_seqs`` sequences (a power of two, at most
     ``bucket``), so that the chip is filled."""
     waves = n_seqs * n_kv_heads * ((n_heads // n_kv_heads + 31) // 32)
-    # measured on MI355X: 1,024 waves fill the chip best, but from 512 waves on one pass without the
-    # merge kernel is faster than two halves with it
-    want = 1 if waves >= 512 else max(1, 1024 // max(1, waves))
+    # measured on MI355X: 1,024 waves (one a SIMD) fill the chip best; two or four splits are merged inside
+    # a workgroup and cost no second kernel
+    want = max(1, 1024 // max(1, waves))
     s = max(1, min(want, bucket))
     return 1 << (s.bit_length() - 1)

@@ -582,10 +582,14 @@ def attention_decode(q, kv, seq_slot, seq_ctx, n_seqs, n_heads, n_kv_heads, head
     _need(seq_slot.numel() >= n_seqs and seq_ctx.numel() >= n_seqs, "per-sequence arrays too short")
     out = torch.empty_like(q)
     part_o = part_ml = None
-    if splits > 1:
-        part_o = torch.empty((n_seqs, n_heads, splits, head_dim), dtype=torch.float32, device=q.device)
-        part_ml = torch.empty((n_seqs, n_heads, splits, 2), dtype=torch.float32, device=q.device)
-    _check(_attn_lib(head_dim).li_attn_decode(
+    lib = _attn_lib(head_dim)
+    # two or four splits are merged inside a workgroup; more are merged by a second kernel
+    parts = lib.li_attn_decode_parts(splits)
+    _need(1 <= parts <= 64, f"attention_decode: {splits} splits")
+    if parts > 1:
+        part_o = torch.empty((n_seqs, n_heads, parts, head_dim), dtype=torch.float32, device=q.device)
+        part_ml = torch.empty((n_seqs, n_heads, parts, 2), dtype=torch.float32, device=q.device)
+    _check(lib.li_attn_decode(
         _ptr(q), _ptr(out), DT[q.dtype], _ptr(k_pages), _ptr(v_pages), c_int64(page_stride), _ptr(page_table),
         page_table.shape[1], _ptr(seq_slot), _ptr(seq_ctx), n_seqs, n_heads, n_kv_heads, c_float(scale),
         int(window or 0), splits, _ptr(part_o), _ptr(part_ml), _stream()), "attn_decode")

@@ -195,7 +195,7 @@ def test_decode_splits_fill_the_chip_and_are_powers_of_two():
         return decode_splits(n, k, h, split_bucket(ctx))
     assert splits(1, 8, 32, 8192) == 64
     assert splits(8, 8, 32, 8192) == 16
-    assert splits(64, 8, 32, 8192) == 1 and splits(32, 8, 32, 8192) == 4
+    assert splits(64, 8, 32, 8192) == 2 and splits(32, 8, 32, 8192) == 4 and splits(128, 8, 32, 8192) == 1
     assert splits(64, 32, 32, 4096) == 1
     assert splits(1, 8, 32, 100) == 1 and splits(1, 1, 64, 640) == 4
     # the bucket is all that the count knows of the lengths: at least two pages a split, at most 64 splits

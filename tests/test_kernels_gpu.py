@@ -346,7 +346,7 @@ def test_attention_whole_prompts_and_decode(ops, H, K, hd, lens, dt):
         out = ops.attention_f32(q_last, view.as_tuple(), pos, seq_slot, H, K, hd, scale, None)
         assert (out.double().cpu() - ref_last).abs().max().item() < tol
     else:
-        for splits in (1, 2, 3, 8):
+        for splits in (1, 2, 3, 4, 8, 16, 24):               # merged inside a workgroup, by the merge kernel, or both
             out = ops.attention_decode(q_last, view.as_tuple(), seq_slot, seq_ctx, len(lens), H, K, hd, scale,
                                        None, splits)
             err = (out.double().cpu() - ref_last).abs().max().item()
