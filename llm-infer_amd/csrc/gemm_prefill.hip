@@ -2,6 +2,13 @@
 // a row-major one).  Epilogues, layouts and the split-K reduction are in gemm_common.h.
 #include "gemm_common.h"
 
+__device__ __forceinline__ f32x4 mfma16(f16x8 a, f16x8 b, f32x4 c) {
+    return __builtin_amdgcn_mfma_f32_16x16x32_f16(a, b, c, 0, 0, 0);
+}
+__device__ __forceinline__ f32x4 mfma16(bf16x8 a, bf16x8 b, f32x4 c) {
+    return __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b, c, 0, 0, 0);
+}
+
 // Which tile a workgroup works on.  Workgroups go to the 8 XCDs in turn (workgroup L to XCD
 // L % 8) and every XCD has an L2 of its own, so the tiles are numbered such that an XCD works on
 // one contiguous run of them; within the run, groups of GM tiles of X go through all tiles of W
@@ -376,6 +383,161 @@ __global__ __launch_bounds__(64 * WAVES) void gemm_dma_kernel(const T* __restric
 }
 
 // ===========================================================================
+// gemm_wreg: the prefill product against a tiled W with W never in LDS.  A tiled weight lies in memory
+// in the order in which the 16x16x32 matrix instruction takes operand A, so a wave loads its fragments of
+// W straight from global memory into registers (1 KiB contiguous a load) and only X goes through LDS
+// (global_load_lds into 1 KiB units of 16 rows x 32 of K, which are operand B as they lie).  Four waves,
+// each with 16 NI rows of W and all 128 rows of X of the tile (64 NI x 128); two workgroups (three of
+// the narrowest tile) share a CU, and one's waits are the other's matrix time.  Per 32 of K a wave
+// issues NI loads of W, 8 LDS reads and 8 NI matrix instructions.  Three stages: the loads of step s + 2
+// (X into LDS, W into a ring of registers) are issued when step s begins; one barrier a step.  The
+// narrower tiles are for products whose number of tiles would otherwise leave a large part of the last
+// round of workgroups empty.
+// ===========================================================================
+template <class T, int NI>
+__global__ __launch_bounds__(256) void gemm_wreg_kernel(const T* __restrict__ X, const T* __restrict__ Wt,
+                                                        int K, int k_per_split, float* __restrict__ ws,
+                                                        int n_begin, Epilogue e) {
+    typedef typename Vec<T>::v8 v8;
+    constexpr int BN = 64 * NI, BM = 128, BK = 32, STAGES = 3;
+    constexpr int MJ = 8;                               // fragments of X per wave and step
+    constexpr int XU = BM / 16, PER_WAVE = XU / 4;      // units of X per stage, and per wave
+    constexpr int STAGE = XU * 1024;
+    extern __shared__ __attribute__((aligned(16))) unsigned char smem_raw[];
+
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int wn = wave;
+    int bx, by, bz;
+    tile_of_workgroup(8, bx, by, bz);
+    const int m0 = bx * BM, n0 = n_begin + by * BN;
+    const int kb = bz * k_per_split, ke = min(K, kb + k_per_split);
+    const int n_steps = (ke - kb) / BK;
+    const int w_blocks = (e.N + 15) >> 4, steps = K >> 5;
+
+    // this wave's rows of W: NI blocks of 16, each a run of 1 KiB units along K
+    const T* wsrc[NI];
+#pragma unroll
+    for (int i = 0; i < NI; ++i) {
+        const int blk = min(n0 / 16 + wn * NI + i, w_blocks - 1);
+        wsrc[i] = Wt + (((int64_t)blk * steps + (kb >> 5)) * 64 + lane) * 8;
+    }
+    // this wave's share of a stage of X: unit u holds rows m0 + 16 u ..; a lane brings 16 bytes of row
+    // lane % 16 at k + 8 (lane / 16)
+    const unsigned char* xbase = (const unsigned char*)(X + kb);
+    uint32_t xoff[PER_WAVE];
+#pragma unroll
+    for (int i = 0; i < PER_WAVE; ++i) {
+        const int u = wave * PER_WAVE + i;
+        const int row = min(m0 + 16 * u + (lane & 15), e.M - 1);
+        xoff[i] = ((uint32_t)row * (uint32_t)K + 8 * (lane >> 4)) * 2;
+    }
+    auto fill = [&](int s, int buf) {
+#pragma unroll
+        for (int i = 0; i < PER_WAVE; ++i) {
+            const int u = wave * PER_WAVE + i;
+            __builtin_amdgcn_global_load_lds(
+                (const __attribute__((address_space(1))) void*)(xbase + (int64_t)s * (BK * 2) + xoff[i]),
+                (__attribute__((address_space(3))) void*)(smem_raw + buf * STAGE + u * 1024), 16, 0, 0);
+        }
+    };
+    // The loads of W are written as instructions so that the compiler does not place waits for them (at
+    // the loop's head it would wait for every load in flight); the waits are placed by hand below.
+    auto fetch_w = [&](int s, v8 (&a)[NI]) {
+#pragma unroll
+        for (int i = 0; i < NI; ++i)
+            asm volatile("global_load_dwordx4 %0, %1, off" : "=v"(a[i]) : "v"(wsrc[i] + (int64_t)s * 512) : "memory");
+    };
+
+    f32x4 acc[NI][MJ];
+#pragma unroll
+    for (int i = 0; i < NI; ++i)
+#pragma unroll
+        for (int j = 0; j < MJ; ++j) acc[i][j] = f32x4{0.f, 0.f, 0.f, 0.f};
+
+    const unsigned char* sB = smem_raw + lane * 16;
+    auto compute = [&](int buf, const v8 (&a)[NI]) {
+        v8 b[MJ];
+        const unsigned char* src = sB + buf * STAGE;
+#pragma unroll
+        for (int j = 0; j < MJ; ++j) b[j] = *(const v8*)(src + j * 1024);
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int j = 0; j < MJ; ++j)
+#pragma unroll
+            for (int i = 0; i < NI; ++i) acc[i][j] = mfma16(a[i], b[j], acc[i][j]);
+        __builtin_amdgcn_sched_barrier(0);
+    };
+
+    // Loads past the last step are not branched around: they fetch the last step again (into a buffer
+    // and registers that nothing reads), which keeps the count of loads in flight fixed.
+    // (The host gives every split of K at least one step.  Without this line the compiler builds a path
+    // for no steps on which the ring's registers are written while the first loads are in flight.)
+    if (n_steps <= 0) return;
+    const int last = n_steps - 1;
+    v8 a0[NI], a1[NI], a2[NI];
+    fill(0, 0);
+    fetch_w(0, a0);
+    fill(min(1, last), 1);
+    fetch_w(min(1, last), a1);
+    // one step of the loop: the loads of step s are complete when at most those of step s + 1 are in flight
+    // (PER_WAVE + NI a step, in order); the barrier then publishes everybody's share of stage s and says that
+    // everybody has read stage s - 1, whose buffer the loads of step s + 2 may fill
+#define WREG_STEP(S, BUF, ACUR, ANEW)                                              \
+    {                                                                              \
+        __builtin_amdgcn_s_waitcnt(0x0F70 | (PER_WAVE + NI));                       \
+        __builtin_amdgcn_s_barrier();                                              \
+        fill(min((S) + 2, last), ((BUF) + 2) % 3);                                 \
+        fetch_w(min((S) + 2, last), ANEW);                                         \
+        __builtin_amdgcn_sched_barrier(0);                                         \
+        compute(BUF, ACUR);                                                        \
+        __builtin_amdgcn_sched_barrier(0);                                         \
+    }
+    for (int s = 0; s < n_steps; s += 3) {
+        WREG_STEP(s, 0, a0, a2)
+        if (s + 1 < n_steps) WREG_STEP(s + 1, 1, a1, a0)
+        if (s + 2 < n_steps) WREG_STEP(s + 2, 2, a2, a1)
+    }
+#undef WREG_STEP
+    // Loads into the ring may still be in flight here (those past the last step).  The compiler does not
+    // know of them: without a use of the ring after the wait it would hand the ring's registers to the
+    // epilogue's values before the wait, and a load that lands late would overwrite an address.
+    __builtin_amdgcn_s_waitcnt(0x0070);
+#pragma unroll
+    for (int i = 0; i < NI; ++i) asm volatile("" ::"v"(a0[i]), "v"(a1[i]), "v"(a2[i]));
+    __builtin_amdgcn_sched_barrier(0);
+    __syncthreads();
+
+    // Epilogue through LDS, a strip of 16 rows of X x 16 NI rows of W at a time: accumulator q of a 16x16
+    // block is W row 4 (lane / 16) + q, X row lane % 16; read back, consecutive lanes hold consecutive
+    // quads of columns of one row.  The loop over the strip's quads is not unrolled (one copy of the
+    // epilogue in the code).
+    constexpr int SLD = 16 * NI + 4, QUADS = 4 * NI;
+    float* stage = (float*)smem_raw + wave * (16 * SLD);
+    const int r = lane & 15, g = lane >> 4;
+#pragma unroll
+    for (int j = 0; j < MJ; ++j) {
+#pragma unroll
+        for (int i = 0; i < NI; ++i) *(f32x4*)(stage + r * SLD + 16 * i + 4 * g) = acc[i][j];
+        __builtin_amdgcn_wave_barrier();
+        const int mb = m0 + 16 * j, nb = n0 + wn * (16 * NI);
+#pragma unroll 1
+        for (int q = lane; q < 16 * QUADS; q += 64) {
+            const int rr = q / QUADS, c = (q % QUADS) * 4;
+            const f32x4 v = *(const f32x4*)(stage + rr * SLD + c);
+            const float vv[4] = {v[0], v[1], v[2], v[3]};
+            if (gridDim.z == 1) epilogue4(e, mb + rr, nb + c, vv);
+            else if (mb + rr < e.M) {
+                float* p = ws + ((int64_t)bz * e.M + mb + rr) * e.N + nb + c;
+#pragma unroll
+                for (int jj = 0; jj < 4; ++jj) if (nb + c + jj < e.N) p[jj] = vv[jj];
+            }
+        }
+        __builtin_amdgcn_wave_barrier();
+    }
+}
+
+// ===========================================================================
 // C interface
 // ===========================================================================
 // tile (rows of W x rows of X / depth): 0 = 128x128/64, 1 = 256x128/32
@@ -434,12 +596,14 @@ extern "C" int li_gemm_dma(const void* X, const void* Wt, int dt, void* C, int o
     if (rc) return rc;
     if (dt != DT_F16 && dt != DT_BF16) return LI_BAD_ARG;
     if (K % 32 != 0 || ((uintptr_t)X & 15) || ((uintptr_t)Wt & 15)) return LI_UNSUPPORTED;
-    if (tile < 0 || tile > 2) return LI_BAD_ARG;
+    if (tile < 0 || tile > 5) return LI_BAD_ARG;
     if ((int64_t)M * K * 2 >= ((int64_t)1 << 32)) return LI_UNSUPPORTED;     // 32-bit offsets into X
     if (splits < 1 || (splits > 1 && !ws)) return LI_BAD_ARG;
     if (n_begin < 0 || n_begin >= N || (n_begin & 15) || n_count < 0 || n_begin + n_count > N) return LI_BAD_ARG;
     if (n_count == 0) n_count = N - n_begin;
-    const int bn = tile ? 256 : 128, bm = tile == 2 ? 256 : 128, bk = 32;
+    // tiles 0 to 2: gemm_dma; 3 to 5: gemm_wreg
+    static const int tile_bn[6] = {128, 256, 256, 256, 192, 128}, tile_bm[6] = {128, 128, 256, 128, 128, 128};
+    const int bn = tile_bn[tile], bm = tile_bm[tile], bk = 32;
     if (n_begin + n_count < N && n_count % bn != 0) return LI_BAD_ARG;       // only the last columns may end inside a tile
     if (splits > 1 && n_count != N) return LI_BAD_ARG;
     if (M == 0) return LI_OK;
@@ -449,7 +613,29 @@ extern "C" int li_gemm_dma(const void* X, const void* Wt, int dt, void* C, int o
     const size_t lds = (size_t)3 * (bn + bm) / 16 * 1024;
     int k_per_split = ((K + splits - 1) / splits + bk - 1) / bk * bk;
     splits = (K + k_per_split - 1) / k_per_split;
-    dim3 grid((M + bm - 1) / bm, (n_count + bn - 1) / bn, splits), block(tile == 2 ? 512 : 256);
+    dim3 grid((M + bm - 1) / bm, (n_count + bn - 1) / bn, splits), block(bm == 256 ? 512 : 256);
+    if (tile >= 3) {
+        // three stages of X; the epilogue stages 16 x (bn / 4 + 4) floats a wave in the same LDS
+        const size_t stages = (size_t)3 * (bm / 16) * 1024, strips = (size_t)4 * 16 * (bn / 4 + 4) * 4;
+        const size_t wlds = stages > strips ? stages : strips;
+#define WGO(T, NI) gemm_wreg_kernel<T, NI><<<grid, block, wlds, stream>>>((const T*)X, (const T*)Wt, K, k_per_split, ws, n_begin, e)
+#define WLAUNCH(T)                           \
+    do {                                     \
+        if (tile == 3) WGO(T, 4);            \
+        else if (tile == 4) WGO(T, 3);       \
+        else WGO(T, 2);                      \
+    } while (0)
+        if (dt == DT_F16) WLAUNCH(f16); else WLAUNCH(bf16);
+#undef WLAUNCH
+#undef WGO
+        LI_CHECK_LAUNCH();
+        if (splits > 1) {
+            const int64_t quads = (int64_t)M * ((N + 3) / 4);
+            splitk_reduce_kernel<<<(unsigned)((quads + 255) / 256), 256, 0, stream>>>(ws, splits, e);
+            LI_CHECK_LAUNCH();
+        }
+        return LI_OK;
+    }
 #define GO(T, BN, BM, WV, ST)                                                                                \
     do {                                                                                               \
         auto kfn = gemm_dma_kernel<T, BN, BM, WV, ST>;                                                 \

@@ -370,9 +370,13 @@ def _stream_shape(n: int, k: int) -> tuple[int, int]:
     return 1, splits_for(g1)
 
 
-_DMA_TILES = {0: (128, 128), 1: (256, 128), 2: (256, 256)}      # rows of W x rows of X
-# microseconds that one round of workgroups (one per CU) takes at K = 4096, measured on MI355X
-_DMA_ROUND_US = {0: 48.0, 1: 72.0, 2: 124.0}
+# rows of W x rows of X of a workgroup.  Tiles 0 to 2 are gemm_dma (W and X through LDS), 3 to 5
+# gemm_wreg (W from memory into registers, X through LDS).
+_DMA_TILES = {0: (128, 128), 1: (256, 128), 2: (256, 256), 3: (256, 128), 4: (192, 128), 5: (128, 128)}
+# Microseconds that one round of workgroups takes at K = 4096, measured on MI355X: entry i is a round
+# with i + 1 workgroups on every CU.  gemm_dma runs one a CU; of gemm_wreg two or three share a CU, and
+# those of a last round that is less full run at the shorter time.
+_DMA_ROUND_US = {0: (48.0,), 1: (72.0,), 2: (124.0,), 3: (72.0, 127.0), 4: (64.0, 105.0), 5: (42.0, 79.0, 135.0)}
 
 
 def _dma_cost(tile: int, splits: int, m: int, n: int, k: int) -> float:
@@ -380,9 +384,11 @@ def _dma_cost(tile: int, splits: int, m: int, n: int, k: int) -> float:
     workgroups at the measured time of a round, not below the time to stream W once; a fixed cost for
     the launch, the first tiles and the epilogue; the partial sums written and read back."""
     bn, bm = _DMA_TILES[tile]
-    rounds = -(-(-(-m // bm) * -(-n // bn) * splits) // 256)
+    times = _DMA_ROUND_US[tile]
+    full, rest = divmod(-(-m // bm) * -(-n // bn) * splits, 256 * len(times))
+    us = full * times[-1] + (times[-(-rest // 256) - 1] if rest else 0.0)
     k_split = -(-(-(-k // splits)) // 32) * 32
-    main = max(rounds * _DMA_ROUND_US[tile] * k_split / 4096, n * k * 2 / 5.5e6)
+    main = max(us * k_split / 4096, n * k * 2 / 5.5e6)
     reduce = 2.5 + 2 * splits * m * n * 4 / 3.0e6 if splits > 1 else 0.0
     return main + 5.5 + reduce
 
@@ -397,12 +403,12 @@ def _dma_plan(m: int, n: int, k: int) -> list:
     a full one: a product of many rounds gets the large tile for as many columns (or, if that fits
     better, rows) as fill whole rounds and a smaller tile for the rest, if that is clearly faster by
     the same estimate."""
-    options = [(t, s) for t in (2, 1, 0) for s in (1, 2, 3, 4, 6, 8, 12, 16) if s == 1 or k // s >= 1024]
+    options = [(t, s) for t in (2, 1, 0, 3, 4, 5) for s in (1, 2, 3, 4, 6, 8, 12, 16) if s == 1 or k // s >= 1024]
     tile, splits = min(options, key=lambda o: (_dma_cost(o[0], o[1], m, n, k), o[1], -o[0]))
     plan, cost = [(tile, splits, 0, 0, 0, 0)], _dma_cost(tile, splits, m, n, k)
     if splits > 1:
         return plan
-    for big in (2, 1):
+    for big in (2, 1):                                          # (gemm_dma's tiles)
         bn, bm = _DMA_TILES[big]
         m_tiles, n_tiles = -(-m // bm), -(-n // bn)
         whole = m_tiles * n_tiles // 256 * 256                 # workgroups of the whole rounds
