@@ -40,46 +40,72 @@ __host__ __device__ __forceinline__ int64_t tiled_offset(int n, int k, int K) {
     return ((((int64_t)(n >> 4) * (K >> 5) + (k >> 5)) * 64) + (((k & 31) >> 3) << 4) + (n & 15)) * 8 + (k & 7);
 }
 
+// Four consecutive elements, the first index a multiple of 4 (one aligned store).
+__device__ __forceinline__ void store_four(void* C, int dt, int64_t i, const float* v) {
+    if (dt == DT_F32) *(f32x4*)((float*)C + i) = f32x4{v[0], v[1], v[2], v[3]};
+    else if (dt == DT_F16) *(f16x4*)((f16*)C + i) = f16x4{(f16)v[0], (f16)v[1], (f16)v[2], (f16)v[3]};
+    else *(bf16x4*)((bf16*)C + i) = bf16x4{(bf16)v[0], (bf16)v[1], (bf16)v[2], (bf16)v[3]};
+}
+
+// The EPI_ROPE epilogue in two parts, so that a kernel can fetch what it reads from memory early:
+// rope_angles gives cos and sin for the pairs at d and d + 2 of a head (row m at position p), and
+// rope_store4 rotates and stores.  include/kernels_cpu.hpp:82-100 and src/model/block.cpp:141-148, on
+// the accumulators.  `page`: the page of the row's cache slot that holds position p (k and v heads).
+__device__ __forceinline__ void rope_angles(const RopeStore& r, int m, int p, int head, int d, f32x2 (&t)[2],
+                                            bool table = false) {          // table: r.cos_sin is there
+#pragma unroll
+    for (int j = 0; j < 2; ++j) {
+        t[j] = f32x2{1.f, 0.f};
+        if (head < r.H + r.K && d + 2 * j < r.rotary_dim) {
+            if (table || r.cos_sin) t[j] = *(const f32x2*)(r.cos_sin + ((int64_t)m * (r.rotary_dim >> 1) + ((d + 2 * j) >> 1)) * 2);
+            else {
+                float sn, cs;
+                sincosf((float)p * r.inv_freq[(d + 2 * j) >> 1], &sn, &cs);
+                t[j] = f32x2{cs, sn};
+            }
+        }
+    }
+}
+
+__device__ __forceinline__ void rope_store4(const RopeStore& r, int m, int head, int d, const float* v, int p,
+                                            int64_t page, const f32x2 (&t)[2]) {
+    float o[4] = {v[0], v[1], v[2], v[3]};
+    if (head < r.H + r.K) {
+#pragma unroll
+        for (int j = 0; j < 4; j += 2) {
+            if (d + j < r.rotary_dim) {
+                const float cs = t[j >> 1][0], sn = t[j >> 1][1];
+                o[j] = v[j] * cs - v[j + 1] * sn;
+                o[j + 1] = v[j] * sn + v[j + 1] * cs;
+            }
+        }
+    }
+    if (head < r.H) {
+        store_four(r.q_out, r.dt, ((int64_t)m * r.H + head) * r.hd + d, o);
+        return;
+    }
+    const int tp = p % PAGE;
+    if (head < r.H + r.K) {
+        // four consecutive d of a key are consecutive in the page
+        store_four(r.k_pages, r.dt, page * r.page_stride + (int64_t)(head - r.H) * k_head_elems(r.hd) + k_offset(tp, d, r.hd), o);
+    } else {
+        const int64_t at = page * r.page_stride + (int64_t)(head - r.H - r.K) * v_head_elems(r.hd);
+#pragma unroll
+        for (int j = 0; j < 4; ++j) store_one(r.v_pages, r.dt, at + v_offset(tp, d + j, r.hd), o[j]);
+    }
+}
+
 // v[0..3] are the results for row m and columns n..n+3 (n a multiple of 4).
 __device__ __forceinline__ void epilogue4(const Epilogue& e, int m, int n, const float* v) {
     if (m >= e.M || n >= e.N) return;
     if (e.mode == EPI_ROPE) {
-        // include/kernels_cpu.hpp:82-100 and src/model/block.cpp:141-148, on the accumulators
         const RopeStore& r = e.rs;
         const int head = n / r.hd, d = n - head * r.hd;       // the 4 columns lie in one head (hd % 16 == 0)
         const int p = r.pos[m];
-        float o[4] = {v[0], v[1], v[2], v[3]};
-        if (head < r.H + r.K) {
-#pragma unroll
-            for (int j = 0; j < 4; j += 2) {
-                if (d + j < r.rotary_dim) {
-                    float sn, cs;
-                    if (r.cos_sin) {
-                        const f32x2 t = *(const f32x2*)(r.cos_sin + ((int64_t)m * (r.rotary_dim >> 1) + ((d + j) >> 1)) * 2);
-                        cs = t[0]; sn = t[1];
-                    } else sincosf((float)p * r.inv_freq[(d + j) >> 1], &sn, &cs);
-                    o[j] = v[j] * cs - v[j + 1] * sn;
-                    o[j + 1] = v[j] * sn + v[j + 1] * cs;
-                }
-            }
-        }
-        if (head < r.H) {
-            const int64_t at = ((int64_t)m * r.H + head) * r.hd + d;
-#pragma unroll
-            for (int j = 0; j < 4; ++j) store_one(r.q_out, r.dt, at + j, o[j]);
-        } else {
-            const int64_t page = r.page_table[(int64_t)r.tok_slot[m] * r.max_pages + p / PAGE];
-            const int tp = p % PAGE;
-            if (head < r.H + r.K) {
-                const int64_t at = page * r.page_stride + (int64_t)(head - r.H) * k_head_elems(r.hd);
-#pragma unroll
-                for (int j = 0; j < 4; ++j) store_one(r.k_pages, r.dt, at + k_offset(tp, d + j, r.hd), o[j]);
-            } else {
-                const int64_t at = page * r.page_stride + (int64_t)(head - r.H - r.K) * v_head_elems(r.hd);
-#pragma unroll
-                for (int j = 0; j < 4; ++j) store_one(r.v_pages, r.dt, at + v_offset(tp, d + j, r.hd), o[j]);
-            }
-        }
+        f32x2 t[2];
+        rope_angles(r, m, p, head, d, t);
+        const int64_t page = head < r.H ? 0 : r.page_table[(int64_t)r.tok_slot[m] * r.max_pages + p / PAGE];
+        rope_store4(r, m, head, d, v, p, page, t);
         return;
     }
     if (e.mode == EPI_SWIGLU || e.mode == EPI_GEGLU) {

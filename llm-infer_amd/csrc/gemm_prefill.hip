@@ -394,14 +394,18 @@ __global__ __launch_bounds__(64 * WAVES) void gemm_dma_kernel(const T* __restric
 // narrower tiles are for products whose number of tiles would otherwise leave a large part of the last
 // round of workgroups empty.
 // ===========================================================================
-template <class T, int NI>
+// MODE: EPI_ADD or EPI_ROPE for a kernel whose epilogue is that one alone and fetches what it reads from
+// memory (the residual; positions, pages and angles) a strip ahead; -1 for every epilogue, chosen at run
+// time, one strip's quads after the other.
+template <class T, int NI, int MJ, int MODE>
 __global__ __launch_bounds__(256) void gemm_wreg_kernel(const T* __restrict__ X, const T* __restrict__ Wt,
                                                         int K, int k_per_split, float* __restrict__ ws,
                                                         int n_begin, Epilogue e) {
     typedef typename Vec<T>::v8 v8;
-    constexpr int BN = 64 * NI, BM = 128, BK = 32, STAGES = 3;
-    constexpr int MJ = 8;                               // fragments of X per wave and step
-    constexpr int XU = BM / 16, PER_WAVE = XU / 4;      // units of X per stage, and per wave
+    // A step is 64 of K: two halves of 32, each one matrix instruction deep.
+    // MJ: fragments of X (16 rows each) per wave and half step; every wave takes all the tile's rows of X
+    constexpr int BN = 64 * NI, BM = 16 * MJ, XBUFS = 3, SLOTS = 4;
+    constexpr int XU = 2 * MJ, PER_WAVE = XU / 4;       // 1 KiB units of X per stage (two halves of MJ), and per wave
     constexpr int STAGE = XU * 1024;
     extern __shared__ __attribute__((aligned(16))) unsigned char smem_raw[];
 
@@ -412,7 +416,7 @@ __global__ __launch_bounds__(256) void gemm_wreg_kernel(const T* __restrict__ X,
     tile_of_workgroup(8, bx, by, bz);
     const int m0 = bx * BM, n0 = n_begin + by * BN;
     const int kb = bz * k_per_split, ke = min(K, kb + k_per_split);
-    const int n_steps = (ke - kb) / BK;
+    const int n_halves = (ke - kb) >> 5, n_steps = n_halves >> 1;       // the host: K and the splits are multiples of 64
     const int w_blocks = (e.N + 15) >> 4, steps = K >> 5;
 
     // this wave's rows of W: NI blocks of 16, each a run of 1 KiB units along K
@@ -422,31 +426,36 @@ __global__ __launch_bounds__(256) void gemm_wreg_kernel(const T* __restrict__ X,
         const int blk = min(n0 / 16 + wn * NI + i, w_blocks - 1);
         wsrc[i] = Wt + (((int64_t)blk * steps + (kb >> 5)) * 64 + lane) * 8;
     }
-    // this wave's share of a stage of X: unit u holds rows m0 + 16 u ..; a lane brings 16 bytes of row
-    // lane % 16 at k + 8 (lane / 16)
+    // this wave's share of a stage of X: unit q = MJ h + u holds half h of rows m0 + 16 u ..; a lane brings
+    // 16 bytes of row lane % 16 at k + 8 (lane / 16)
     const unsigned char* xbase = (const unsigned char*)(X + kb);
     uint32_t xoff[PER_WAVE];
 #pragma unroll
     for (int i = 0; i < PER_WAVE; ++i) {
-        const int u = wave * PER_WAVE + i;
+        const int u = (wave * PER_WAVE + i) % MJ;
         const int row = min(m0 + 16 * u + (lane & 15), e.M - 1);
         xoff[i] = ((uint32_t)row * (uint32_t)K + 8 * (lane >> 4)) * 2;
     }
-    auto fill = [&](int s, int buf) {
+    // Loads past the last half of K are not branched around: they fetch the last half again (into a buffer
+    // and registers that nothing reads), which keeps the count of loads in flight fixed.
+    const int last = n_halves - 1;
+    auto fill = [&](int s, int buf_off) {
 #pragma unroll
         for (int i = 0; i < PER_WAVE; ++i) {
-            const int u = wave * PER_WAVE + i;
+            const int q = wave * PER_WAVE + i;
+            const int half = min(2 * s + q / MJ, last);
             __builtin_amdgcn_global_load_lds(
-                (const __attribute__((address_space(1))) void*)(xbase + (int64_t)s * (BK * 2) + xoff[i]),
-                (__attribute__((address_space(3))) void*)(smem_raw + buf * STAGE + u * 1024), 16, 0, 0);
+                (const __attribute__((address_space(1))) void*)(xbase + (int64_t)half * 64 + xoff[i]),
+                (__attribute__((address_space(3))) void*)(smem_raw + buf_off + q * 1024), 16, 0, 0);
         }
     };
     // The loads of W are written as instructions so that the compiler does not place waits for them (at
     // the loop's head it would wait for every load in flight); the waits are placed by hand below.
-    auto fetch_w = [&](int s, v8 (&a)[NI]) {
+    auto fetch_w = [&](int half, v8 (&a)[NI]) {
+        const int64_t at = (int64_t)min(half, last) * 512;
 #pragma unroll
         for (int i = 0; i < NI; ++i)
-            asm volatile("global_load_dwordx4 %0, %1, off" : "=v"(a[i]) : "v"(wsrc[i] + (int64_t)s * 512) : "memory");
+            asm volatile("global_load_dwordx4 %0, %1, off" : "=v"(a[i]) : "v"(wsrc[i] + at) : "memory");
     };
 
     f32x4 acc[NI][MJ];
@@ -455,85 +464,213 @@ __global__ __launch_bounds__(256) void gemm_wreg_kernel(const T* __restrict__ X,
 #pragma unroll
         for (int j = 0; j < MJ; ++j) acc[i][j] = f32x4{0.f, 0.f, 0.f, 0.f};
 
-    const unsigned char* sB = smem_raw + lane * 16;
-    auto compute = [&](int buf, const v8 (&a)[NI]) {
-        v8 b[MJ];
-        const unsigned char* src = sB + buf * STAGE;
-#pragma unroll
-        for (int j = 0; j < MJ; ++j) b[j] = *(const v8*)(src + j * 1024);
-        __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-        for (int j = 0; j < MJ; ++j)
-#pragma unroll
-            for (int i = 0; i < NI; ++i) acc[i][j] = mfma16(a[i], b[j], acc[i][j]);
-        __builtin_amdgcn_sched_barrier(0);
-    };
+    // Half a step: the matrix instructions on one slot of W's fragments and on the fragments of X that are
+    // in b[]; as soon as the instructions that use b[j] are issued, b[j] is read again for the half after
+    // this one, so the LDS reads run under the matrix instructions, and so do the loads of W, which go
+    // into a slot as soon as its half is issued.  Between two barriers a wave issues 16 NI matrix
+    // instructions, and outside them only the wait, the barrier and its four loads of X.
+    // The LDS reads are written as instructions too, with the waits by hand: the read of b[j] is followed
+    // by seven others before b[j] is used, and LDS reads complete in order, so "at most 7 in flight" is the
+    // wait before every group of matrix instructions.  (Left to the compiler, each half begins with a wait
+    // for all eight, the last of which has only just been issued.)
+    v8 b[MJ];
+    const uint32_t lds_lane = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) unsigned char*)smem_raw + lane * 16;
+#define WREG_READ(J, FROM) asm volatile("ds_read_b128 %0, %1 offset:%2" : "=v"(b[J]) : "v"(FROM), "n"((J) * 1024));
+#define WREG_GROUP(J, A, NEXT)                                                             \
+    {                                                                                      \
+        __builtin_amdgcn_s_waitcnt(0xC07F | ((MJ - 1) << 8));   /* lgkmcnt(MJ - 1), nothing else */ \
+        __builtin_amdgcn_sched_barrier(0);                                                 \
+        _Pragma("unroll") for (int i = 0; i < NI; ++i) acc[i][J] = mfma16(A[i], b[J], acc[i][J]); \
+        __builtin_amdgcn_sched_barrier(0);                                                 \
+        WREG_READ(J, NEXT)                                                                 \
+        __builtin_amdgcn_sched_barrier(0);                                                 \
+    }
+#define WREG_EIGHT(F, ...) F(0, __VA_ARGS__) F(1, __VA_ARGS__) F(2, __VA_ARGS__) F(3, __VA_ARGS__) \
+                           F(4, __VA_ARGS__) F(5, __VA_ARGS__) F(6, __VA_ARGS__) F(7, __VA_ARGS__)
+#define WREG_NEXT_EIGHT(F, ...) F(8, __VA_ARGS__) F(9, __VA_ARGS__) F(10, __VA_ARGS__) F(11, __VA_ARGS__) \
+                                F(12, __VA_ARGS__) F(13, __VA_ARGS__) F(14, __VA_ARGS__) F(15, __VA_ARGS__)
+#define WREG_HALF(A, NEXT)                                                                 \
+    {                                                                                      \
+        const uint32_t next_ = (NEXT);                                                     \
+        WREG_EIGHT(WREG_GROUP, A, next_)                                                   \
+        if constexpr (MJ == 16) { WREG_NEXT_EIGHT(WREG_GROUP, A, next_) }                  \
+    }
+    static_assert(MJ == 8 || MJ == 16, "the groups of a half are written out");
 
-    // Loads past the last step are not branched around: they fetch the last step again (into a buffer
-    // and registers that nothing reads), which keeps the count of loads in flight fixed.
     // (The host gives every split of K at least one step.  Without this line the compiler builds a path
     // for no steps on which the ring's registers are written while the first loads are in flight.)
     if (n_steps <= 0) return;
-    const int last = n_steps - 1;
-    v8 a0[NI], a1[NI], a2[NI];
+    // In flight, in order: at the head of step s the loads of X of step s + 2 are issued, in its middle
+    // those of W's first half of step s + 2, at its end those of the second half.  Step s needs X of step
+    // s + 1 (its second half reads ahead into it) and its own W: all but the 2 NI loads issued last.
+    v8 ring[SLOTS][NI];
+    static_assert(PER_WAVE + 2 * NI <= 63 && 2 * NI <= 15, "the waits' counts");
     fill(0, 0);
-    fetch_w(0, a0);
-    fill(min(1, last), 1);
-    fetch_w(min(1, last), a1);
-    // one step of the loop: the loads of step s are complete when at most those of step s + 1 are in flight
-    // (PER_WAVE + NI a step, in order); the barrier then publishes everybody's share of stage s and says that
-    // everybody has read stage s - 1, whose buffer the loads of step s + 2 may fill
-#define WREG_STEP(S, BUF, ACUR, ANEW)                                              \
-    {                                                                              \
-        __builtin_amdgcn_s_waitcnt(0x0F70 | (PER_WAVE + NI));                       \
-        __builtin_amdgcn_s_barrier();                                              \
-        fill(min((S) + 2, last), ((BUF) + 2) % 3);                                 \
-        fetch_w(min((S) + 2, last), ANEW);                                         \
-        __builtin_amdgcn_sched_barrier(0);                                         \
-        compute(BUF, ACUR);                                                        \
-        __builtin_amdgcn_sched_barrier(0);                                         \
-    }
-    for (int s = 0; s < n_steps; s += 3) {
-        WREG_STEP(s, 0, a0, a2)
-        if (s + 1 < n_steps) WREG_STEP(s + 1, 1, a1, a0)
-        if (s + 2 < n_steps) WREG_STEP(s + 2, 2, a2, a1)
-    }
-#undef WREG_STEP
-    // Loads into the ring may still be in flight here (those past the last step).  The compiler does not
-    // know of them: without a use of the ring after the wait it would hand the ring's registers to the
-    // epilogue's values before the wait, and a load that lands late would overwrite an address.
-    __builtin_amdgcn_s_waitcnt(0x0070);
+    fetch_w(0, ring[0]);
+    fetch_w(1, ring[1]);
+    fill(1, STAGE);
+    fetch_w(2, ring[2]);
+    fetch_w(3, ring[3]);
+    // X of step 0 has landed (the count's upper two bits are bits 14 and 15 of the instruction's field)
+    __builtin_amdgcn_s_waitcnt(0x0F70 | ((PER_WAVE + 2 * NI) & 15) | (((PER_WAVE + 2 * NI) >> 4) << 14));
+    __builtin_amdgcn_s_barrier();
+    WREG_EIGHT(WREG_READ, lds_lane)
+    if constexpr (MJ == 16) { WREG_NEXT_EIGHT(WREG_READ, lds_lane) }
+    int cur = 0;                                                   // byte offset of the buffer of step s
+    for (int s = 0; s < n_steps; s += 2) {
 #pragma unroll
-    for (int i = 0; i < NI; ++i) asm volatile("" ::"v"(a0[i]), "v"(a1[i]), "v"(a2[i]));
+        for (int u = 0; u < 2; ++u) {                              // two steps a turn of the ring
+            if (s + u < n_steps) {
+                const int nxt = cur == (XBUFS - 1) * STAGE ? 0 : cur + STAGE;
+                const int free_buf = nxt == (XBUFS - 1) * STAGE ? 0 : nxt + STAGE;
+                // X of step s + 1 and W of step s have landed (all but the 2 NI loads issued last), and this
+                // wave's reads of the buffer that is filled next are done (all but the MJ issued last, which
+                // read the buffer of this step; the field holds 15 at most); the barrier publishes the one
+                // and frees the other
+                __builtin_amdgcn_s_waitcnt(0x0070 | ((MJ < 15 ? MJ : 15) << 8) | (2 * NI));
+                __builtin_amdgcn_s_barrier();
+                fill(s + u + 2, free_buf);
+                __builtin_amdgcn_sched_barrier(0);
+                WREG_HALF(ring[2 * u], lds_lane + cur + MJ * 1024)
+                fetch_w(2 * (s + u + 2), ring[2 * u]);
+                __builtin_amdgcn_sched_barrier(0);
+                WREG_HALF(ring[2 * u + 1], lds_lane + nxt)
+                fetch_w(2 * (s + u + 2) + 1, ring[2 * u + 1]);
+                __builtin_amdgcn_sched_barrier(0);
+                cur = nxt;
+            }
+        }
+    }
+#undef WREG_HALF
+#undef WREG_NEXT_EIGHT
+#undef WREG_EIGHT
+#undef WREG_GROUP
+#undef WREG_READ
+    __builtin_amdgcn_s_waitcnt(0x0070);
+    // Loads into the ring and reads into b[] may still be in flight here (those past the last step).  The
+    // compiler does not know of them: without a use of these registers after the wait it would hand them to
+    // the epilogue's values before the wait, and a load that lands late would overwrite an address.
+#pragma unroll
+    for (int u = 0; u < SLOTS; ++u)
+#pragma unroll
+        for (int i = 0; i < NI; ++i) asm volatile("" ::"v"(ring[u][i]));
+#pragma unroll
+    for (int j = 0; j < MJ; ++j) asm volatile("" ::"v"(b[j]));
     __builtin_amdgcn_sched_barrier(0);
-    __syncthreads();
 
     // Epilogue through LDS, a strip of 16 rows of X x 16 NI rows of W at a time: accumulator q of a 16x16
     // block is W row 4 (lane / 16) + q, X row lane % 16; read back, consecutive lanes hold consecutive
-    // quads of columns of one row.  The loop over the strip's quads is not unrolled (one copy of the
-    // epilogue in the code).
-    constexpr int SLD = 16 * NI + 4, QUADS = 4 * NI;
-    float* stage = (float*)smem_raw + wave * (16 * SLD);
-    const int r = lane & 15, g = lane >> 4;
-#pragma unroll
-    for (int j = 0; j < MJ; ++j) {
-#pragma unroll
-        for (int i = 0; i < NI; ++i) *(f32x4*)(stage + r * SLD + 16 * i + 4 * g) = acc[i][j];
-        __builtin_amdgcn_wave_barrier();
-        const int mb = m0 + 16 * j, nb = n0 + wn * (16 * NI);
-#pragma unroll 1
-        for (int q = lane; q < 16 * QUADS; q += 64) {
-            const int rr = q / QUADS, c = (q % QUADS) * 4;
-            const f32x4 v = *(const f32x4*)(stage + rr * SLD + c);
-            const float vv[4] = {v[0], v[1], v[2], v[3]};
-            if (gridDim.z == 1) epilogue4(e, mb + rr, nb + c, vv);
-            else if (mb + rr < e.M) {
-                float* p = ws + ((int64_t)bz * e.M + mb + rr) * e.N + nb + c;
-#pragma unroll
-                for (int jj = 0; jj < 4; ++jj) if (nb + c + jj < e.N) p[jj] = vv[jj];
-            }
+    // quads of columns of one row.  A wave has room for two strips.
+    constexpr int SLD = 16 * NI + 4, QUADS = 4 * NI, STRIP = 16 * SLD;
+    constexpr int INFO = XBUFS * STAGE > 4 * 2 * STRIP * 4 ? XBUFS * STAGE : 4 * 2 * STRIP * 4;   // behind the stages and the strips
+    int* row_pos = (int*)(smem_raw + INFO);
+    int* row_page = row_pos + BM;
+    if constexpr (MODE == EPI_ROPE) {
+        // position and cache page of the tile's rows, once (two dependent loads a row)
+        if (tid < BM) {
+            const int m = min(m0 + tid, e.M - 1), p = e.rs.pos[m];
+            row_pos[tid] = p;
+            row_page[tid] = (e.rs.K > 0 && n0 + BN > e.rs.H * e.rs.hd)
+                                ? e.rs.page_table[(int64_t)e.rs.tok_slot[m] * e.rs.max_pages + p / PAGE] : 0;
         }
-        __builtin_amdgcn_wave_barrier();
+    }
+    __syncthreads();
+    float* stage = (float*)smem_raw + wave * (2 * STRIP);
+    const int r = lane & 15, g = lane >> 4;
+    const int nb = n0 + wn * (16 * NI);                 // this wave's first column
+    auto to_stage = [&](int j, int place) {
+#pragma unroll
+        for (int i = 0; i < NI; ++i) *(f32x4*)(stage + place * STRIP + r * SLD + 16 * i + 4 * g) = acc[i][j];
+    };
+
+    if constexpr (MODE == EPI_ADD) {
+        // C += product (float32, N a multiple of 4, one split: the host sees to it).  NI quads a lane and
+        // strip, in row row_of[it], from column col_of[it]; the residual of strip j + 1 is fetched before
+        // strip j is added and stored.
+        float* C = (float*)e.C;
+        int row_of[NI], col_of[NI];
+#pragma unroll
+        for (int it = 0; it < NI; ++it) {
+            const int q = lane + 64 * it;
+            row_of[it] = q / QUADS;
+            col_of[it] = nb + (q % QUADS) * 4;
+        }
+        f32x4 res[2][NI];
+        auto fetch = [&](int j, f32x4 (&c)[NI]) {
+#pragma unroll
+            for (int it = 0; it < NI; ++it) {
+                const int m = m0 + 16 * j + row_of[it];
+                if (m < e.M && col_of[it] < e.N) c[it] = *(const f32x4*)(C + (int64_t)m * e.N + col_of[it]);
+            }
+        };
+        fetch(0, res[0]);
+#pragma unroll
+        for (int j = 0; j < MJ; ++j) {
+            to_stage(j, 0);
+            __builtin_amdgcn_wave_barrier();
+            if (j + 1 < MJ) fetch(j + 1, res[(j + 1) & 1]);
+#pragma unroll
+            for (int it = 0; it < NI; ++it) {
+                const int m = m0 + 16 * j + row_of[it];
+                if (m < e.M && col_of[it] < e.N) {
+                    f32x4 o = res[j & 1][it];
+                    const f32x4 v = *(const f32x4*)(stage + row_of[it] * SLD + (col_of[it] - nb));
+                    o[0] += v[0]; o[1] += v[1]; o[2] += v[2]; o[3] += v[3];
+                    *(f32x4*)(C + (int64_t)m * e.N + col_of[it]) = o;
+                }
+            }
+            __builtin_amdgcn_wave_barrier();
+        }
+    } else {
+        // Two strips a pass; the loop over their quads is not unrolled (one copy of the epilogue's code a
+        // pass).  With MODE == EPI_ROPE: rotation and cache write with the table of angles (the host sees
+        // to it), positions and pages from LDS, the angles of a quad fetched while the quad before it is
+        // rotated and stored.
+        const RopeStore& rs = e.rs;
+        auto place_of = [&](int q, int& row, int& n) {      // quad q of a pass: row of the tile's strip pair, column
+            const int strip = q / (16 * QUADS), qq = q - strip * (16 * QUADS);
+            row = 16 * strip + qq / QUADS;
+            n = nb + (qq % QUADS) * 4;
+        };
+#pragma unroll
+        for (int jc = 0; jc < MJ; jc += 2) {
+            to_stage(jc, 0);
+            to_stage(jc + 1, 1);
+            __builtin_amdgcn_wave_barrier();
+            const int mb = m0 + 16 * jc;
+            f32x2 ang[2] = {f32x2{1.f, 0.f}, f32x2{1.f, 0.f}};
+            int row, n;
+            place_of(lane, row, n);
+            if constexpr (MODE == EPI_ROPE) {
+                if (mb + row < e.M && n < e.N) rope_angles(rs, mb + row, 0, n / rs.hd, n % rs.hd, ang, true);
+            }
+#pragma unroll 1
+            for (int q = lane; q < 2 * 16 * QUADS; q += 64) {
+                const f32x4 v = *(const f32x4*)(stage + (row >> 4) * STRIP + (row & 15) * SLD + (n - nb));
+                const float vv[4] = {v[0], v[1], v[2], v[3]};
+                const int m = mb + row, col = n;
+                if constexpr (MODE == EPI_ROPE) {
+                    const f32x2 now[2] = {ang[0], ang[1]};
+                    if (q + 64 < 2 * 16 * QUADS) {
+                        place_of(q + 64, row, n);
+                        if (mb + row < e.M && n < e.N) rope_angles(rs, mb + row, 0, n / rs.hd, n % rs.hd, ang, true);
+                    }
+                    if (m < e.M && col < e.N) {
+                        const int head = col / rs.hd;
+                        rope_store4(rs, m, head, col - head * rs.hd, vv, row_pos[m - m0], row_page[m - m0], now);
+                    }
+                } else {
+                    if (q + 64 < 2 * 16 * QUADS) place_of(q + 64, row, n);
+                    if (gridDim.z == 1) epilogue4(e, m, col, vv);
+                    else if (m < e.M) {
+                        float* p = ws + ((int64_t)bz * e.M + m) * e.N + col;
+#pragma unroll
+                        for (int jj = 0; jj < 4; ++jj) if (col + jj < e.N) p[jj] = vv[jj];
+                    }
+                }
+            }
+            __builtin_amdgcn_wave_barrier();
+        }
     }
 }
 
@@ -585,8 +722,10 @@ extern "C" int li_gemm_big(const void* X, const void* W, int tiled, int dt, void
     return LI_OK;
 }
 
-// tile: 0 = 128 x 128, 1 = 256 x 128, 2 = 256 x 256 with 8 waves (rows of W x rows of X); BK = 32; W tiled.
-//  The launch computes the columns n_begin .. n_begin + n_count - 1 of the product
+// tile (rows of W x rows of X): 0 = 128 x 128, 1 = 256 x 128, 2 = 256 x 256 with 8 waves: gemm_dma, K in steps
+// of 32; 3 = 256 x 128, 4 = 192 x 128, 5 = 128 x 128, 6 = 256 x 256: gemm_wreg, K (and every split of it) a
+// multiple of 64.
+// W tiled.  The launch computes the columns n_begin .. n_begin + n_count - 1 of the product
 // (n_begin a multiple of 16; n_count 0: all from n_begin on), so that a product whose tiles do not
 // fill the last round of workgroups can finish with a smaller tile; K is split only for all columns.
 extern "C" int li_gemm_dma(const void* X, const void* Wt, int dt, void* C, int out_dt, int mode,
@@ -596,14 +735,15 @@ extern "C" int li_gemm_dma(const void* X, const void* Wt, int dt, void* C, int o
     if (rc) return rc;
     if (dt != DT_F16 && dt != DT_BF16) return LI_BAD_ARG;
     if (K % 32 != 0 || ((uintptr_t)X & 15) || ((uintptr_t)Wt & 15)) return LI_UNSUPPORTED;
-    if (tile < 0 || tile > 5) return LI_BAD_ARG;
+    if (tile < 0 || tile > 6) return LI_BAD_ARG;
     if ((int64_t)M * K * 2 >= ((int64_t)1 << 32)) return LI_UNSUPPORTED;     // 32-bit offsets into X
     if (splits < 1 || (splits > 1 && !ws)) return LI_BAD_ARG;
     if (n_begin < 0 || n_begin >= N || (n_begin & 15) || n_count < 0 || n_begin + n_count > N) return LI_BAD_ARG;
     if (n_count == 0) n_count = N - n_begin;
-    // tiles 0 to 2: gemm_dma; 3 to 5: gemm_wreg
-    static const int tile_bn[6] = {128, 256, 256, 256, 192, 128}, tile_bm[6] = {128, 128, 256, 128, 128, 128};
-    const int bn = tile_bn[tile], bm = tile_bm[tile], bk = 32;
+    // tiles 0 to 2: gemm_dma; 3 to 6: gemm_wreg
+    static const int tile_bn[7] = {128, 256, 256, 256, 192, 128, 256}, tile_bm[7] = {128, 128, 256, 128, 128, 128, 256};
+    const int bn = tile_bn[tile], bm = tile_bm[tile], bk = tile >= 3 ? 64 : 32;
+    if (K % bk != 0) return LI_UNSUPPORTED;                                  // gemm_wreg steps by 64 of K
     if (n_begin + n_count < N && n_count % bn != 0) return LI_BAD_ARG;       // only the last columns may end inside a tile
     if (splits > 1 && n_count != N) return LI_BAD_ARG;
     if (M == 0) return LI_OK;
@@ -613,20 +753,38 @@ extern "C" int li_gemm_dma(const void* X, const void* Wt, int dt, void* C, int o
     const size_t lds = (size_t)3 * (bn + bm) / 16 * 1024;
     int k_per_split = ((K + splits - 1) / splits + bk - 1) / bk * bk;
     splits = (K + k_per_split - 1) / k_per_split;
-    dim3 grid((M + bm - 1) / bm, (n_count + bn - 1) / bn, splits), block(bm == 256 ? 512 : 256);
+    dim3 grid((M + bm - 1) / bm, (n_count + bn - 1) / bn, splits), block(tile == 2 ? 512 : 256);
     if (tile >= 3) {
-        // three stages of X; the epilogue stages 16 x (bn / 4 + 4) floats a wave in the same LDS
-        const size_t stages = (size_t)3 * (bm / 16) * 1024, strips = (size_t)4 * 16 * (bn / 4 + 4) * 4;
-        const size_t wlds = stages > strips ? stages : strips;
-#define WGO(T, NI) gemm_wreg_kernel<T, NI><<<grid, block, wlds, stream>>>((const T*)X, (const T*)Wt, K, k_per_split, ws, n_begin, e)
-#define WLAUNCH(T)                           \
-    do {                                     \
-        if (tile == 3) WGO(T, 4);            \
-        else if (tile == 4) WGO(T, 3);       \
-        else WGO(T, 2);                      \
+        // three stages of X; the epilogue stages two strips of 16 x (bn / 4 + 4) floats a wave in the same LDS, and
+        // behind both lie a position and a page for each of the tile's rows
+        const size_t stages = (size_t)3 * 2 * (bm / 16) * 1024, strips = (size_t)4 * 2 * 16 * (bn / 4 + 4) * 4;   // (a step is 64 of K)
+        const size_t wlds = (stages > strips ? stages : strips) + (size_t)2 * bm * 4;
+        // the kernels of one epilogue: the residual sum into float32 with whole quads of columns; the
+        // rotation with a table of angles
+        const int one = splits > 1 ? -1 : (mode == EPI_ADD && N % 4 == 0) ? EPI_ADD : (mode == EPI_ROPE && e.rs.cos_sin) ? EPI_ROPE : -1;
+#define WGO(T, NI, MJ, MODE)                                                                            \
+    do {                                                                                               \
+        auto kfn = gemm_wreg_kernel<T, NI, MJ, MODE>;                                                  \
+        if (wlds > 65536 && hipFuncSetAttribute((const void*)kfn, hipFuncAttributeMaxDynamicSharedMemorySize, (int)wlds) != hipSuccess) \
+            return LI_HIP_ERROR;                                                                       \
+        kfn<<<grid, block, wlds, stream>>>((const T*)X, (const T*)Wt, K, k_per_split, ws, n_begin, e);  \
+    } while (0)
+#define WMODE(T, NI, MJ)                                 \
+    do {                                                 \
+        if (one == EPI_ADD) WGO(T, NI, MJ, EPI_ADD);     \
+        else if (one == EPI_ROPE) WGO(T, NI, MJ, EPI_ROPE); \
+        else WGO(T, NI, MJ, -1);                         \
+    } while (0)
+#define WLAUNCH(T)                               \
+    do {                                         \
+        if (tile == 3) WMODE(T, 4, 8);           \
+        else if (tile == 4) WMODE(T, 3, 8);      \
+        else if (tile == 5) WMODE(T, 2, 8);      \
+        else WMODE(T, 4, 16);                    \
     } while (0)
         if (dt == DT_F16) WLAUNCH(f16); else WLAUNCH(bf16);
 #undef WLAUNCH
+#undef WMODE
 #undef WGO
         LI_CHECK_LAUNCH();
         if (splits > 1) {

@@ -337,6 +337,7 @@ def _run_dma(x, wd, out, out_dt, mode, m, n, k, n_out, plan, rope) -> None:
     for tile, splits, n_begin, n_count, m_begin, m_count in plan:
         rows = m_count or m - m_begin
         _need(0 <= m_begin < m and m_begin + rows <= m, "gemm_dma: rows outside the product")
+        _need(tile < 3 or k % 64 == 0, "gemm_wreg (tiles 3 to 6): K must be a multiple of 64")
         ws = _workspace(splits * rows * n, x.device) if splits > 1 else None
         xp = c_void_p(x.data_ptr() + m_begin * k * x.element_size())
         op = c_void_p(out.data_ptr() + m_begin * n_out * out.element_size()) if out is not None else c_void_p(0)
@@ -370,40 +371,46 @@ def _stream_shape(n: int, k: int) -> tuple[int, int]:
     return 1, splits_for(g1)
 
 
-# rows of W x rows of X of a workgroup.  Tiles 0 to 2 are gemm_dma (W and X through LDS), 3 to 5
-# gemm_wreg (W from memory into registers, X through LDS).
-_DMA_TILES = {0: (128, 128), 1: (256, 128), 2: (256, 256), 3: (256, 128), 4: (192, 128), 5: (128, 128)}
-# Microseconds that one round of workgroups takes at K = 4096, measured on MI355X: entry i is a round
-# with i + 1 workgroups on every CU.  gemm_dma runs one a CU; of gemm_wreg two or three share a CU, and
-# those of a last round that is less full run at the shorter time.
-_DMA_ROUND_US = {0: (48.0,), 1: (72.0,), 2: (124.0,), 3: (72.0, 127.0), 4: (64.0, 105.0), 5: (42.0, 79.0, 135.0)}
+# rows of W x rows of X of a workgroup.  Tiles 0 to 2 are gemm_dma (W and X through LDS), 3 to 6
+# gemm_wreg (W from memory into registers, X through LDS; K in steps of 64).
+_DMA_TILES = {0: (128, 128), 1: (256, 128), 2: (256, 256), 3: (256, 128), 4: (192, 128), 5: (128, 128), 6: (256, 256)}
+# Microseconds that one round of workgroups takes, measured on MI355X, as (a, c): a K / 4096 + c.  Entry i
+# is a round with i + 1 workgroups on every CU.  gemm_dma and the largest tile of gemm_wreg run one a CU;
+# of the other tiles of gemm_wreg two or three share a CU, and those of a last round that is less full run
+# at the shorter time.
+_DMA_ROUND_US = {0: ((48.0, 0.0),), 1: ((72.0, 0.0),), 2: ((124.0, 0.0),),
+                 3: ((55.5, 11.3), (121.0, 0.0)), 4: ((47.0, 10.7), (101.0, 0.0)),
+                 5: ((46.1, 4.9), (79.7, 4.3), (123.0, 0.0)), 6: ((104.8, 20.0),)}
 
 
 def _dma_cost(tile: int, splits: int, m: int, n: int, k: int) -> float:
-    """Estimated microseconds of one gemm_dma launch (and its split-K reduction): rounds of
+    """Estimated microseconds of one launch of the prefill product (and its split-K reduction): rounds of
     workgroups at the measured time of a round, not below the time to stream W once; a fixed cost for
     the launch, the first tiles and the epilogue; the partial sums written and read back."""
     bn, bm = _DMA_TILES[tile]
     times = _DMA_ROUND_US[tile]
     full, rest = divmod(-(-m // bm) * -(-n // bn) * splits, 256 * len(times))
-    us = full * times[-1] + (times[-(-rest // 256) - 1] if rest else 0.0)
     k_split = -(-(-(-k // splits)) // 32) * 32
-    main = max(us * k_split / 4096, n * k * 2 / 5.5e6)
+    us = 0.0
+    for count, (a, c) in ((full, times[-1]), (1 if rest else 0, times[-(-rest // 256) - 1])):
+        us += count * (a * k_split / 4096 + c)
+    main = max(us, n * k * 2 / 5.5e6)
     reduce = 2.5 + 2 * splits * m * n * 4 / 3.0e6 if splits > 1 else 0.0
     return main + 5.5 + reduce
 
 
 @functools.lru_cache(maxsize=4096)
 def _dma_plan(m: int, n: int, k: int) -> list:
-    """The launches of gemm_dma for a product: (tile, splits of K, first column, columns, first row,
-    rows) each (0 columns or rows: all from the first on).
+    """The launches of the prefill product (gemm_dma and gemm_wreg, one entry point): (tile, splits of
+    K, first column, columns, first row, rows) each (0 columns or rows: all from the first on).
     Tile and splits are the pair with the least estimated time (`_dma_cost`): few rows of X want
     K split so that most CUs get a workgroup, but every split adds partial sums to write and read.
-    Workgroups run in rounds of one per CU, and a last round that is nearly empty costs as much as
-    a full one: a product of many rounds gets the large tile for as many columns (or, if that fits
-    better, rows) as fill whole rounds and a smaller tile for the rest, if that is clearly faster by
-    the same estimate."""
-    options = [(t, s) for t in (2, 1, 0, 3, 4, 5) for s in (1, 2, 3, 4, 6, 8, 12, 16) if s == 1 or k // s >= 1024]
+    gemm_wreg's tiles are there when K is a multiple of 64.  gemm_dma's workgroups run in rounds of
+    one per CU, and a last round that is nearly empty costs as much as a full one: a product of many
+    rounds may get its large tile for as many columns (or, if that fits better, rows) as fill whole
+    rounds and a smaller tile for the rest, if that is clearly faster by the same estimate."""
+    tiles = (2, 1, 0, 3, 4, 5, 6) if k % 64 == 0 else (2, 1, 0)            # gemm_wreg steps by 64 of K
+    options = [(t, s) for t in tiles for s in (1, 2, 3, 4, 6, 8, 12, 16) if s == 1 or k // s >= 1024]
     tile, splits = min(options, key=lambda o: (_dma_cost(o[0], o[1], m, n, k), o[1], -o[0]))
     plan, cost = [(tile, splits, 0, 0, 0, 0)], _dma_cost(tile, splits, m, n, k)
     if splits > 1:
