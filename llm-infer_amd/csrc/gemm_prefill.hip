@@ -426,26 +426,29 @@ __global__ __launch_bounds__(256) void gemm_wreg_kernel(const T* __restrict__ X,
         const int blk = min(n0 / 16 + wn * NI + i, w_blocks - 1);
         wsrc[i] = Wt + (((int64_t)blk * steps + (kb >> 5)) * 64 + lane) * 8;
     }
-    // this wave's share of a stage of X: unit q = MJ h + u holds half h of rows m0 + 16 u ..; a lane brings
-    // 16 bytes of row lane % 16 at k + 8 (lane / 16)
+    // This wave's share of a stage of X.  A 1 KiB unit holds 8 rows x 64 of K, so that the 8 lanes of a row
+    // fetch one whole 128-byte line (16 rows x 32 of K, the operand's own order, would fetch two half
+    // lines a row and pass twice as many lines through the CU's cache).  Lane 8 p + c of unit q brings
+    // chunk c ^ p (8 of K) of row m0 + 8 q + p: the exclusive-or spreads the 8 rows, which lie 128 bytes
+    // apart in LDS, over all banks when 16 lanes read one chunk of 16 rows as an operand.
     const unsigned char* xbase = (const unsigned char*)(X + kb);
     uint32_t xoff[PER_WAVE];
 #pragma unroll
     for (int i = 0; i < PER_WAVE; ++i) {
-        const int u = (wave * PER_WAVE + i) % MJ;
-        const int row = min(m0 + 16 * u + (lane & 15), e.M - 1);
-        xoff[i] = ((uint32_t)row * (uint32_t)K + 8 * (lane >> 4)) * 2;
+        const int q = wave * PER_WAVE + i, p = lane >> 3;
+        const int row = min(m0 + 8 * q + p, e.M - 1);
+        xoff[i] = ((uint32_t)row * (uint32_t)K + 8 * ((lane & 7) ^ p)) * 2;
     }
-    // Loads past the last half of K are not branched around: they fetch the last half again (into a buffer
+    // Loads past the last step of K are not branched around: they fetch the last step again (into a buffer
     // and registers that nothing reads), which keeps the count of loads in flight fixed.
     const int last = n_halves - 1;
     auto fill = [&](int s, int buf_off) {
+        const int64_t at = (int64_t)min(s, n_steps - 1) * 128;
 #pragma unroll
         for (int i = 0; i < PER_WAVE; ++i) {
             const int q = wave * PER_WAVE + i;
-            const int half = min(2 * s + q / MJ, last);
             __builtin_amdgcn_global_load_lds(
-                (const __attribute__((address_space(1))) void*)(xbase + (int64_t)half * 64 + xoff[i]),
+                (const __attribute__((address_space(1))) void*)(xbase + at + xoff[i]),
                 (__attribute__((address_space(3))) void*)(smem_raw + buf_off + q * 1024), 16, 0, 0);
         }
     };
@@ -474,8 +477,13 @@ __global__ __launch_bounds__(256) void gemm_wreg_kernel(const T* __restrict__ X,
     // wait before every group of matrix instructions.  (Left to the compiler, each half begins with a wait
     // for all eight, the last of which has only just been issued.)
     v8 b[MJ];
-    const uint32_t lds_lane = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) unsigned char*)smem_raw + lane * 16;
-#define WREG_READ(J, FROM) asm volatile("ds_read_b128 %0, %1 offset:%2" : "=v"(b[J]) : "v"(FROM), "n"((J) * 1024));
+    // where lane (r = lane % 16, g = lane / 16) finds row r, chunk 4 h + g (half h) of fragment 0: unit
+    // r / 8, place 8 (r % 8) + ((4 h + g) ^ r % 8); fragment j lies 2 KiB on
+    const uint32_t lds_base = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) unsigned char*)smem_raw +
+                              ((lane >> 3) & 1) * 1024 + (lane & 7) * 128;
+    const uint32_t lds_lane = lds_base + ((lane >> 4) ^ (lane & 7)) * 16;
+    const uint32_t lds_lane2 = lds_base + ((4 + (lane >> 4)) ^ (lane & 7)) * 16;
+#define WREG_READ(J, FROM) asm volatile("ds_read_b128 %0, %1 offset:%2" : "=v"(b[J]) : "v"(FROM), "n"((J) * 2048));
 #define WREG_GROUP(J, A, NEXT)                                                             \
     {                                                                                      \
         __builtin_amdgcn_s_waitcnt(0xC07F | ((MJ - 1) << 8));   /* lgkmcnt(MJ - 1), nothing else */ \
@@ -531,7 +539,7 @@ __global__ __launch_bounds__(256) void gemm_wreg_kernel(const T* __restrict__ X,
                 __builtin_amdgcn_s_barrier();
                 fill(s + u + 2, free_buf);
                 __builtin_amdgcn_sched_barrier(0);
-                WREG_HALF(ring[2 * u], lds_lane + cur + MJ * 1024)
+                WREG_HALF(ring[2 * u], lds_lane2 + cur)
                 fetch_w(2 * (s + u + 2), ring[2 * u]);
                 __builtin_amdgcn_sched_barrier(0);
                 WREG_HALF(ring[2 * u + 1], lds_lane + nxt)

@@ -379,8 +379,8 @@ _DMA_TILES = {0: (128, 128), 1: (256, 128), 2: (256, 256), 3: (256, 128), 4: (19
 # of the other tiles of gemm_wreg two or three share a CU, and those of a last round that is less full run
 # at the shorter time.
 _DMA_ROUND_US = {0: ((48.0, 0.0),), 1: ((72.0, 0.0),), 2: ((124.0, 0.0),),
-                 3: ((55.5, 11.3), (121.0, 0.0)), 4: ((47.0, 10.7), (101.0, 0.0)),
-                 5: ((46.1, 4.9), (79.7, 4.3), (123.0, 0.0)), 6: ((104.8, 20.0),)}
+                 3: ((53.0, 9.0), (103.0, 5.0)), 4: ((35.0, 13.0), (73.0, 12.0)),
+                 5: ((31.4, 3.4), (57.1, 3.8), (89.0, 0.0)), 6: ((104.0, 14.0),)}
 
 
 def _dma_cost(tile: int, splits: int, m: int, n: int, k: int) -> float:

@@ -239,7 +239,7 @@ def test_gate_activation_alone(ops):
         assert ops.swiglu(gu, torch.bfloat16, gelu=gelu).dtype == torch.bfloat16
 
 
-@pytest.mark.parametrize("M,N,K", [(2048, 8560, 736), (5000, 4048, 736), (8192, 2400, 1536)])
+@pytest.mark.parametrize("M,N,K", [(2048, 8560, 736), (5000, 4048, 736)])
 def test_products_that_end_with_a_smaller_tile(ops, M, N, K):
     """Sizes at which the planner itself splits a product: the large tile for the columns (or rows) that
     fill whole rounds of workgroups, a smaller tile for the rest."""
