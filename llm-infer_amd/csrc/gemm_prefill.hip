@@ -385,26 +385,29 @@ __global__ __launch_bounds__(64 * WAVES) void gemm_dma_kernel(const T* __restric
 // ===========================================================================
 // gemm_wreg: the prefill product against a tiled W with W never in LDS.  A tiled weight lies in memory
 // in the order in which the 16x16x32 matrix instruction takes operand A, so a wave loads its fragments of
-// W straight from global memory into registers (1 KiB contiguous a load) and only X goes through LDS
-// (global_load_lds into 1 KiB units of 16 rows x 32 of K, which are operand B as they lie).  Four waves,
-// each with 16 NI rows of W and all 128 rows of X of the tile (64 NI x 128); two workgroups (three of
-// the narrowest tile) share a CU, and one's waits are the other's matrix time.  Per 32 of K a wave
-// issues NI loads of W, 8 LDS reads and 8 NI matrix instructions.  Three stages: the loads of step s + 2
-// (X into LDS, W into a ring of registers) are issued when step s begins; one barrier a step.  The
-// narrower tiles are for products whose number of tiles would otherwise leave a large part of the last
-// round of workgroups empty.
+// W straight from global memory into a ring of registers (1 KiB contiguous a load: 8 whole lines) and only
+// X goes through LDS (global_load_lds).  Four waves, each with 16 NI rows of W and all 128 rows of X of the
+// tile (64 NI x 128); two workgroups (three of the narrowest tile) share a CU.  A step is 64 of K: between
+// two barriers a wave issues 16 NI matrix instructions, and the LDS reads of the next fragments of X and
+// the loads of W two steps ahead are issued between them, so that outside the matrix instructions a step
+// has only its wait, its barrier and four loads of X.  What was measured on the way (M = 8,192, random
+// float16): one barrier per 32 of K with all LDS reads before the matrix instructions 1.08 to 1.12 PFLOP/s;
+// reads under the matrix instructions and 64 of K a barrier 1.11 to 1.18; X fetched as whole 128-byte
+// lines instead of two half lines a row 1.23 to 1.32 (the CU's cache takes a request per line touched).
+// The narrower tiles are for products whose number of tiles would otherwise leave a large part of the
+// last round of workgroups empty.
 // ===========================================================================
 // MODE: EPI_ADD or EPI_ROPE for a kernel whose epilogue is that one alone and fetches what it reads from
-// memory (the residual; positions, pages and angles) a strip ahead; -1 for every epilogue, chosen at run
-// time, one strip's quads after the other.
-template <class T, int NI, int MJ, int MODE>
+// memory early (the residual a strip ahead; positions and pages once, angles a quad ahead); -1 for every
+// epilogue, chosen at run time.
+template <class T, int NI, int MODE>
 __global__ __launch_bounds__(256) void gemm_wreg_kernel(const T* __restrict__ X, const T* __restrict__ Wt,
                                                         int K, int k_per_split, float* __restrict__ ws,
                                                         int n_begin, Epilogue e) {
     typedef typename Vec<T>::v8 v8;
     // A step is 64 of K: two halves of 32, each one matrix instruction deep.
     // MJ: fragments of X (16 rows each) per wave and half step; every wave takes all the tile's rows of X
-    constexpr int BN = 64 * NI, BM = 16 * MJ, XBUFS = 3, SLOTS = 4;
+    constexpr int MJ = 8, BN = 64 * NI, BM = 16 * MJ, XBUFS = 3, SLOTS = 4;
     constexpr int XU = 2 * MJ, PER_WAVE = XU / 4;       // 1 KiB units of X per stage (two halves of MJ), and per wave
     constexpr int STAGE = XU * 1024;
     extern __shared__ __attribute__((aligned(16))) unsigned char smem_raw[];
@@ -495,15 +498,12 @@ __global__ __launch_bounds__(256) void gemm_wreg_kernel(const T* __restrict__ X,
     }
 #define WREG_EIGHT(F, ...) F(0, __VA_ARGS__) F(1, __VA_ARGS__) F(2, __VA_ARGS__) F(3, __VA_ARGS__) \
                            F(4, __VA_ARGS__) F(5, __VA_ARGS__) F(6, __VA_ARGS__) F(7, __VA_ARGS__)
-#define WREG_NEXT_EIGHT(F, ...) F(8, __VA_ARGS__) F(9, __VA_ARGS__) F(10, __VA_ARGS__) F(11, __VA_ARGS__) \
-                                F(12, __VA_ARGS__) F(13, __VA_ARGS__) F(14, __VA_ARGS__) F(15, __VA_ARGS__)
 #define WREG_HALF(A, NEXT)                                                                 \
     {                                                                                      \
         const uint32_t next_ = (NEXT);                                                     \
         WREG_EIGHT(WREG_GROUP, A, next_)                                                   \
-        if constexpr (MJ == 16) { WREG_NEXT_EIGHT(WREG_GROUP, A, next_) }                  \
     }
-    static_assert(MJ == 8 || MJ == 16, "the groups of a half are written out");
+    static_assert(MJ == 8, "the groups of a half are written out");
 
     // (The host gives every split of K at least one step.  Without this line the compiler builds a path
     // for no steps on which the ring's registers are written while the first loads are in flight.)
@@ -512,18 +512,17 @@ __global__ __launch_bounds__(256) void gemm_wreg_kernel(const T* __restrict__ X,
     // those of W's first half of step s + 2, at its end those of the second half.  Step s needs X of step
     // s + 1 (its second half reads ahead into it) and its own W: all but the 2 NI loads issued last.
     v8 ring[SLOTS][NI];
-    static_assert(PER_WAVE + 2 * NI <= 63 && 2 * NI <= 15, "the waits' counts");
+    static_assert(PER_WAVE + 2 * NI <= 15, "the waits' counts");
     fill(0, 0);
     fetch_w(0, ring[0]);
     fetch_w(1, ring[1]);
     fill(1, STAGE);
     fetch_w(2, ring[2]);
     fetch_w(3, ring[3]);
-    // X of step 0 has landed (the count's upper two bits are bits 14 and 15 of the instruction's field)
-    __builtin_amdgcn_s_waitcnt(0x0F70 | ((PER_WAVE + 2 * NI) & 15) | (((PER_WAVE + 2 * NI) >> 4) << 14));
+    // X of step 0 has landed
+    __builtin_amdgcn_s_waitcnt(0x0F70 | (PER_WAVE + 2 * NI));
     __builtin_amdgcn_s_barrier();
     WREG_EIGHT(WREG_READ, lds_lane)
-    if constexpr (MJ == 16) { WREG_NEXT_EIGHT(WREG_READ, lds_lane) }
     int cur = 0;                                                   // byte offset of the buffer of step s
     for (int s = 0; s < n_steps; s += 2) {
 #pragma unroll
@@ -533,9 +532,8 @@ __global__ __launch_bounds__(256) void gemm_wreg_kernel(const T* __restrict__ X,
                 const int free_buf = nxt == (XBUFS - 1) * STAGE ? 0 : nxt + STAGE;
                 // X of step s + 1 and W of step s have landed (all but the 2 NI loads issued last), and this
                 // wave's reads of the buffer that is filled next are done (all but the MJ issued last, which
-                // read the buffer of this step; the field holds 15 at most); the barrier publishes the one
-                // and frees the other
-                __builtin_amdgcn_s_waitcnt(0x0070 | ((MJ < 15 ? MJ : 15) << 8) | (2 * NI));
+                // read the buffer of this step); the barrier publishes the one and frees the other
+                __builtin_amdgcn_s_waitcnt(0x0070 | (MJ << 8) | (2 * NI));
                 __builtin_amdgcn_s_barrier();
                 fill(s + u + 2, free_buf);
                 __builtin_amdgcn_sched_barrier(0);
@@ -550,7 +548,6 @@ __global__ __launch_bounds__(256) void gemm_wreg_kernel(const T* __restrict__ X,
         }
     }
 #undef WREG_HALF
-#undef WREG_NEXT_EIGHT
 #undef WREG_EIGHT
 #undef WREG_GROUP
 #undef WREG_READ
@@ -731,8 +728,7 @@ extern "C" int li_gemm_big(const void* X, const void* W, int tiled, int dt, void
 }
 
 // tile (rows of W x rows of X): 0 = 128 x 128, 1 = 256 x 128, 2 = 256 x 256 with 8 waves: gemm_dma, K in steps
-// of 32; 3 = 256 x 128, 4 = 192 x 128, 5 = 128 x 128, 6 = 256 x 256: gemm_wreg, K (and every split of it) a
-// multiple of 64.
+// of 32; 3 = 256 x 128, 4 = 192 x 128, 5 = 128 x 128: gemm_wreg, K (and every split of it) a multiple of 64.
 // W tiled.  The launch computes the columns n_begin .. n_begin + n_count - 1 of the product
 // (n_begin a multiple of 16; n_count 0: all from n_begin on), so that a product whose tiles do not
 // fill the last round of workgroups can finish with a smaller tile; K is split only for all columns.
@@ -743,13 +739,13 @@ extern "C" int li_gemm_dma(const void* X, const void* Wt, int dt, void* C, int o
     if (rc) return rc;
     if (dt != DT_F16 && dt != DT_BF16) return LI_BAD_ARG;
     if (K % 32 != 0 || ((uintptr_t)X & 15) || ((uintptr_t)Wt & 15)) return LI_UNSUPPORTED;
-    if (tile < 0 || tile > 6) return LI_BAD_ARG;
+    if (tile < 0 || tile > 5) return LI_BAD_ARG;
     if ((int64_t)M * K * 2 >= ((int64_t)1 << 32)) return LI_UNSUPPORTED;     // 32-bit offsets into X
     if (splits < 1 || (splits > 1 && !ws)) return LI_BAD_ARG;
     if (n_begin < 0 || n_begin >= N || (n_begin & 15) || n_count < 0 || n_begin + n_count > N) return LI_BAD_ARG;
     if (n_count == 0) n_count = N - n_begin;
-    // tiles 0 to 2: gemm_dma; 3 to 6: gemm_wreg
-    static const int tile_bn[7] = {128, 256, 256, 256, 192, 128, 256}, tile_bm[7] = {128, 128, 256, 128, 128, 128, 256};
+    // tiles 0 to 2: gemm_dma; 3 to 5: gemm_wreg
+    static const int tile_bn[6] = {128, 256, 256, 256, 192, 128}, tile_bm[6] = {128, 128, 256, 128, 128, 128};
     const int bn = tile_bn[tile], bm = tile_bm[tile], bk = tile >= 3 ? 64 : 32;
     if (K % bk != 0) return LI_UNSUPPORTED;                                  // gemm_wreg steps by 64 of K
     if (n_begin + n_count < N && n_count % bn != 0) return LI_BAD_ARG;       // only the last columns may end inside a tile
@@ -770,25 +766,18 @@ extern "C" int li_gemm_dma(const void* X, const void* Wt, int dt, void* C, int o
         // the kernels of one epilogue: the residual sum into float32 with whole quads of columns; the
         // rotation with a table of angles
         const int one = splits > 1 ? -1 : (mode == EPI_ADD && N % 4 == 0) ? EPI_ADD : (mode == EPI_ROPE && e.rs.cos_sin) ? EPI_ROPE : -1;
-#define WGO(T, NI, MJ, MODE)                                                                            \
-    do {                                                                                               \
-        auto kfn = gemm_wreg_kernel<T, NI, MJ, MODE>;                                                  \
-        if (wlds > 65536 && hipFuncSetAttribute((const void*)kfn, hipFuncAttributeMaxDynamicSharedMemorySize, (int)wlds) != hipSuccess) \
-            return LI_HIP_ERROR;                                                                       \
-        kfn<<<grid, block, wlds, stream>>>((const T*)X, (const T*)Wt, K, k_per_split, ws, n_begin, e);  \
+#define WGO(T, NI, MODE) gemm_wreg_kernel<T, NI, MODE><<<grid, block, wlds, stream>>>((const T*)X, (const T*)Wt, K, k_per_split, ws, n_begin, e)
+#define WMODE(T, NI)                                 \
+    do {                                             \
+        if (one == EPI_ADD) WGO(T, NI, EPI_ADD);     \
+        else if (one == EPI_ROPE) WGO(T, NI, EPI_ROPE); \
+        else WGO(T, NI, -1);                         \
     } while (0)
-#define WMODE(T, NI, MJ)                                 \
-    do {                                                 \
-        if (one == EPI_ADD) WGO(T, NI, MJ, EPI_ADD);     \
-        else if (one == EPI_ROPE) WGO(T, NI, MJ, EPI_ROPE); \
-        else WGO(T, NI, MJ, -1);                         \
-    } while (0)
-#define WLAUNCH(T)                               \
-    do {                                         \
-        if (tile == 3) WMODE(T, 4, 8);           \
-        else if (tile == 4) WMODE(T, 3, 8);      \
-        else if (tile == 5) WMODE(T, 2, 8);      \
-        else WMODE(T, 4, 16);                    \
+#define WLAUNCH(T)                           \
+    do {                                     \
+        if (tile == 3) WMODE(T, 4);          \
+        else if (tile == 4) WMODE(T, 3);     \
+        else WMODE(T, 2);                    \
     } while (0)
         if (dt == DT_F16) WLAUNCH(f16); else WLAUNCH(bf16);
 #undef WLAUNCH

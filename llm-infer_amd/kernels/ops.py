@@ -337,7 +337,7 @@ def _run_dma(x, wd, out, out_dt, mode, m, n, k, n_out, plan, rope) -> None:
     for tile, splits, n_begin, n_count, m_begin, m_count in plan:
         rows = m_count or m - m_begin
         _need(0 <= m_begin < m and m_begin + rows <= m, "gemm_dma: rows outside the product")
-        _need(tile < 3 or k % 64 == 0, "gemm_wreg (tiles 3 to 6): K must be a multiple of 64")
+        _need(tile < 3 or k % 64 == 0, "gemm_wreg (tiles 3 to 5): K must be a multiple of 64")
         ws = _workspace(splits * rows * n, x.device) if splits > 1 else None
         xp = c_void_p(x.data_ptr() + m_begin * k * x.element_size())
         op = c_void_p(out.data_ptr() + m_begin * n_out * out.element_size()) if out is not None else c_void_p(0)
@@ -371,16 +371,15 @@ def _stream_shape(n: int, k: int) -> tuple[int, int]:
     return 1, splits_for(g1)
 
 
-# rows of W x rows of X of a workgroup.  Tiles 0 to 2 are gemm_dma (W and X through LDS), 3 to 6
+# rows of W x rows of X of a workgroup.  Tiles 0 to 2 are gemm_dma (W and X through LDS), 3 to 5
 # gemm_wreg (W from memory into registers, X through LDS; K in steps of 64).
-_DMA_TILES = {0: (128, 128), 1: (256, 128), 2: (256, 256), 3: (256, 128), 4: (192, 128), 5: (128, 128), 6: (256, 256)}
+_DMA_TILES = {0: (128, 128), 1: (256, 128), 2: (256, 256), 3: (256, 128), 4: (192, 128), 5: (128, 128)}
 # Microseconds that one round of workgroups takes, measured on MI355X, as (a, c): a K / 4096 + c.  Entry i
-# is a round with i + 1 workgroups on every CU.  gemm_dma and the largest tile of gemm_wreg run one a CU;
-# of the other tiles of gemm_wreg two or three share a CU, and those of a last round that is less full run
-# at the shorter time.
+# is a round with i + 1 workgroups on every CU.  gemm_dma runs one a CU; of gemm_wreg two or three share a
+# CU, and those of a last round that is less full run at the shorter time.
 _DMA_ROUND_US = {0: ((48.0, 0.0),), 1: ((72.0, 0.0),), 2: ((124.0, 0.0),),
                  3: ((53.0, 9.0), (103.0, 5.0)), 4: ((35.0, 13.0), (73.0, 12.0)),
-                 5: ((31.4, 3.4), (57.1, 3.8), (89.0, 0.0)), 6: ((104.0, 14.0),)}
+                 5: ((31.4, 3.4), (57.1, 3.8), (89.0, 0.0))}
 
 
 def _dma_cost(tile: int, splits: int, m: int, n: int, k: int) -> float:
@@ -409,7 +408,7 @@ def _dma_plan(m: int, n: int, k: int) -> list:
     one per CU, and a last round that is nearly empty costs as much as a full one: a product of many
     rounds may get its large tile for as many columns (or, if that fits better, rows) as fill whole
     rounds and a smaller tile for the rest, if that is clearly faster by the same estimate."""
-    tiles = (2, 1, 0, 3, 4, 5, 6) if k % 64 == 0 else (2, 1, 0)            # gemm_wreg steps by 64 of K
+    tiles = (2, 1, 0, 3, 4, 5) if k % 64 == 0 else (2, 1, 0)            # gemm_wreg steps by 64 of K
     options = [(t, s) for t in tiles for s in (1, 2, 3, 4, 6, 8, 12, 16) if s == 1 or k // s >= 1024]
     tile, splits = min(options, key=lambda o: (_dma_cost(o[0], o[1], m, n, k), o[1], -o[0]))
     plan, cost = [(tile, splits, 0, 0, 0, 0)], _dma_cost(tile, splits, m, n, k)
