@@ -11,7 +11,6 @@
 //               LDS, optional split over K into a float32 workspace.
 //   gemv_mfma   up to 16 rows of X (row-major W), gemv_tiled up to 64 rows (tiled W): W is
 //               streamed once from HBM straight into the matrix cores' operand registers.
-//   gemm_stream 17 to 128 rows of X against a tiled W, X shared through LDS.
 #include "gemm_common.h"
 
 // ===========================================================================
@@ -453,125 +452,6 @@ __global__ __launch_bounds__(64 * KW) void gemv_tiled_kernel(const T* __restrict
 }
 
 // ===========================================================================
-// gemm_stream: 17 to 128 rows of X against a tiled W.  Such a product reads W once and is
-// bound by that read, but has too many rows of X to fetch them per wave: the 4 waves of a
-// workgroup own different rows of W (NT tiles of 16 each) and one share of K, and the X
-// slice of that share goes through LDS, 128 elements of K a stage, in the order
-// [k/8][row][8] that operand B reads without bank conflicts.  W travels global ->
-// registers -> operand A, two stages ahead of the matrix cores (three register sets), X
-// global -> registers -> the other LDS buffer one stage ahead; one barrier a stage.  K is split over
-// blockIdx.y where the rows of W alone cannot fill the chip; the partials are summed in
-// split order by splitk_reduce_kernel.
-// ===========================================================================
-template <class T, int NT, int MT>
-__global__ __launch_bounds__(256, 2) void gemm_stream_kernel(const T* __restrict__ X, const T* __restrict__ Wt,
-                                                             int K, int k_per_split, float* __restrict__ ws,
-                                                             Epilogue e) {
-    typedef typename Vec<T>::v8 v8;
-    constexpr int KC = 128, KS = KC / 32;                // elements of K and matrix steps per stage
-    constexpr int MP = MT * 16 + 1;                      // rows per k/8 group, padded: conflict-free stores
-    constexpr int BUF = (KC / 8) * MP;                   // 16-byte units of one buffer
-    extern __shared__ __attribute__((aligned(16))) unsigned char smem_raw[];
-    v8* sx = (v8*)smem_raw;
-
-    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-    const int r = lane & 15, g = lane >> 4;
-    const int n_tiles = (e.N + 15) >> 4;
-    const int steps = K >> 5;
-    const int tile0 = (blockIdx.x * 4 + wave) * NT;
-    const int kb = blockIdx.y * k_per_split, ke = min(K, kb + k_per_split);
-
-    const T* wt[NT];
-#pragma unroll
-    for (int t = 0; t < NT; ++t) wt[t] = Wt + ((int64_t)min(tile0 + t, n_tiles - 1) * steps * 64 + lane) * 8;
-    // this thread's 16-byte pieces of a stage of X: column group tid % 16 of rows tid / 16 + 16 i
-    const int xk8 = tid & 15, xrow0 = tid >> 4;
-    const T* xp[MT];
-#pragma unroll
-    for (int i = 0; i < MT; ++i) xp[i] = X + (int64_t)min(xrow0 + 16 * i, e.M - 1) * K + xk8 * 8;
-
-    f32x4 acc[NT][MT];
-#pragma unroll
-    for (int t = 0; t < NT; ++t)
-#pragma unroll
-        for (int j = 0; j < MT; ++j) acc[t][j] = f32x4{0.f, 0.f, 0.f, 0.f};
-
-    // Three register sets for W: the loads of stage s + 2 are issued before stage s is multiplied,
-    // so two stages are in flight per wave.  Loads are unconditional, from addresses clamped into
-    // this workgroup's share (the waits the compiler places then count exactly); what lies beyond
-    // the share of K is never multiplied, rows of X beyond M are zeroed on their way into LDS.
-    v8 ra[3][NT][KS], rx[MT];
-    const int s_last = (ke >> 5) - 1;
-    auto fetch_w = [&](int k0, v8 (&a)[NT][KS]) {
-        const int s0 = k0 >> 5;
-#pragma unroll
-        for (int t = 0; t < NT; ++t)
-#pragma unroll
-            for (int u = 0; u < KS; ++u) a[t][u] = *(const v8*)(wt[t] + (int64_t)min(s0 + u, s_last) * 512);
-    };
-    auto fetch_x = [&](int k0) {
-#pragma unroll
-        for (int i = 0; i < MT; ++i) rx[i] = *(const v8*)(xp[i] + max(0, min(k0, K - 8 - xk8 * 8)));
-    };
-    auto stash = [&](int buf) {
-        const v8 z = {};
-#pragma unroll
-        for (int i = 0; i < MT; ++i) sx[buf * BUF + xk8 * MP + xrow0 + 16 * i] = (xrow0 + 16 * i < e.M) ? rx[i] : z;
-    };
-    auto multiply = [&](int k0, int buf, v8 (&a)[NT][KS]) {
-        const int live = min(KS, (ke - k0) >> 5);
-#pragma unroll
-        for (int u = 0; u < KS; ++u) {
-            if (u < live) {
-                v8 b[MT];
-#pragma unroll
-                for (int j = 0; j < MT; ++j) b[j] = sx[buf * BUF + (4 * u + g) * MP + 16 * j + r];
-#pragma unroll
-                for (int t = 0; t < NT; ++t)
-#pragma unroll
-                    for (int j = 0; j < MT; ++j) acc[t][j] = mfma16(a[t][u], b[j], acc[t][j]);
-            }
-        }
-    };
-
-    fetch_w(kb, ra[0]);
-    fetch_x(kb);
-    fetch_w(kb + KC, ra[1]);
-    stash(0);
-    __syncthreads();
-    int buf = 0;
-    for (int k0 = kb; k0 < ke; k0 += 3 * KC) {
-#pragma unroll
-        for (int d = 0; d < 3; ++d) {
-            const int ks = k0 + d * KC;
-            if (ks >= ke) break;
-            fetch_x(ks + KC);
-            fetch_w(ks + 2 * KC, ra[(d + 2) % 3]);
-            __builtin_amdgcn_sched_barrier(0);
-            multiply(ks, buf, ra[d]);
-            stash(buf ^ 1);
-            __syncthreads();
-            buf ^= 1;
-        }
-    }
-
-    const bool split = gridDim.y > 1;
-#pragma unroll
-    for (int t = 0; t < NT; ++t)
-#pragma unroll
-        for (int j = 0; j < MT; ++j) {
-            const int m = 16 * j + r, n = (tile0 + t) * 16 + 4 * g;
-            float v[4] = {acc[t][j][0], acc[t][j][1], acc[t][j][2], acc[t][j][3]};
-            if (!split) epilogue4(e, m, n, v);
-            else if (m < e.M) {
-                float* p = ws + ((int64_t)blockIdx.y * e.M + m) * e.N + n;
-#pragma unroll
-                for (int q = 0; q < 4; ++q) if (n + q < e.N) p[q] = v[q];
-            }
-        }
-}
-
-// ===========================================================================
 // C interface
 // ===========================================================================
 extern "C" int li_gemm_fma(const void* X, int x_dt, const void* W, int w_dt, void* C, int out_dt, int mode,
@@ -744,55 +624,6 @@ extern "C" int li_gemv_tiled(const void* X, const void* Wt, int dt, void* C, int
 #undef PICK_KW
 #undef LAUNCH
     LI_CHECK_LAUNCH();
-    return LI_OK;
-}
-
-// 17..128 rows of X, W tiled.  nt: tiles of 16 rows of W per wave (1 or 2); ws: splits * M * N floats
-extern "C" int li_gemm_stream(const void* X, const void* Wt, int dt, void* C, int out_dt, int mode,
-                              int M, int N, int K, int nt, int splits, float* ws, const RopeStore* rs,
-                              hipStream_t stream) {
-    int rc = check_common(X, Wt, C, M, N, K, mode, out_dt);
-    if (rc) return rc;
-    if (dt != DT_F16 && dt != DT_BF16) return LI_BAD_ARG;
-    if (M > 128 || (nt != 1 && nt != 2)) return LI_BAD_ARG;
-    if (K % 32 != 0 || ((uintptr_t)X & 15) || ((uintptr_t)Wt & 15)) return LI_UNSUPPORTED;
-    if (splits < 1 || (splits > 1 && !ws)) return LI_BAD_ARG;
-    if (M == 0) return LI_OK;
-    Epilogue e;
-    rc = make_epilogue(e, C, mode, out_dt, M, N, rs);
-    if (rc) return rc;
-    const int mt = M <= 32 ? 2 : (M <= 64 ? 4 : 8);
-    const int kc = 128;
-    int k_per_split = ((K + splits - 1) / splits + kc - 1) / kc * kc;
-    splits = (K + k_per_split - 1) / k_per_split;
-    const int n_tiles = (N + 15) / 16;
-    dim3 grid((n_tiles + 4 * nt - 1) / (4 * nt), splits), block(256);
-    const size_t lds = (size_t)2 * (kc / 8) * (mt * 16 + 1) * 16;
-#define GO(T, NT, MT)                                                                                  \
-    do {                                                                                               \
-        auto kfn = gemm_stream_kernel<T, NT, MT>;                                                      \
-        if (hipFuncSetAttribute((const void*)kfn, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds) != hipSuccess) \
-            return LI_HIP_ERROR;                                                                       \
-        kfn<<<grid, block, lds, stream>>>((const T*)X, (const T*)Wt, K, k_per_split, ws, e);           \
-    } while (0)
-#define PICK(T)                                        \
-    do {                                               \
-        if (nt == 1 && mt == 2) GO(T, 1, 2);           \
-        else if (nt == 1 && mt == 4) GO(T, 1, 4);      \
-        else if (nt == 1) GO(T, 1, 8);                 \
-        else if (mt == 2) GO(T, 2, 2);                 \
-        else if (mt == 4) GO(T, 2, 4);                 \
-        else GO(T, 2, 8);                              \
-    } while (0)
-    if (dt == DT_F16) PICK(f16); else PICK(bf16);
-#undef PICK
-#undef GO
-    LI_CHECK_LAUNCH();
-    if (splits > 1) {
-        const int64_t quads = (int64_t)M * ((N + 3) / 4);
-        splitk_reduce_kernel<<<(unsigned)((quads + 255) / 256), 256, 0, stream>>>(ws, splits, e);
-        LI_CHECK_LAUNCH();
-    }
     return LI_OK;
 }
 

@@ -243,9 +243,8 @@ def linear(x: torch.Tensor, w, mode: int = EPI_STORE, out: torch.Tensor | None =
     kind = force or ("fma" if not fast_ok else ("gemv_mfma" if m <= 16 else ("big" if m > 32 else "mfma")))
     if tiled:
         _need(fast_ok and kind != "fma", "a tiled weight needs 16-bit activations of its dtype")
-        # up to 16 rows (32 for a small matrix) every wave fetches the rows of X itself; up to 96
-        # rows (128 against a matrix of many rows) they go through LDS once per workgroup; beyond
-        # that the tiled GEMM is faster
+        # up to 16 rows (32 for a small matrix) every wave fetches the rows of X itself; beyond that
+        # the tiled GEMM is faster
         if kind == "gemv_mfma" or (force is None and (m <= 16 or (m <= 32 and n * k <= (1 << 25)))):
             ro = rsc = None
             nxt = getattr(out, "_li_next_norm", None) if mode == EPI_ADD else None
@@ -266,18 +265,8 @@ def linear(x: torch.Tensor, w, mode: int = EPI_STORE, out: torch.Tensor | None =
                 out._li_rows = (xw, ss, scale, nxt, out._version)
             return out
         _need(lazy is None, "a norm is finished by gemv_tiled alone")
-        if force is None and (m <= 96 or (m <= 128 and n >= 16384)):
-            kind = "stream"
-        elif force is None and m * k * 2 < (1 << 32):
+        if force is None and m * k * 2 < (1 << 32):
             kind = "dma"
-    if kind.startswith("stream"):
-        _need(tiled and fast_ok and m <= 128, "gemm_stream: a tiled weight and at most 128 rows")
-        parts = kind.split(":")
-        nt, splits = (int(parts[1]), int(parts[2])) if len(parts) > 2 else _stream_shape(n, k)
-        ws = _workspace(splits * m * n, x.device) if splits > 1 else None
-        _check(lib.li_gemm_stream(_ptr(x), _ptr(wd), DT[x.dtype], _ptr(out), out_dt, mode, m, n, k, nt, splits,
-                                  _ptr(ws), rs, _stream()), "gemm_stream")
-        return out
     if kind.startswith("dma"):
         _need(tiled and fast_ok and m * k * 2 < (1 << 32), "gemm_dma: a tiled weight, X below 4 GiB")
         _run_dma(x, wd, out, out_dt, mode, m, n, k, n_out, _forced_dma_plan(kind) or _dma_plan(m, n, k), _rope)
@@ -353,22 +342,6 @@ def _run_dma(x, wd, out, out_dt, mode, m, n, k, n_out, plan, rope) -> None:
             rp = ctypes.byref(shifted)
         _check(lib.li_gemm_dma(xp, _ptr(wd), DT[x.dtype], op, out_dt, mode, rows, n, k, tile, splits,
                                _ptr(ws), rp, n_begin, n_count, _stream()), "gemm_dma")
-
-
-def _stream_shape(n: int, k: int) -> tuple[int, int]:
-    """Tiles of W per wave and splits of K for gemm_stream (measured on MI355X): two tiles per
-    wave halve the traffic of X if that still leaves a workgroup for most of the 256 CUs; K is
-    split down to 1024 elements per workgroup to get there."""
-    def splits_for(groups):
-        want = max(1, 256 // groups)
-        want = 1 << (want.bit_length() - 1)
-        return max(1, min(want, k // 1024, 16))
-    g2 = -(-n // 128)
-    s2 = splits_for(g2)
-    if g2 * s2 >= 192:
-        return 2, s2
-    g1 = -(-n // 64)
-    return 1, splits_for(g1)
 
 
 # rows of W x rows of X of a workgroup.  Tiles 0 to 2 are gemm_dma (W and X through LDS), 3 to 5

@@ -136,8 +136,6 @@ def test_linear_tiled_weights(ops, M, N, K, dt):
     # and the first rows with one tile, the rest with another
     kinds += [f"dmarows:{a}:{r}:{b}" for a, r, b in ((2, 256, 0), (1, 128, 0), (0, 128, 2), (3, 128, 5), (5, 128, 4))
               if r < M and (wreg or max(a, b) < 3)]
-    if M <= 128:
-        kinds += ["stream", "stream:1:1", "stream:2:1", "stream:1:3", "stream:2:16"]
     for kind in kinds:
         for mode in (0, 1, 2, 4):
             if mode in (2, 4) and N % 2:
@@ -531,7 +529,7 @@ def test_rotation_fused_into_the_projection(ops, dt, T, H, K, hd, rot, d):
             continue
         ww = ops.tile_weight(w) if tiled else w
         wreg = ["dma:3", "dma:4:2", "dma:5"] if d % 64 == 0 else []
-        for kind in kinds + ((["dma:0", "dma:1:2", "dma:2"] + wreg + (["dma2:0:128:1"] + (["dma2:5:128:3"] if wreg else []) if (H + 2 * K) * hd > 128 else []) + (["dmarows:0:128:1"] if T > 128 else []) + (["stream:1:1", "stream:2:2"] if T <= 128 else [])) if tiled else []):
+        for kind in kinds + ((["dma:0", "dma:1:2", "dma:2"] + wreg + (["dma2:0:128:1"] + (["dma2:5:128:3"] if wreg else []) if (H + 2 * K) * hd > 128 else []) + (["dmarows:0:128:1"] if T > 128 else [])) if tiled else []):
             if tiled and kind == "fma":
                 continue
             c1, v1 = fresh()
