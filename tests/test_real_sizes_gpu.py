@@ -2,9 +2,9 @@
 context, in 32-bit and in float16, under the three ways of cutting requests into steps.
 
 The tiny configurations never reach the code that serves real sizes: head size 128 with four query
-heads a KV head, a down projection with K = 14,336, products of 17 to 96 rows that split K, the
-prefill product's launch plans (several tiles, a plan of two launches over rows with the rotation in
-its epilogue), page tables beyond 128 pages, 64 splits of the decode attention, rotation angles at
+heads a KV head, a down projection with K = 14,336, products of 17 to 300 rows that split K, the
+prefill product's tiles (256, 192 and 128 rows of W, a last tile of rows that is partly empty, the
+kernels whose epilogue is the residual sum or the rotation alone), page tables beyond 128 pages, 64 splits of the decode attention, rotation angles at
 positions in the thousands.  Here they lie on a tested path: two layers of the Llama-3.1-8B layer
 shape, one layer of the Llama-2-7B shape (32 KV heads), and a small model with a request of 9,000
 tokens."""
@@ -36,7 +36,7 @@ CONFIGS = {
              "vocab_size": 300, "rope_theta": 500000.0, "rms_norm_eps": 1e-5, "max_position_embeddings": 16384,
              "tie_word_embeddings": True, "hidden_act": "silu", "torch_dtype": "float16"},
 }
-# 1,300 rows: the q/k/v product of the 7B layer runs as two launches over rows, each with the rotation
+# 1,300 rows: eleven tiles of rows, the last a fifth full; the 7B layer's q/k/v product takes the 192-row tile
 LENGTHS = {"8b": [1, 17, 64, 65, 300], "7b": [1, 17, 64, 65, 300, 1300], "long": [9000]}
 
 
