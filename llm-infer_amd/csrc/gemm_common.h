@@ -111,6 +111,16 @@ __device__ __forceinline__ void epilogue4(const Epilogue& e, int m, int n, const
     if (e.mode == EPI_SWIGLU || e.mode == EPI_GEGLU) {
         // columns 2j (gate) and 2j+1 (up) give h[m, j] = act(gate) * up   (src/model/block.cpp:203-214)
         const int64_t row = (int64_t)m * (e.N >> 1);
+        if (n + 3 < e.N && (e.N & 3) == 0) {
+            // both values of the quad in one store (the pair's index is even, and so is N / 2)
+            const float h0 = gate_activation(v[0], e.mode == EPI_GEGLU) * v[1];
+            const float h1 = gate_activation(v[2], e.mode == EPI_GEGLU) * v[3];
+            const int64_t at = row + (n >> 1);
+            if (e.out_dt == DT_F32) *(f32x2*)((float*)e.C + at) = f32x2{h0, h1};
+            else if (e.out_dt == DT_F16) *(f16x2*)((f16*)e.C + at) = f16x2{(f16)h0, (f16)h1};
+            else *(bf16x2*)((bf16*)e.C + at) = bf16x2{(bf16)h0, (bf16)h1};
+            return;
+        }
 #pragma unroll
         for (int j = 0; j < 4; j += 2) {
             if (n + j + 1 < e.N) {
