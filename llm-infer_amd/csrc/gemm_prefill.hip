@@ -1,5 +1,5 @@
-// The prefill products: more than 96 rows of X (gemm_dma against a tiled weight, gemm_big against
-// a row-major one).  Epilogues, layouts and the split-K reduction are in gemm_common.h.
+// The products of more than 16 rows of X: gemm_wreg against a tiled weight, gemm_big against a
+// row-major one.  Epilogues, layouts and the split-K reduction are in gemm_common.h.
 #include "gemm_common.h"
 
 __device__ __forceinline__ f32x4 mfma16(f16x8 a, f16x8 b, f32x4 c) {
@@ -202,187 +202,6 @@ __global__ __launch_bounds__(256) void gemm_big_kernel(const T* __restrict__ X, 
 }
 
 // ===========================================================================
-// gemm_dma: the prefill product against a tiled W, with both operands going from global
-// memory straight into LDS (global_load_lds, 16 bytes a lane): no staging registers, no
-// LDS store instructions.  A load instruction of a wave fills 1 KiB of LDS in lane order,
-// so a tile lies in LDS as units of 16 rows x 32 elements of K in the order of the tiled
-// weight, [lane = 16*((k%32)/8) + row%16][k%8]: a unit of W is copied as it lies in
-// memory, a unit of X is gathered by the lanes (16 rows, 64 contiguous bytes each).  A
-// fragment of the 32x32x16 instruction is read from two such units, 16 lanes a contiguous
-// 256 bytes, which is free of bank conflicts without padding.  BK = 32 (K of a tiled weight
-// is a multiple of 32, so no tile is cut in K); rows beyond M or N are read from clamped
-// addresses and dropped by the epilogue.  Three LDS buffers: the loads of tile t + 2 are
-// issued while tile t is multiplied; one barrier per tile.
-// ===========================================================================
-template <class T, int BN, int BM, int WAVES, int STAGES>
-__global__ __launch_bounds__(64 * WAVES) void gemm_dma_kernel(const T* __restrict__ X, const T* __restrict__ Wt,
-                                                          int K, int k_per_split, float* __restrict__ ws,
-                                                          int n_begin, Epilogue e) {
-    typedef typename Vec<T>::v8 v8;
-    constexpr int BK = 32;
-    constexpr int TN = BN / 2, TM = BM / (WAVES / 2), NB = TN / 32, MB = TM / 32;   // 2 waves along N
-    constexpr int WU = BN / 16, XU = BM / 16, UNITS = WU + XU;       // 1 KiB units of a stage
-    constexpr int PER_WAVE = UNITS / WAVES;
-    constexpr int STAGE = UNITS * 1024;                              // bytes
-    static_assert(UNITS % WAVES == 0, "units of a stage are dealt to the waves");
-    extern __shared__ __attribute__((aligned(16))) unsigned char smem_raw[];
-
-    const int tid = threadIdx.x, lane = tid & 63;
-    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);       // uniform: what depends on it stays scalar
-    const int wn = wave & 1, wm = wave >> 1;
-    int bx, by, bz;
-    tile_of_workgroup(BM == 256 ? 4 : 8, bx, by, bz);
-    const int m0 = bx * BM, n0 = n_begin + by * BN;                  // the grid covers rows n_begin.. of W
-    const int kb = bz * k_per_split, ke = min(K, kb + k_per_split);
-    const int n_tiles = (ke - kb) / BK;
-    const int w_blocks = (e.N + 15) >> 4, steps = K >> 5;
-
-    // Where the 16 bytes of this lane come from, for each of the wave's units: a base address that
-    // is the same for the whole wave and moves on by `step` bytes per tile of K, plus a 32-bit
-    // offset of the lane (the host checks that X has fewer than 4 GiB).
-    const unsigned char* base[PER_WAVE];
-    uint32_t lane_off[PER_WAVE];
-    int step[PER_WAVE];
-#pragma unroll
-    for (int i = 0; i < PER_WAVE; ++i) {
-        const int u = wave * PER_WAVE + i;
-        if (u < WU) {
-            const int blk = min(n0 / 16 + u, w_blocks - 1);
-            base[i] = (const unsigned char*)(Wt + ((int64_t)blk * steps + (kb >> 5)) * 512);
-            lane_off[i] = lane * 16;
-            step[i] = 1024;
-        } else {
-            const int row = min(m0 + 16 * (u - WU) + (lane & 15), e.M - 1);
-            base[i] = (const unsigned char*)(X + kb);
-            lane_off[i] = ((uint32_t)row * (uint32_t)K + 8 * (lane >> 4)) * 2;
-            step[i] = BK * 2;
-        }
-    }
-    auto issue = [&](int t, int buf) {
-#pragma unroll
-        for (int i = 0; i < PER_WAVE; ++i) {
-            const int u = wave * PER_WAVE + i;
-            __builtin_amdgcn_global_load_lds(
-                (const __attribute__((address_space(1))) void*)(base[i] + (int64_t)t * step[i] + lane_off[i]),
-                (__attribute__((address_space(3))) void*)(smem_raw + buf * STAGE + u * 1024), 16, 0, 0);
-        }
-    };
-
-    f32x16 acc[NB][MB];
-#pragma unroll
-    for (int a = 0; a < NB; ++a)
-#pragma unroll
-        for (int b = 0; b < MB; ++b)
-#pragma unroll
-            for (int r = 0; r < 16; ++r) acc[a][b][r] = 0.f;
-
-    // byte offset of this lane's piece of a fragment within its pair of units, for k-step 0
-    const int frag = ((lane & 31) >> 4) * 1024 + (16 * (lane >> 5) + (lane & 15)) * 16;
-    const unsigned char* sW = smem_raw + (wn * TN / 16) * 1024 + frag;
-    const unsigned char* sX = smem_raw + (WU + wm * TM / 16) * 1024 + frag;
-    auto read_frags = [&](int buf, int ks, v8 (&a)[NB], v8 (&b)[MB]) {
-#pragma unroll
-        for (int j = 0; j < MB; ++j) b[j] = *(const v8*)(sX + buf * STAGE + j * 2048 + ks * 512);
-#pragma unroll
-        for (int i = 0; i < NB; ++i) a[i] = *(const v8*)(sW + buf * STAGE + i * 2048 + ks * 512);
-    };
-    auto multiply = [&](const v8 (&a)[NB], const v8 (&b)[MB], int lo, int hi) {
-#pragma unroll
-        for (int i = 0; i < NB; ++i)
-            if (i >= lo && i < hi) {
-#pragma unroll
-                for (int j = 0; j < MB; ++j) acc[i][j] = mfma32(a[i], b[j], acc[i][j]);
-            }
-    };
-
-    // The loop works in half tiles (16 of the 32 elements of K): while the matrix cores work on
-    // one half, the fragments of the next are on their way from LDS.  In the middle of tile t every
-    // wave has read all of it, so the barrier there both publishes tile t + 1 and frees the buffer
-    // of tile t for the loads of tile t + STAGES: loads run STAGES - 1 tiles ahead.
-    // (A bare s_barrier: __syncthreads would also wait for the loads still in flight.)
-    // One copy of the body, the buffer a run-time offset: unrolled by the three buffers the
-    // register allocator spills.  After the last tile the reads for "the next tile" fetch stale
-    // data that nothing uses.
-    v8 a0[NB], b0[MB], a1[NB], b1[MB];
-    // waits until at most `tiles` of the tiles whose loads were issued last are still in flight
-    auto wait_tiles = [&](int tiles, bool lds_too) {
-        if (lds_too) {
-            if (tiles <= 0) __builtin_amdgcn_s_waitcnt(0x0070);
-            else if (tiles == 1) __builtin_amdgcn_s_waitcnt(0x0070 | PER_WAVE);
-            else if (tiles == 2) __builtin_amdgcn_s_waitcnt(0x0070 | (2 * PER_WAVE));
-            else __builtin_amdgcn_s_waitcnt(0x0070 | (3 * PER_WAVE));
-        } else {
-            if (tiles <= 0) __builtin_amdgcn_s_waitcnt(0x0F70);
-            else if (tiles == 1) __builtin_amdgcn_s_waitcnt(0x0F70 | PER_WAVE);
-            else if (tiles == 2) __builtin_amdgcn_s_waitcnt(0x0F70 | (2 * PER_WAVE));
-            else if (tiles == 3) __builtin_amdgcn_s_waitcnt(0x0F70 | (3 * PER_WAVE));
-            else __builtin_amdgcn_s_waitcnt(0x0F70 | (3 * PER_WAVE));
-        }
-    };
-    static_assert(STAGES >= 3 && STAGES <= 5 && (STAGES - 2) * PER_WAVE <= 15, "stages");
-#pragma unroll
-    for (int i = 0; i < STAGES; ++i)
-        if (i < n_tiles) issue(i, i);
-    wait_tiles(min(min(STAGES, n_tiles) - 1, 3), false);
-    __builtin_amdgcn_s_barrier();
-    read_frags(0, 0, a0, b0);
-    int cur = 0;
-#pragma unroll 1
-    for (int t = 0; t < n_tiles; ++t) {
-        const int nxt = cur == STAGES - 1 ? 0 : cur + 1;
-        // the second half's fragments are requested between the matrix instructions of the first
-        // half: requested before them, the wait the compiler places for the first half's fragments
-        // (it merges the loop's entry and back edge pessimistically) would cover these reads too
-        multiply(a0, b0, 0, NB / 2);
-        __builtin_amdgcn_sched_barrier(0);
-        read_frags(cur, 1, a1, b1);
-        __builtin_amdgcn_sched_barrier(0);
-        multiply(a0, b0, NB / 2, NB);
-        __builtin_amdgcn_sched_barrier(0);
-        // tile t + 1 has landed (up to STAGES - 2 later ones may be in flight); this wave's reads
-        // of tile t are done
-        wait_tiles(min(STAGES - 2, n_tiles - 2 - t), true);
-        __builtin_amdgcn_s_barrier();
-        if (t + STAGES < n_tiles) issue(t + STAGES, cur);
-        multiply(a1, b1, 0, NB / 2);
-        __builtin_amdgcn_sched_barrier(0);
-        read_frags(nxt, 0, a0, b0);
-        __builtin_amdgcn_sched_barrier(0);
-        multiply(a1, b1, NB / 2, NB);
-        __builtin_amdgcn_sched_barrier(0);
-        cur = nxt;
-    }
-    __syncthreads();
-    constexpr int SLD = 36;
-    float* stage = (float*)smem_raw + wave * (32 * SLD);
-#pragma unroll
-    for (int i = 0; i < NB; ++i)
-#pragma unroll
-        for (int j = 0; j < MB; ++j) {
-#pragma unroll
-            for (int g = 0; g < 4; ++g) {
-                f32x4 v = {acc[i][j][4 * g], acc[i][j][4 * g + 1], acc[i][j][4 * g + 2], acc[i][j][4 * g + 3]};
-                *(f32x4*)(stage + (lane & 31) * SLD + 8 * g + 4 * (lane >> 5)) = v;
-            }
-            __builtin_amdgcn_wave_barrier();
-            const int mb = m0 + wm * TM + j * 32, nb = n0 + wn * TN + i * 32;
-#pragma unroll 1
-            for (int q = lane; q < 256; q += 64) {
-                const int r = q >> 3, c = (q & 7) * 4;
-                const f32x4 v = *(const f32x4*)(stage + r * SLD + c);
-                const float vv[4] = {v[0], v[1], v[2], v[3]};
-                if (gridDim.z == 1) epilogue4(e, mb + r, nb + c, vv);
-                else if (mb + r < e.M) {
-                    float* p = ws + ((int64_t)bz * e.M + mb + r) * e.N + nb + c;
-#pragma unroll
-                    for (int jj = 0; jj < 4; ++jj) if (nb + c + jj < e.N) p[jj] = vv[jj];
-                }
-            }
-            __builtin_amdgcn_wave_barrier();
-        }
-}
-
-// ===========================================================================
 // gemm_wreg: the prefill product against a tiled W with W never in LDS.  A tiled weight lies in memory
 // in the order in which the 16x16x32 matrix instruction takes operand A, so a wave loads its fragments of
 // W straight from global memory into a ring of registers (1 KiB contiguous a load: 8 whole lines) and only
@@ -402,8 +221,7 @@ __global__ __launch_bounds__(64 * WAVES) void gemm_dma_kernel(const T* __restric
 // epilogue, chosen at run time.
 template <class T, int NI, int MODE>
 __global__ __launch_bounds__(256) void gemm_wreg_kernel(const T* __restrict__ X, const T* __restrict__ Wt,
-                                                        int K, int k_per_split, float* __restrict__ ws,
-                                                        int n_begin, Epilogue e) {
+                                                        int K, int k_per_split, float* __restrict__ ws, Epilogue e) {
     typedef typename Vec<T>::v8 v8;
     // A step is 64 of K: two halves of 32, each one matrix instruction deep.
     // MJ: fragments of X (16 rows each) per wave and half step; every wave takes all the tile's rows of X
@@ -417,9 +235,10 @@ __global__ __launch_bounds__(256) void gemm_wreg_kernel(const T* __restrict__ X,
     const int wn = wave;
     int bx, by, bz;
     tile_of_workgroup(8, bx, by, bz);
-    const int m0 = bx * BM, n0 = n_begin + by * BN;
+    const int m0 = bx * BM, n0 = by * BN;
     const int kb = bz * k_per_split, ke = min(K, kb + k_per_split);
-    const int n_halves = (ke - kb) >> 5, n_steps = n_halves >> 1;       // the host: K and the splits are multiples of 64
+    // a share of K that is 32 more than a multiple of 64 ends with a step of one half
+    const int n_halves = (ke - kb) >> 5, n_steps = (n_halves + 1) >> 1;
     const int w_blocks = (e.N + 15) >> 4, steps = K >> 5;
 
     // this wave's rows of W: NI blocks of 16, each a run of 1 KiB units along K
@@ -444,14 +263,19 @@ __global__ __launch_bounds__(256) void gemm_wreg_kernel(const T* __restrict__ X,
     }
     // Loads past the last step of K are not branched around: they fetch the last step again (into a buffer
     // and registers that nothing reads), which keeps the count of loads in flight fixed.
+    // In a last step of one half the lanes whose chunk lies in the second half fetch the first half's
+    // chunk again (the row may end there); nothing reads what they bring.
     const int last = n_halves - 1;
+    const uint32_t odd_back = ((n_halves & 1) && ((lane & 7) ^ (lane >> 3)) >= 4) ? 64 : 0;
     auto fill = [&](int s, int buf_off) {
-        const int64_t at = (int64_t)min(s, n_steps - 1) * 128;
+        const int st = min(s, n_steps - 1);
+        const int64_t at = (int64_t)st * 128;
+        const uint32_t back = st == n_steps - 1 ? odd_back : 0;
 #pragma unroll
         for (int i = 0; i < PER_WAVE; ++i) {
             const int q = wave * PER_WAVE + i;
             __builtin_amdgcn_global_load_lds(
-                (const __attribute__((address_space(1))) void*)(xbase + at + xoff[i]),
+                (const __attribute__((address_space(1))) void*)(xbase + at + (xoff[i] - back)),
                 (__attribute__((address_space(3))) void*)(smem_raw + buf_off + q * 1024), 16, 0, 0);
         }
     };
@@ -540,7 +364,7 @@ __global__ __launch_bounds__(256) void gemm_wreg_kernel(const T* __restrict__ X,
                 WREG_HALF(ring[2 * u], lds_lane2 + cur)
                 fetch_w(2 * (s + u + 2), ring[2 * u]);
                 __builtin_amdgcn_sched_barrier(0);
-                WREG_HALF(ring[2 * u + 1], lds_lane + nxt)
+                if (2 * (s + u) + 1 < n_halves) WREG_HALF(ring[2 * u + 1], lds_lane + nxt)
                 fetch_w(2 * (s + u + 2) + 1, ring[2 * u + 1]);
                 __builtin_amdgcn_sched_barrier(0);
                 cur = nxt;
@@ -727,85 +551,49 @@ extern "C" int li_gemm_big(const void* X, const void* W, int tiled, int dt, void
     return LI_OK;
 }
 
-// tile (rows of W x rows of X): 0 = 128 x 128, 1 = 256 x 128, 2 = 256 x 256 with 8 waves: gemm_dma, K in steps
-// of 32; 3 = 256 x 128, 4 = 192 x 128, 5 = 128 x 128: gemm_wreg, K (and every split of it) a multiple of 64.
-// W tiled.  The launch computes the columns n_begin .. n_begin + n_count - 1 of the product
-// (n_begin a multiple of 16; n_count 0: all from n_begin on), so that a product whose tiles do not
-// fill the last round of workgroups can finish with a smaller tile; K is split only for all columns.
-extern "C" int li_gemm_dma(const void* X, const void* Wt, int dt, void* C, int out_dt, int mode,
-                           int M, int N, int K, int tile, int splits, float* ws, const RopeStore* rs,
-                           int n_begin, int n_count, hipStream_t stream) {
+// tile (rows of W x rows of X): 0 = 256 x 128, 1 = 192 x 128, 2 = 128 x 128.  W tiled (K a multiple of 32),
+// X below 4 GiB (the kernel addresses it with 32-bit offsets); ws: splits * M * N floats when K is split.
+extern "C" int li_gemm_wreg(const void* X, const void* Wt, int dt, void* C, int out_dt, int mode,
+                            int M, int N, int K, int tile, int splits, float* ws, const RopeStore* rs,
+                            hipStream_t stream) {
     int rc = check_common(X, Wt, C, M, N, K, mode, out_dt);
     if (rc) return rc;
     if (dt != DT_F16 && dt != DT_BF16) return LI_BAD_ARG;
     if (K % 32 != 0 || ((uintptr_t)X & 15) || ((uintptr_t)Wt & 15)) return LI_UNSUPPORTED;
-    if (tile < 0 || tile > 5) return LI_BAD_ARG;
-    if ((int64_t)M * K * 2 >= ((int64_t)1 << 32)) return LI_UNSUPPORTED;     // 32-bit offsets into X
+    if (tile < 0 || tile > 2) return LI_BAD_ARG;
+    if ((int64_t)M * K * 2 >= ((int64_t)1 << 32)) return LI_UNSUPPORTED;
     if (splits < 1 || (splits > 1 && !ws)) return LI_BAD_ARG;
-    if (n_begin < 0 || n_begin >= N || (n_begin & 15) || n_count < 0 || n_begin + n_count > N) return LI_BAD_ARG;
-    if (n_count == 0) n_count = N - n_begin;
-    // tiles 0 to 2: gemm_dma; 3 to 5: gemm_wreg
-    static const int tile_bn[6] = {128, 256, 256, 256, 192, 128}, tile_bm[6] = {128, 128, 256, 128, 128, 128};
-    const int bn = tile_bn[tile], bm = tile_bm[tile], bk = tile >= 3 ? 64 : 32;
-    if (K % bk != 0) return LI_UNSUPPORTED;                                  // gemm_wreg steps by 64 of K
-    if (n_begin + n_count < N && n_count % bn != 0) return LI_BAD_ARG;       // only the last columns may end inside a tile
-    if (splits > 1 && n_count != N) return LI_BAD_ARG;
     if (M == 0) return LI_OK;
     Epilogue e;
     rc = make_epilogue(e, C, mode, out_dt, M, N, rs);
     if (rc) return rc;
-    const size_t lds = (size_t)3 * (bn + bm) / 16 * 1024;
+    const int bn = 256 - 64 * tile, bm = 128, bk = 32;
     int k_per_split = ((K + splits - 1) / splits + bk - 1) / bk * bk;
     splits = (K + k_per_split - 1) / k_per_split;
-    dim3 grid((M + bm - 1) / bm, (n_count + bn - 1) / bn, splits), block(tile == 2 ? 512 : 256);
-    if (tile >= 3) {
-        // three stages of X; the epilogue stages two strips of 16 x (bn / 4 + 4) floats a wave in the same LDS, and
-        // behind both lie a position and a page for each of the tile's rows
-        const size_t stages = (size_t)3 * 2 * (bm / 16) * 1024, strips = (size_t)4 * 2 * 16 * (bn / 4 + 4) * 4;   // (a step is 64 of K)
-        const size_t wlds = (stages > strips ? stages : strips) + (size_t)2 * bm * 4;
-        // the kernels of one epilogue: the residual sum into float32 with whole quads of columns; the
-        // rotation with a table of angles
-        const int one = splits > 1 ? -1 : (mode == EPI_ADD && N % 4 == 0) ? EPI_ADD : (mode == EPI_ROPE && e.rs.cos_sin) ? EPI_ROPE : -1;
-#define WGO(T, NI, MODE) gemm_wreg_kernel<T, NI, MODE><<<grid, block, wlds, stream>>>((const T*)X, (const T*)Wt, K, k_per_split, ws, n_begin, e)
-#define WMODE(T, NI)                                 \
-    do {                                             \
-        if (one == EPI_ADD) WGO(T, NI, EPI_ADD);     \
-        else if (one == EPI_ROPE) WGO(T, NI, EPI_ROPE); \
-        else WGO(T, NI, -1);                         \
+    dim3 grid((M + bm - 1) / bm, (N + bn - 1) / bn, splits), block(256);
+    // three stages of X (a step is 64 of K); the epilogue stages two strips of 16 x (bn / 4 + 4) floats a wave
+    // in the same LDS, and behind both lie a position and a page for each of the tile's rows
+    const size_t stages = (size_t)3 * 2 * (bm / 16) * 1024, strips = (size_t)4 * 2 * 16 * (bn / 4 + 4) * 4;
+    const size_t lds = (stages > strips ? stages : strips) + (size_t)2 * bm * 4;
+    // the kernels of one epilogue: the residual sum into float32 with whole quads of columns; the
+    // rotation with a table of angles
+    const int one = splits > 1 ? -1 : (mode == EPI_ADD && N % 4 == 0) ? EPI_ADD : (mode == EPI_ROPE && e.rs.cos_sin) ? EPI_ROPE : -1;
+#define GO(T, NI, MODE) gemm_wreg_kernel<T, NI, MODE><<<grid, block, lds, stream>>>((const T*)X, (const T*)Wt, K, k_per_split, ws, e)
+#define BY_MODE(T, NI)                              \
+    do {                                            \
+        if (one == EPI_ADD) GO(T, NI, EPI_ADD);     \
+        else if (one == EPI_ROPE) GO(T, NI, EPI_ROPE); \
+        else GO(T, NI, -1);                         \
     } while (0)
-#define WLAUNCH(T)                           \
+#define LAUNCH(T)                            \
     do {                                     \
-        if (tile == 3) WMODE(T, 4);          \
-        else if (tile == 4) WMODE(T, 3);     \
-        else WMODE(T, 2);                    \
-    } while (0)
-        if (dt == DT_F16) WLAUNCH(f16); else WLAUNCH(bf16);
-#undef WLAUNCH
-#undef WMODE
-#undef WGO
-        LI_CHECK_LAUNCH();
-        if (splits > 1) {
-            const int64_t quads = (int64_t)M * ((N + 3) / 4);
-            splitk_reduce_kernel<<<(unsigned)((quads + 255) / 256), 256, 0, stream>>>(ws, splits, e);
-            LI_CHECK_LAUNCH();
-        }
-        return LI_OK;
-    }
-#define GO(T, BN, BM, WV, ST)                                                                                \
-    do {                                                                                               \
-        auto kfn = gemm_dma_kernel<T, BN, BM, WV, ST>;                                                 \
-        if (hipFuncSetAttribute((const void*)kfn, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds) != hipSuccess) \
-            return LI_HIP_ERROR;                                                                       \
-        kfn<<<grid, block, lds, stream>>>((const T*)X, (const T*)Wt, K, k_per_split, ws, n_begin, e);  \
-    } while (0)
-#define LAUNCH(T)                                    \
-    do {                                             \
-        if (tile == 0) GO(T, 128, 128, 4, 3);        \
-        else if (tile == 1) GO(T, 256, 128, 4, 3);   \
-        else GO(T, 256, 256, 8, 3);                  \
+        if (tile == 0) BY_MODE(T, 4);        \
+        else if (tile == 1) BY_MODE(T, 3);   \
+        else BY_MODE(T, 2);                  \
     } while (0)
     if (dt == DT_F16) LAUNCH(f16); else LAUNCH(bf16);
 #undef LAUNCH
+#undef BY_MODE
 #undef GO
     LI_CHECK_LAUNCH();
     if (splits > 1) {
@@ -815,4 +603,3 @@ extern "C" int li_gemm_dma(const void* X, const void* Wt, int dt, void* C, int o
     }
     return LI_OK;
 }
-

@@ -266,10 +266,16 @@ def linear(x: torch.Tensor, w, mode: int = EPI_STORE, out: torch.Tensor | None =
             return out
         _need(lazy is None, "a norm is finished by gemv_tiled alone")
         if force is None and m * k * 2 < (1 << 32):
-            kind = "dma"
-    if kind.startswith("dma"):
-        _need(tiled and fast_ok and m * k * 2 < (1 << 32), "gemm_dma: a tiled weight, X below 4 GiB")
-        _run_dma(x, wd, out, out_dt, mode, m, n, k, n_out, _forced_dma_plan(kind) or _dma_plan(m, n, k), _rope)
+            kind = "wreg"
+    if kind.startswith("wreg"):                                # "wreg[:<tile>[:<splits>]]" (a test's choice)
+        _need(tiled and fast_ok and m * k * 2 < (1 << 32), "gemm_wreg: a tiled weight, X below 4 GiB")
+        parts = kind.split(":")
+        tile, splits = _wreg_plan(m, n, k)
+        if len(parts) > 1:
+            tile, splits = int(parts[1]), int(parts[2]) if len(parts) > 2 else 1
+        ws = _workspace(splits * m * n, x.device) if splits > 1 else None
+        _check(lib.li_gemm_wreg(_ptr(x), _ptr(wd), DT[x.dtype], _ptr(out), out_dt, mode, m, n, k, tile, splits,
+                                _ptr(ws), rs, _stream()), "gemm_wreg")
         return out
     if kind == "fma":
         _check(lib.li_gemm_fma(_ptr(x), DT[x.dtype], _ptr(w), DT[w.dtype], _ptr(out), out_dt, mode,
@@ -304,63 +310,21 @@ def linear(x: torch.Tensor, w, mode: int = EPI_STORE, out: torch.Tensor | None =
     return out
 
 
-def _forced_dma_plan(kind: str):
-    """The plan that a test asks for: "dma:<tile>[:<splits>]", "dma2:<tile>:<columns>:<tile of the rest>",
-    "dmarows:<tile>:<rows>:<tile of the rest>"; None for plain "dma" (the planner decides)."""
-    parts = kind.split(":")
-    if parts[0] == "dma2":
-        return [(int(parts[1]), 1, 0, int(parts[2]), 0, 0), (int(parts[3]), 1, int(parts[2]), 0, 0, 0)]
-    if parts[0] == "dmarows":
-        return [(int(parts[1]), 1, 0, 0, 0, int(parts[2])), (int(parts[3]), 1, 0, 0, int(parts[2]), 0)]
-    if len(parts) > 1:
-        return [(int(parts[1]), int(parts[2]) if len(parts) > 2 else 1, 0, 0, 0, 0)]
-    return None
-
-
-def _run_dma(x, wd, out, out_dt, mode, m, n, k, n_out, plan, rope) -> None:
-    """The launches of a plan (`_dma_plan`): each covers a range of columns and of rows of the product;
-    a launch that does not start at row 0 gets X, the output and the rotation epilogue's per-row
-    arrays from its first row on."""
-    lib = core()
-    element_bytes = {0: 4, 1: 2, 2: 2}                     # by dtype code
-    for tile, splits, n_begin, n_count, m_begin, m_count in plan:
-        rows = m_count or m - m_begin
-        _need(0 <= m_begin < m and m_begin + rows <= m, "gemm_dma: rows outside the product")
-        _need(tile < 3 or k % 64 == 0, "gemm_wreg (tiles 3 to 5): K must be a multiple of 64")
-        ws = _workspace(splits * rows * n, x.device) if splits > 1 else None
-        xp = c_void_p(x.data_ptr() + m_begin * k * x.element_size())
-        op = c_void_p(out.data_ptr() + m_begin * n_out * out.element_size()) if out is not None else c_void_p(0)
-        rp = ctypes.byref(rope) if rope is not None else None
-        if rope is not None and m_begin:
-            shifted = _RopeStore()
-            ctypes.pointer(shifted)[0] = rope
-            per_row = (("pos", 4), ("tok_slot", 4), ("cos_sin", rope.rotary_dim // 2 * 2 * 4),
-                       ("q_out", rope.H * rope.hd * element_bytes[rope.dt]))
-            for field, step in per_row:
-                v = getattr(rope, field)
-                setattr(shifted, field, v + m_begin * step if v else v)
-            rp = ctypes.byref(shifted)
-        _check(lib.li_gemm_dma(xp, _ptr(wd), DT[x.dtype], op, out_dt, mode, rows, n, k, tile, splits,
-                               _ptr(ws), rp, n_begin, n_count, _stream()), "gemm_dma")
-
-
-# rows of W x rows of X of a workgroup.  Tiles 0 to 2 are gemm_dma (W and X through LDS), 3 to 5
-# gemm_wreg (W from memory into registers, X through LDS; K in steps of 64).
-_DMA_TILES = {0: (128, 128), 1: (256, 128), 2: (256, 256), 3: (256, 128), 4: (192, 128), 5: (128, 128)}
+# rows of W x rows of X of a workgroup of gemm_wreg
+_WREG_TILES = {0: (256, 128), 1: (192, 128), 2: (128, 128)}
 # Microseconds that one round of workgroups takes, measured on MI355X, as (a, c): a K / 4096 + c.  Entry i
-# is a round with i + 1 workgroups on every CU.  gemm_dma runs one a CU; of gemm_wreg two or three share a
-# CU, and those of a last round that is less full run at the shorter time.
-_DMA_ROUND_US = {0: ((48.0, 0.0),), 1: ((72.0, 0.0),), 2: ((124.0, 0.0),),
-                 3: ((53.0, 9.0), (103.0, 5.0)), 4: ((35.0, 13.0), (73.0, 12.0)),
-                 5: ((31.4, 3.4), (57.1, 3.8), (89.0, 0.0))}
+# is a round with i + 1 workgroups on every CU: two share a CU (three of the narrowest tile), and those of a
+# last round that is less full run at the shorter time.
+_WREG_ROUND_US = {0: ((53.0, 9.0), (103.0, 5.0)), 1: ((35.0, 13.0), (73.0, 12.0)),
+                  2: ((31.4, 3.4), (57.1, 3.8), (89.0, 0.0))}
 
 
-def _dma_cost(tile: int, splits: int, m: int, n: int, k: int) -> float:
-    """Estimated microseconds of one launch of the prefill product (and its split-K reduction): rounds of
-    workgroups at the measured time of a round, not below the time to stream W once; a fixed cost for
-    the launch, the first tiles and the epilogue; the partial sums written and read back."""
-    bn, bm = _DMA_TILES[tile]
-    times = _DMA_ROUND_US[tile]
+def _wreg_cost(tile: int, splits: int, m: int, n: int, k: int) -> float:
+    """Estimated microseconds of one gemm_wreg launch (and its split-K reduction): rounds of workgroups
+    at the measured time of a round, not below the time to stream W once; a fixed cost for the launch,
+    the first tiles and the epilogue; the partial sums written and read back."""
+    bn, bm = _WREG_TILES[tile]
+    times = _WREG_ROUND_US[tile]
     full, rest = divmod(-(-m // bm) * -(-n // bn) * splits, 256 * len(times))
     k_split = -(-(-(-k // splits)) // 32) * 32
     us = 0.0
@@ -372,37 +336,12 @@ def _dma_cost(tile: int, splits: int, m: int, n: int, k: int) -> float:
 
 
 @functools.lru_cache(maxsize=4096)
-def _dma_plan(m: int, n: int, k: int) -> list:
-    """The launches of the prefill product (gemm_dma and gemm_wreg, one entry point): (tile, splits of
-    K, first column, columns, first row, rows) each (0 columns or rows: all from the first on).
-    Tile and splits are the pair with the least estimated time (`_dma_cost`): few rows of X want
-    K split so that most CUs get a workgroup, but every split adds partial sums to write and read.
-    gemm_wreg's tiles are there when K is a multiple of 64.  gemm_dma's workgroups run in rounds of
-    one per CU, and a last round that is nearly empty costs as much as a full one: a product of many
-    rounds may get its large tile for as many columns (or, if that fits better, rows) as fill whole
-    rounds and a smaller tile for the rest, if that is clearly faster by the same estimate."""
-    tiles = (2, 1, 0, 3, 4, 5) if k % 64 == 0 else (2, 1, 0)            # gemm_wreg steps by 64 of K
-    options = [(t, s) for t in tiles for s in (1, 2, 3, 4, 6, 8, 12, 16) if s == 1 or k // s >= 1024]
-    tile, splits = min(options, key=lambda o: (_dma_cost(o[0], o[1], m, n, k), o[1], -o[0]))
-    plan, cost = [(tile, splits, 0, 0, 0, 0)], _dma_cost(tile, splits, m, n, k)
-    if splits > 1:
-        return plan
-    for big in (2, 1):                                          # (gemm_dma's tiles)
-        bn, bm = _DMA_TILES[big]
-        m_tiles, n_tiles = -(-m // bm), -(-n // bn)
-        whole = m_tiles * n_tiles // 256 * 256                 # workgroups of the whole rounds
-        cols, rows = whole // m_tiles * bn, whole // n_tiles * bm
-        if 0 < cols < n:
-            rest = min(range(big), key=lambda t: (_dma_cost(t, 1, m, n - cols, k), -t))
-            c = _dma_cost(big, 1, m, cols, k) + _dma_cost(rest, 1, m, n - cols, k)
-            if c < 0.95 * cost:                # the estimate is coarse: only a clear gain is taken
-                plan, cost = [(big, 1, 0, cols, 0, 0), (rest, 1, cols, 0, 0, 0)], c
-        if 0 < rows < m:
-            rest = min(range(big), key=lambda t: (_dma_cost(t, 1, m - rows, n, k), -t))
-            c = _dma_cost(big, 1, rows, n, k) + _dma_cost(rest, 1, m - rows, n, k)
-            if c < 0.95 * cost:
-                plan, cost = [(big, 1, 0, 0, 0, rows), (rest, 1, 0, 0, rows, 0)], c
-    return plan
+def _wreg_plan(m: int, n: int, k: int) -> tuple[int, int]:
+    """Tile and splits of K for a product: the pair with the least estimated time (`_wreg_cost`).  Few rows
+    of X want K split so that most CUs get a workgroup, but every split adds partial sums to write and
+    read; the narrower tiles are for products whose tiles would leave much of the last round empty."""
+    options = [(t, s) for t in (0, 1, 2) for s in (1, 2, 3, 4, 6, 8, 12, 16) if s == 1 or k // s >= 1024]
+    return min(options, key=lambda o: (_wreg_cost(o[0], o[1], m, n, k), o[1], o[0]))
 
 
 def _big_tile(m: int, n: int) -> int:

@@ -207,34 +207,21 @@ def test_decode_splits_fill_the_chip_and_are_powers_of_two():
             assert s & (s - 1) == 0 and 1 <= s <= max(1, pages // 2)
 
 
-def test_launch_plans_cover_every_product_once():
-    """What the planner of the prefill GEMM hands the kernel: launches that tile the product without
-    gap or overlap, a first part that ends on the large tile's grid, K split only for a whole product."""
+def test_the_prefill_product_plan():
+    """What the planner of the prefill product hands the kernel: a tile it has, K split only where a split
+    keeps at least 1,024 of K, few rows of X split (the chip has 256 CUs to fill), many rows not."""
     import random as _r
 
-    from llm_infer_amd.kernels.ops import _DMA_TILES, _dma_plan
+    from llm_infer_amd.kernels.ops import _WREG_TILES, _wreg_cost, _wreg_plan
     rng = _r.Random(0)
     shapes = [(2048, 28672, 4096), (33186, 2048, 8192), (3000, 6144, 4096), (97, 4096, 14336), (130, 128256, 4096)]
-    shapes += [(rng.randint(97, 40000), 16 * rng.randint(1, 2000), 32 * rng.randint(1, 500)) for _ in range(300)]
+    shapes += [(rng.randint(17, 40000), 16 * rng.randint(1, 2000), 32 * rng.randint(1, 500)) for _ in range(300)]
     for m, n, k in shapes:
-        plan = _dma_plan(m, n, k)
-        assert 1 <= len(plan) <= 2
-        covered = 0
-        for tile, splits, n_begin, n_count, m_begin, m_count in plan:
-            bn, bm = _DMA_TILES[tile]
-            cols, rows = n_count or n - n_begin, m_count or m - m_begin
-            assert 0 <= n_begin < n and 0 <= m_begin < m and n_begin % 16 == 0
-            assert n_begin + cols <= n and m_begin + rows <= m
-            assert splits >= 1 and (splits == 1 or (len(plan) == 1 and k // splits >= 1024))
-            if n_begin + cols < n:
-                assert cols % bn == 0             # only the last columns may end inside a tile
-            if m_begin + rows < m:
-                assert rows % bm == 0
-            covered += cols * rows
-        assert covered == m * n, (m, n, k, plan)
-        if len(plan) == 2:
-            (_, _, nb0, nc0, mb0, mc0), (_, _, nb1, _, mb1, _) = plan
-            assert (nb0, mb0) == (0, 0) and ((nb1 == nc0 and mb1 == 0 and mc0 == 0) or (mb1 == mc0 and nb1 == 0 and nc0 == 0))
+        tile, splits = _wreg_plan(m, n, k)
+        assert tile in _WREG_TILES and splits >= 1 and (splits == 1 or k // splits >= 1024)
+        assert _wreg_cost(tile, splits, m, n, k) <= min(_wreg_cost(t, 1, m, n, k) for t in _WREG_TILES)
+    assert _wreg_plan(64, 4096, 4096)[1] > 1 and _wreg_plan(8192, 4096, 4096) == (0, 1)
+    assert _wreg_plan(2048, 6144, 4096)[0] == 1           # 512 tiles of 192 x 128: two on every CU
 
 
 def test_cache_rounding_option_is_for_a_float32_cache():

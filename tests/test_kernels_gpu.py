@@ -123,19 +123,8 @@ def test_linear_tiled_weights(ops, M, N, K, dt):
     assert ops.is_tiled(wt) and wt.logical == (N, K) and wt.numel() == (N + 15) // 16 * 16 * K and wt.owner == "device"
     assert torch.equal(ops.untile(wt), w.to(DEV))
     kinds = [None, "mfma:0:1", "mfma:1:2", "mfma:2:1", "big:0", "big:1", "big:0:2", "big:1:5"] + (["gemv_mfma"] if M <= 16 else [])
-    kinds += ["dma", "dma:0", "dma:1", "dma:2", "dma:0:2", "dma:1:5", "dma:2:3"]
-    wreg = K % 64 == 0                # W into registers (tiles of 256, 192, 128 rows of W): K in steps of 64
-    if wreg:
-        kinds += ["dma:3", "dma:4", "dma:5", "dma:3:2", "dma:4:5", "dma:5:3"]
-    else:
-        with pytest.raises(ops.KernelError, match="multiple of 64"):
-            ops.linear(x, wt, force="dma:3")
-    # the first columns with one tile, the rest with another (the first count a multiple of the first tile)
-    kinds += [f"dma2:{a}:{c}:{b}" for a, c, b in ((2, 256, 1), (2, 512, 0), (1, 512, 0), (0, 128, 2), (3, 256, 5), (4, 192, 3), (5, 128, 4))
-              if c < N and (wreg or max(a, b) < 3)]
-    # and the first rows with one tile, the rest with another
-    kinds += [f"dmarows:{a}:{r}:{b}" for a, r, b in ((2, 256, 0), (1, 128, 0), (0, 128, 2), (3, 128, 5), (5, 128, 4))
-              if r < M and (wreg or max(a, b) < 3)]
+    # W into registers (tiles of 256, 192, 128 rows of W): the planner's choice and every tile, K whole and split
+    kinds += ["wreg", "wreg:0", "wreg:1", "wreg:2", "wreg:0:2", "wreg:1:5", "wreg:2:3"]
     for kind in kinds:
         for mode in (0, 1, 2, 4):
             if mode in (2, 4) and N % 2:
@@ -237,11 +226,10 @@ def test_gate_activation_alone(ops):
         assert ops.swiglu(gu, torch.bfloat16, gelu=gelu).dtype == torch.bfloat16
 
 
-@pytest.mark.parametrize("M,N,K", [(2048, 8560, 736), (5000, 4048, 736)])
-def test_products_that_end_with_a_smaller_tile(ops, M, N, K):
-    """Sizes at which the planner itself splits a product: the large tile for the columns (or rows) that
-    fill whole rounds of workgroups, a smaller tile for the rest."""
-    assert len(ops._dma_plan(M, N, K)) == 2
+@pytest.mark.parametrize("M,N,K", [(2048, 8560, 736), (5000, 4048, 736), (1300, 12288, 4096)])
+def test_large_products(ops, M, N, K):
+    """Products of many tiles as the planner runs them: a K that is 32 more than a multiple of 64, widths and
+    heights that end inside a tile."""
     g = torch.Generator().manual_seed(M + N)
     x = torch.randn(M, K, generator=g).to(torch.float16).to(DEV)
     w = (torch.randn(N, K, generator=g) / math.sqrt(K)).to(torch.float16).to(DEV)
@@ -528,8 +516,7 @@ def test_rotation_fused_into_the_projection(ops, dt, T, H, K, hd, rot, d):
         if tiled and d % 32:
             continue
         ww = ops.tile_weight(w) if tiled else w
-        wreg = ["dma:3", "dma:4:2", "dma:5"] if d % 64 == 0 else []
-        for kind in kinds + ((["dma:0", "dma:1:2", "dma:2"] + wreg + (["dma2:0:128:1"] + (["dma2:5:128:3"] if wreg else []) if (H + 2 * K) * hd > 128 else []) + (["dmarows:0:128:1"] if T > 128 else [])) if tiled else []):
+        for kind in kinds + (["wreg:0", "wreg:1:2", "wreg:2"] if tiled else []):
             if tiled and kind == "fma":
                 continue
             c1, v1 = fresh()
