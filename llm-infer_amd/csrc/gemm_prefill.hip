@@ -219,6 +219,8 @@ __global__ __launch_bounds__(256) void gemm_big_kernel(const T* __restrict__ X, 
 // MODE: EPI_ADD or EPI_ROPE for a kernel whose epilogue is that one alone and fetches what it reads from
 // memory early (the residual a strip ahead; positions and pages once, angles a quad ahead); -1 for every
 // epilogue, chosen at run time.
+// The loop counts its own loads and LDS reads in flight (s_waitcnt by hand), so the compiler must add none:
+// no spills (the build checks that the kernel uses no scratch memory).
 template <class T, int NI, int MODE>
 __global__ __launch_bounds__(256) void gemm_wreg_kernel(const T* __restrict__ X, const T* __restrict__ Wt,
                                                         int K, int k_per_split, float* __restrict__ ws, Epilogue e) {
@@ -226,7 +228,7 @@ __global__ __launch_bounds__(256) void gemm_wreg_kernel(const T* __restrict__ X,
     // A step is 64 of K: two halves of 32, each one matrix instruction deep.
     // MJ: fragments of X (16 rows each) per wave and half step; every wave takes all the tile's rows of X
     constexpr int MJ = 8, BN = 64 * NI, BM = 16 * MJ, XBUFS = 3, SLOTS = 4;
-    constexpr int XU = 2 * MJ, PER_WAVE = XU / 4;       // 1 KiB units of X per stage (two halves of MJ), and per wave
+    constexpr int XU = BM / 8, PER_WAVE = XU / 4;       // 1 KiB units of X per stage (8 rows x 64 of K each), and per wave
     constexpr int STAGE = XU * 1024;
     extern __shared__ __attribute__((aligned(16))) unsigned char smem_raw[];
 

@@ -233,6 +233,21 @@ def test_cache_rounding_option_is_for_a_float32_cache():
     assert c.groups[0].round_to == torch.float16
 
 
+def test_a_build_whose_hand_counted_kernel_spills_is_refused():
+    """gemm_wreg places its own waits by counting its loads; a spill would be a load it does not count."""
+    from llm_infer_amd.kernels import build
+    ok = ("x.hip:1:1: remark: Function Name: _Z16gemm_wreg_kernelIDF16_Li4ELin1EEv [-Rpass-analysis=kernel-resource-usage]\n"
+          "x.hip:1:1: remark:     ScratchSize [bytes/lane]: 0 [-Rpass-analysis=kernel-resource-usage]\n"
+          "x.hip:9:1: remark: Function Name: _Z15gemm_big_kernelIDF16_E [-Rpass-analysis=kernel-resource-usage]\n"
+          "x.hip:9:1: remark:     ScratchSize [bytes/lane]: 48 [-Rpass-analysis=kernel-resource-usage]\n")
+    build._check_no_scratch(ok, "gemm_wreg_kernel", "x.hip")            # another kernel's scratch is its own business
+    with pytest.raises(build.BuildError, match="16 bytes of scratch"):
+        build._check_no_scratch(ok.replace("lane]: 0", "lane]: 16"), "gemm_wreg_kernel", "x.hip")
+    with pytest.raises(build.BuildError, match="no resource usage"):
+        build._check_no_scratch("", "gemm_wreg_kernel", "x.hip")
+    assert build.NO_SCRATCH == {"gemm_prefill.hip": "gemm_wreg_kernel"}
+
+
 def test_build_folder_is_the_same_for_builds_that_run_side_by_side(tmp_path, monkeypatch):
     """Every library of one build lands in one folder: the probe for a writable folder must not
     collide between threads (a collision once sent some libraries to the temporary folder)."""
