@@ -195,6 +195,107 @@ static __global__ void splitk_reduce_kernel(const float* __restrict__ ws, int sp
 }
 
 
+// The RMS norm that reads the rows of a residual sum next (src/model/block.cpp:127, 191): weight [N], eps, and
+// where its result goes ([M, N] of out_dt).
+struct NormAfter {
+    const float* w;
+    void* out;
+    int out_dt;
+    float eps;
+};
+
+// For C += X W^T with K split: the sum of the partials (ascending split order, as splitk_reduce_kernel), the
+// residual sum, and the norm of the finished row, a workgroup a row.  The norm is rmsnorm_vec_kernel's, value for
+// value: same pieces per thread, same order of the sum of squares, same expression.  N a multiple of 4, at most
+// 4 V blockDim.x; pointers 16-byte aligned.
+template <class TO, int V>
+static __global__ void splitk_add_norm_kernel(const float* __restrict__ ws, int splits, float* __restrict__ C,
+                                              int M, int N, const float* __restrict__ w, TO* __restrict__ out,
+                                              float eps) {
+    struct alignas(4 * sizeof(TO)) Out4 { TO v[4]; };
+    __shared__ float scratch[16];
+    const int r = blockIdx.x, n4 = N >> 2;
+    f32x4* xr = (f32x4*)(C + (int64_t)r * N);
+    const f32x4* w4 = (const f32x4*)w;
+    Out4* o = (Out4*)(out + (int64_t)r * N);
+    const int64_t stride4 = (int64_t)M * n4;
+    f32x4 xv[V], wv[V];
+#pragma unroll
+    for (int j = 0; j < V; ++j) {
+        const int i = threadIdx.x + j * blockDim.x;
+        xv[j] = f32x4{0.f, 0.f, 0.f, 0.f};
+        if (i < n4) {
+            const f32x4* p = (const f32x4*)ws + (int64_t)r * n4 + i;
+            f32x4 v = {0.f, 0.f, 0.f, 0.f};
+            f32x4 c = xr[i];
+            // four splits' loads in flight at a time; the sums stay in ascending split order
+            int s = 0;
+            for (; s + 4 <= splits; s += 4) {
+                f32x4 t[4];
+#pragma unroll
+                for (int u = 0; u < 4; ++u) t[u] = p[(s + u) * stride4];
+#pragma unroll
+                for (int u = 0; u < 4; ++u)
+#pragma unroll
+                    for (int q = 0; q < 4; ++q) v[q] += t[u][q];
+            }
+            for (; s < splits; ++s) {
+                const f32x4 t = p[s * stride4];
+#pragma unroll
+                for (int q = 0; q < 4; ++q) v[q] += t[q];
+            }
+#pragma unroll
+            for (int q = 0; q < 4; ++q) c[q] += v[q];
+            xr[i] = c;
+            xv[j] = c;
+        }
+    }
+#pragma unroll
+    for (int j = 0; j < V; ++j) {
+        const int i = threadIdx.x + j * blockDim.x;
+        wv[j] = i < n4 ? w4[i] : f32x4{0.f, 0.f, 0.f, 0.f};
+    }
+    float ss = 0.f;
+#pragma unroll
+    for (int j = 0; j < V; ++j)
+#pragma unroll
+        for (int q = 0; q < 4; ++q) ss += xv[j][q] * xv[j][q];
+    ss = block_sum(ss, scratch);
+    const float rms = sqrtf(ss / (float)N + eps);
+#pragma unroll
+    for (int j = 0; j < V; ++j) {
+        const int i = threadIdx.x + j * blockDim.x;
+        if (i < n4) {
+            Out4 t;
+#pragma unroll
+            for (int q = 0; q < 4; ++q) t.v[q] = from_f32<TO>(xv[j][q] / rms * wv[j][q]);
+            o[i] = t;
+        }
+    }
+}
+
+// Whether splitk_add_norm_kernel can stand for splitk_reduce_kernel + the norm kernel.
+static bool norm_after_fits(const NormAfter* na, const Epilogue& e, const float* ws) {
+    return na && na->w && na->out && e.mode == EPI_ADD && e.N % 4 == 0 && e.N <= 8192 &&
+           (na->out_dt == DT_F16 || na->out_dt == DT_BF16 || na->out_dt == DT_F32) &&
+           !(((uintptr_t)ws | (uintptr_t)e.C | (uintptr_t)na->w | (uintptr_t)na->out) & 15);
+}
+
+static void launch_splitk_add_norm(const float* ws, int splits, const Epilogue& e, const NormAfter* na,
+                                   hipStream_t stream) {
+    // threads and pieces per thread as li_rmsnorm chooses them
+    const int n4 = e.N / 4;
+    const int threads = n4 <= 64 ? 64 : (n4 <= 256 ? 128 : (n4 <= 1024 ? 256 : 512));
+    const bool two = n4 <= 2 * threads;
+#define GO(TO)                                                                                                  \
+    do {                                                                                                        \
+        if (two) splitk_add_norm_kernel<TO, 2><<<e.M, threads, 0, stream>>>(ws, splits, (float*)e.C, e.M, e.N, na->w, (TO*)na->out, na->eps); \
+        else splitk_add_norm_kernel<TO, 4><<<e.M, threads, 0, stream>>>(ws, splits, (float*)e.C, e.M, e.N, na->w, (TO*)na->out, na->eps);     \
+    } while (0)
+    if (na->out_dt == DT_F32) GO(float); else if (na->out_dt == DT_F16) GO(f16); else GO(bf16);
+#undef GO
+}
+
 static int make_epilogue(Epilogue& e, void* C, int mode, int out_dt, int M, int N, const RopeStore* rs) {
     e.C = C; e.mode = mode; e.out_dt = out_dt; e.M = M; e.N = N;
     e.rs = RopeStore{};

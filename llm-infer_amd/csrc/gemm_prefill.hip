@@ -555,9 +555,11 @@ extern "C" int li_gemm_big(const void* X, const void* W, int tiled, int dt, void
 
 // tile (rows of W x rows of X): 0 = 256 x 128, 1 = 192 x 128, 2 = 128 x 128.  W tiled (K a multiple of 32),
 // X below 4 GiB (the kernel addresses it with 32-bit offsets); ws: splits * M * N floats when K is split.
+// `na` (or null): with K split and the residual sum as epilogue, the kernel that adds the partial sums also
+// takes the norm of the finished rows; it must fit (norm_after_fits), the caller has checked the same.
 extern "C" int li_gemm_wreg(const void* X, const void* Wt, int dt, void* C, int out_dt, int mode,
                             int M, int N, int K, int tile, int splits, float* ws, const RopeStore* rs,
-                            hipStream_t stream) {
+                            const NormAfter* na, hipStream_t stream) {
     int rc = check_common(X, Wt, C, M, N, K, mode, out_dt);
     if (rc) return rc;
     if (dt != DT_F16 && dt != DT_BF16) return LI_BAD_ARG;
@@ -572,6 +574,7 @@ extern "C" int li_gemm_wreg(const void* X, const void* Wt, int dt, void* C, int 
     const int bn = 256 - 64 * tile, bm = 128, bk = 32;
     int k_per_split = ((K + splits - 1) / splits + bk - 1) / bk * bk;
     splits = (K + k_per_split - 1) / k_per_split;
+    if (na && !(splits > 1 && norm_after_fits(na, e, ws))) return LI_BAD_ARG;
     dim3 grid((M + bm - 1) / bm, (N + bn - 1) / bn, splits), block(256);
     // three stages of X (a step is 64 of K); the epilogue stages two strips of 16 x (bn / 4 + 4) floats a wave
     // in the same LDS, and behind both lie a position and a page for each of the tile's rows
@@ -598,7 +601,10 @@ extern "C" int li_gemm_wreg(const void* X, const void* Wt, int dt, void* C, int 
 #undef BY_MODE
 #undef GO
     LI_CHECK_LAUNCH();
-    if (splits > 1) {
+    if (splits > 1 && na) {
+        launch_splitk_add_norm(ws, splits, e, na, stream);
+        LI_CHECK_LAUNCH();
+    } else if (splits > 1) {
         const int64_t quads = (int64_t)M * ((N + 3) / 4);
         splitk_reduce_kernel<<<(unsigned)((quads + 255) / 256), 256, 0, stream>>>(ws, splits, e);
         LI_CHECK_LAUNCH();

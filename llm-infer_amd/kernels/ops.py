@@ -128,16 +128,33 @@ class LazyNorm:
         return rmsnorm(self.x, self.weight, self.eps, self.dtype)
 
 
-def expect_norm(x: torch.Tensor, weight) -> None:
-    """Says which norm weight (float32 [width], or None) will read the rows of ``x`` next.  A product
-    that adds into ``x`` may then prepare that norm (``LazyNorm``).  Only a hint: a norm with another
-    weight, or rows that something else has written to since, get the norm kernel."""
+def expect_norm(x: torch.Tensor, weight, eps: float | None = None) -> None:
+    """Says which RMS norm (weight float32 [width], or None; its eps) will read the rows of ``x`` next.
+    A product that adds into ``x`` may then prepare that norm (``LazyNorm``) or take it whole
+    (``prepared_rmsnorm``).  Only a hint: a norm with another weight or eps, or rows that something else
+    has written to since, get the norm kernel."""
     x._li_next_norm = weight
+    x._li_next_eps = eps
 
 
 def _drop_row_stats(x) -> None:
     if x is not None and getattr(x, "_li_rows", None) is not None:
         x._li_rows = None
+    if x is not None and getattr(x, "_li_normed", None) is not None:
+        x._li_normed = None
+
+
+def prepared_rmsnorm(x: torch.Tensor, w: torch.Tensor, eps: float, out_dtype):
+    """The norm of all rows of ``x`` if the product that last added into ``x`` has taken it already (with K
+    split, the kernel that adds the partial sums has the finished rows in its hands): same weight tensor,
+    same eps and type, and nothing has written to ``x`` since; else None."""
+    rec = getattr(x, "_li_normed", None)
+    if rec is None:
+        return None
+    normed, weight, rec_eps, version = rec
+    if weight is not w or rec_eps != eps or version != x._version or normed.dtype != out_dtype or normed.shape != x.shape:
+        return None
+    return normed
 
 
 def lazy_rmsnorm(x: torch.Tensor, w: torch.Tensor, eps: float, out_dtype):
@@ -152,6 +169,10 @@ def lazy_rmsnorm(x: torch.Tensor, w: torch.Tensor, eps: float, out_dtype):
     if weight is not w or version != x._version or xw.dtype != out_dtype or xw.shape != x.shape:
         return None
     return LazyNorm(x, w, eps, out_dtype, xw, ss, scale)
+
+
+class _NormAfter(ctypes.Structure):
+    _fields_ = [("w", c_void_p), ("out", c_void_p), ("out_dt", c_int), ("eps", c_float)]
 
 
 class _RopeStore(ctypes.Structure):
@@ -274,8 +295,20 @@ def linear(x: torch.Tensor, w, mode: int = EPI_STORE, out: torch.Tensor | None =
         if len(parts) > 1:
             tile, splits = int(parts[1]), int(parts[2]) if len(parts) > 2 else 1
         ws = _workspace(splits * m * n, x.device) if splits > 1 else None
+        # with K split, the kernel that adds the partial sums to the residual also takes the norm that reads
+        # the finished rows next, if the block has said which one that is
+        na = normed = None
+        nxt, eps = getattr(out, "_li_next_norm", None), getattr(out, "_li_next_eps", None)
+        k_split = -(-(-(-k // splits)) // 32) * 32
+        if (mode == EPI_ADD and -(-k // k_split) > 1 and nxt is not None and eps is not None and n % 4 == 0 and n <= 8192
+                and nxt.dtype == torch.float32 and nxt.shape == (n,) and nxt.is_cuda
+                and (ws.data_ptr() | out.data_ptr() | nxt.data_ptr()) % 16 == 0):
+            normed = torch.empty((m, n), dtype=x.dtype, device=x.device)
+            na = _NormAfter(nxt.data_ptr(), normed.data_ptr(), DT[x.dtype], eps)
         _check(lib.li_gemm_wreg(_ptr(x), _ptr(wd), DT[x.dtype], _ptr(out), out_dt, mode, m, n, k, tile, splits,
-                                _ptr(ws), rs, _stream()), "gemm_wreg")
+                                _ptr(ws), rs, ctypes.byref(na) if na is not None else None, _stream()), "gemm_wreg")
+        if na is not None:
+            out._li_normed = (normed, nxt, eps, out._version)
         return out
     if kind == "fma":
         _check(lib.li_gemm_fma(_ptr(x), DT[x.dtype], _ptr(w), DT[w.dtype], _ptr(out), out_dt, mode,

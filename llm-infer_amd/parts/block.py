@@ -83,7 +83,8 @@ class PreNormBlock(Block):
                 h = s.norm.forward(x)
             # and the product that completes the rows of x may prepare the norm that reads them next
             after = self.sublayers[i + 1].norm if i + 1 < len(self.sublayers) else next_norm
-            ops.expect_norm(x, after.weight if getattr(after, "can_be_lazy", False) else None)
+            lazy_after = getattr(after, "can_be_lazy", False)
+            ops.expect_norm(x, after.weight if lazy_after else None, after.eps if lazy_after else None)
             if s.role == "mixer":
                 s.part.forward(h, ctx, next(views), x, owns_cache)
             else:

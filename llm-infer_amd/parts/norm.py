@@ -32,4 +32,8 @@ class RMSNorm(Part):
             deferred = ops.lazy_rmsnorm(x, self.weight, self.eps, self.dtype)
             if deferred is not None:
                 return deferred
+        if rows is None:
+            ready = ops.prepared_rmsnorm(x, self.weight, self.eps, self.dtype)    # taken by the product before
+            if ready is not None:
+                return ready
         return ops.rmsnorm(x, self.weight, self.eps, self.dtype, rows)

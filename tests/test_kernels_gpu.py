@@ -226,6 +226,45 @@ def test_gate_activation_alone(ops):
         assert ops.swiglu(gu, torch.bfloat16, gelu=gelu).dtype == torch.bfloat16
 
 
+@pytest.mark.parametrize("dt", F16S)
+@pytest.mark.parametrize("M,d,K2", [(17, 256, 2048), (64, 4096, 4096), (200, 1000, 8192), (300, 96, 2080)])
+def test_norm_taken_by_the_sum_of_split_products(ops, M, d, K2, dt):
+    """With K split, the kernel that adds the partial sums into the residual rows also takes the norm that
+    reads them next: bit for bit what the reduction and the norm kernel give, one kernel less.  Void as soon
+    as anything else writes to the rows, for another weight or eps, and never made when K is not split."""
+    g = torch.Generator().manual_seed(M + d)
+    x0 = torch.randn(M, d, generator=g) * 3
+    a = (torch.randn(M, K2, generator=g) * 0.5).to(dt).to(DEV)
+    wot = ops.tile_weight((torch.randn(d, K2, generator=g) * 0.05).to(dt).to(DEV))
+    wn = (1 + 0.1 * torch.randn(d, generator=g)).to(DEV)
+    eps = 1e-5
+    plain = x0.to(DEV)
+    ops.linear(a, wot, ops.EPI_ADD, out=plain, force="wreg:2:2")
+    assert ops.prepared_rmsnorm(plain, wn, eps, dt) is None                 # nobody said which norm comes next
+    x = x0.to(DEV)
+    ops.expect_norm(x, wn, eps)
+    ops.linear(a, wot, ops.EPI_ADD, out=x, force="wreg:2:2")
+    assert torch.equal(x, plain)
+    ready = ops.prepared_rmsnorm(x, wn, eps, dt)
+    assert ready is not None and ready.dtype == dt and torch.equal(ready, ops.rmsnorm(x, wn, eps, dt))
+    assert ops.prepared_rmsnorm(x, wn.clone(), eps, dt) is None and ops.prepared_rmsnorm(x, wn, 2 * eps, dt) is None
+    assert ops.prepared_rmsnorm(x, wn, eps, torch.float32) is None
+    x += 1.0
+    assert ops.prepared_rmsnorm(x, wn, eps, dt) is None                     # torch wrote to the rows
+    y = x0.to(DEV)
+    ops.expect_norm(y, wn, eps)
+    ops.linear(a, wot, ops.EPI_ADD, out=y, force="wreg:2:2")
+    ops.linear(a, wot, ops.EPI_ADD, out=y, force="wreg:2:1")                # a product without a split wrote to them
+    assert ops.prepared_rmsnorm(y, wn, eps, dt) is None
+    # the planner's own choice at these sizes
+    z = x0.to(DEV)
+    ops.expect_norm(z, wn, eps)
+    ops.linear(a, wot, ops.EPI_ADD, out=z)
+    ready = ops.prepared_rmsnorm(z, wn, eps, dt)
+    assert ready is None or torch.equal(ready, ops.rmsnorm(z, wn, eps, dt))
+    assert M < 64 or ops._wreg_plan(M, d, K2)[1] == 1 or ready is not None
+
+
 @pytest.mark.parametrize("M,N,K", [(2048, 8560, 736), (5000, 4048, 736), (1300, 12288, 4096)])
 def test_large_products(ops, M, N, K):
     """Products of many tiles as the planner runs them: a K that is 32 more than a multiple of 64, widths and
