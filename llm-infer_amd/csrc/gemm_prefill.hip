@@ -83,7 +83,9 @@ __global__ __launch_bounds__(256) void gemm_big_kernel(const T* __restrict__ X, 
         wkc[c] = TILED ? (((chunk >> 6) % KSTEPS) << 5) + (((chunk >> 4) & 3) << 3) : (chunk % CPR) * 8;
         wok[c] = n0 + row < n_limit;
         const int n = min(n0 + row, n_limit - 1);
-        wsrc[c] = TILED ? W + tiled_offset(n, wkc[c], K) : W + (int64_t)n * K + wkc[c];
+        // (a chunk that lies beyond a K shorter than the tile is never used: its address is clamped too)
+        const int kc = min(wkc[c], K - 8);
+        wsrc[c] = TILED ? W + tiled_offset(n, kc, K) : W + (int64_t)n * K + kc;
         wdst[c] = row * LD + wkc[c];
     }
 #pragma unroll
@@ -91,7 +93,7 @@ __global__ __launch_bounds__(256) void gemm_big_kernel(const T* __restrict__ X, 
         const int chunk = tid + c * 256, row = chunk / CPR;
         xkc[c] = (chunk % CPR) * 8;
         xok[c] = m0 + row < e.M;
-        xsrc[c] = X + (int64_t)min(m0 + row, e.M - 1) * K + xkc[c];
+        xsrc[c] = X + (int64_t)min(m0 + row, e.M - 1) * K + min(xkc[c], K - 8);
         xdst[c] = BN * LD + row * LD + xkc[c];
     }
     // loads are raw; the mask (rows beyond the matrix, k beyond K) is applied when the tile is
