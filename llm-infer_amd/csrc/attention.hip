@@ -20,6 +20,7 @@
 // float32 kernel: one workgroup per (token, head), keys in ascending order, so a
 // result does not depend on how the step was cut or batched.
 #include "common.h"
+#include <type_traits>
 
 #ifndef HEAD_DIM
 #error "compile with -DHEAD_DIM=<head size>"
@@ -88,23 +89,6 @@ struct WaveAttn {
         softmax_step(s, t0, lo, hi, scale2, masked);
     }
 
-    // The same with the key fragments fetched where they are used.
-    __device__ __forceinline__ void scores_streamed(const T* kpage, f32x16 (&s)[2], int t0, int lo, int hi,
-                                                    float scale2, bool masked = true) {
-        const int lane = threadIdx.x & 63;
-#pragma unroll
-        for (int b = 0; b < 2; ++b) {
-#pragma unroll
-            for (int r = 0; r < 16; ++r) s[b][r] = 0.f;
-#pragma unroll
-            for (int ks = 0; ks < KS; ++ks) {
-                const v8 kf = *(const v8*)(kpage + ((b * KS + ks) * 64 + lane) * 8);
-                s[b] = mfma32(kf, q[ks], s[b]);
-            }
-        }
-        softmax_step(s, t0, lo, hi, scale2, masked);
-    }
-
     // scale2 > 0.  A page whose keys all lie inside lo..hi for every lane of the wave (the
     // caller knows: `masked` false) skips the comparisons.
     __device__ __forceinline__ void softmax_step(f32x16 (&s)[2], int t0, int lo, int hi, float scale2,
@@ -165,36 +149,176 @@ struct WaveAttn {
         }
     }
 
-    // One page, phases in order; the values are fetched where they are used, which keeps the
-    // register count low enough for several waves per SIMD.
-    __device__ __forceinline__ void page(const T* kpage, const T* vpage, int t0, int lo, int hi, float scale2,
-                                         bool masked = true) {
+    __device__ __forceinline__ float total() const { return l + __shfl_xor(l, 32, WAVE); }
+};
+
+// ---------------------------------------------------------------------------
+// prefill.  A workgroup of 4 waves shares the pages of one KV head through LDS.  With GW query
+// heads of a KV head packed into a workgroup (GW = 4, 2 or 1, the largest that divides the
+// group), wave w owns head w % GW and the 32-token block w / GW of the workgroup's 128 / GW
+// tokens, so every page is fetched once for up to 4 heads.
+// The scores of page p+1 are computed while the probabilities of page p are:
+// a wave issues its instructions in order, so a matrix instruction followed by the vector work
+// of a few scores keeps both units busy, where a page's 16 matrix instructions followed by its
+// softmax left each unit idle in turn.  Per step p the LDS holds the keys of page p+1 and the
+// values of page p (keys travel a page ahead of the values), fetched by global_load_lds two
+// steps before they are read, two buffers each, one barrier a step.  The arithmetic and its
+// order are those of WaveAttn (scores, softmax_step, mix), which the decode kernel uses.
+// ---------------------------------------------------------------------------
+// The value is computed by this point of the program and not later: without it the compiler
+// moves vector work that nothing nearby uses to where it is used, out from between the matrix
+// instructions that were to cover it.
+#define HERE(x) asm volatile("" : "+v"(x))
+
+template <int I, int N, class F>
+__device__ __forceinline__ void static_for(F&& f) {
+    if constexpr (I < N) {
+        f(std::integral_constant<int, I>{});
+        static_for<I + 1, N>(f);
+    }
+}
+// 16 bytes a lane from LDS, written as an instruction: the compiler knows of no wait it needs,
+// the caller waits by count (s_waitcnt lgkmcnt) before the first use.
+template <int OFFSET, class V>
+__device__ __forceinline__ void lds_read16(V& to, uint32_t addr) {
+    asm volatile("ds_read_b128 %0, %1 offset:%2" : "=v"(to) : "v"(addr), "n"(OFFSET));
+}
+
+template <class T>
+struct PrefillWave {
+    typedef typename Vec<T>::v8 v8;
+    v8 q[KS];
+    f32x16 o[DB];
+    float m, l, m_safe, alpha;
+
+    __device__ __forceinline__ void init(const T* qrow) {
         const int lane = threadIdx.x & 63;
-        f32x16 s[2];
-        scores_streamed(kpage, s, t0, lo, hi, scale2, masked);
 #pragma unroll
-        for (int tj = 0; tj < 4; ++tj) {
-            v8 pf;
-#pragma unroll
-            for (int i = 0; i < 8; ++i) pf[i] = from_f32<T>(s[tj >> 1][8 * (tj & 1) + i]);
-#pragma unroll
-            for (int b = 0; b < DB; ++b) {
-                const v8 vf = *(const v8*)(vpage + ((b * 4 + tj) * 64 + lane) * 8);
-                o[b] = mfma32(vf, pf, o[b]);
-            }
+        for (int s = 0; s < KS; ++s) {
+            v8 z = {};
+            q[s] = qrow ? *(const v8*)(qrow + 16 * s + 8 * (lane >> 5)) : z;
         }
+#pragma unroll
+        for (int b = 0; b < DB; ++b)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) o[b][r] = 0.f;
+        m = -INFINITY;
+        l = 0.f;
+        m_safe = 0.f;
+        alpha = 0.f;
+    }
+
+    // n = K Q^T for the page whose fragments this lane reads at LDS address kaddr; with SOFT, between
+    // its matrix instructions, the probabilities of the page before from its scores c (maximum and
+    // alpha already known).  The fragment reads are written as instructions, AHEAD of their use, and
+    // waited for by count: left to the compiler every other matrix instruction waited for all of them.
+    template <bool SOFT>
+    __device__ __forceinline__ void scores(uint32_t kaddr, f32x16 (&n)[2], const f32x16 (&c)[2], v8 (&pf)[4],
+                                           float scale2) {
+        constexpr int NM = 2 * KS, AHEAD = NM < 4 ? NM : 4;
+        v8 kf[NM];
+        static_for<0, AHEAD>([&](auto ic) {
+            constexpr int i = decltype(ic)::value;
+            lds_read16<((i & 1) * KS + (i >> 1)) * 1024>(kf[i], kaddr);
+        });
+        float psum = 0.f;
+#pragma unroll
+        for (int b = 0; b < 2; ++b)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) n[b][r] = 0.f;
+        static_for<0, NM>([&](auto ic) {
+            constexpr int i = decltype(ic)::value, b = i & 1, ks = i >> 1, nx = i + AHEAD;
+            if constexpr (nx < NM) lds_read16<((nx & 1) * KS + (nx >> 1)) * 1024>(kf[nx], kaddr);
+            __builtin_amdgcn_s_waitcnt(0xC07F | ((nx < NM ? AHEAD : NM - 1 - i) << 8));   // lgkmcnt: fragment i is here
+            __builtin_amdgcn_sched_barrier(0);
+            n[b] = mfma32(kf[i], q[ks], n[b]);
+            if (SOFT) {
+#pragma unroll
+                for (int e = i * 32 / NM; e < (i + 1) * 32 / NM; ++e) {
+                    float p = __builtin_amdgcn_exp2f(fmaf(c[e >> 4][e & 15], scale2, -m_safe));
+                    psum += p;
+                    HERE(p);
+                    pf[e >> 3][e & 7] = from_f32<T>(p);
+                }
+                HERE(psum);
+            }
+            __builtin_amdgcn_sched_barrier(0);
+        });
+        if (SOFT) l = l * alpha + psum;
+    }
+
+    // The probabilities alone (the last page of a wave).
+    __device__ __forceinline__ void softmax_only(const f32x16 (&c)[2], v8 (&pf)[4], float scale2) {
+        float psum = 0.f;
+#pragma unroll
+        for (int e = 0; e < 32; ++e) {
+            const float p = __builtin_amdgcn_exp2f(fmaf(c[e >> 4][e & 15], scale2, -m_safe));
+            psum += p;
+            pf[e >> 3][e & 7] = from_f32<T>(p);
+        }
+        l = l * alpha + psum;
+    }
+
+    __device__ __forceinline__ void mask(f32x16 (&n)[2], int t0, int lo, int hi) const {
+        const int lane = threadIdx.x & 63;
+#pragma unroll
+        for (int b = 0; b < 2; ++b)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) {
+                const int t = t0 + 32 * b + 8 * (r >> 2) + 4 * (lane >> 5) + (r & 3);
+                n[b][r] = (t >= lo && t <= hi) ? n[b][r] : -INFINITY;
+            }
+    }
+
+    // The running maximum takes in a page's largest score mx; alpha is what the sums so far are
+    // to be multiplied by before that page is added.
+    __device__ __forceinline__ void take_max(float mx, float scale2) {
+        mx = fmaxf(mx, __shfl_xor(mx, 32, WAVE)) * scale2;
+        const float m_new = fmaxf(m, mx);
+        m_safe = (m_new == -INFINITY) ? 0.f : m_new;
+        alpha = __builtin_amdgcn_exp2f(m - m_safe);
+        m = m_new;
+    }
+
+    __device__ __forceinline__ void rescale() {
+        if (__builtin_amdgcn_ballot_w64(alpha != 1.f) != 0) {
+#pragma unroll
+            for (int b = 0; b < DB; ++b)
+#pragma unroll
+                for (int r = 0; r < 16; ++r) o[b][r] *= alpha;
+        }
+    }
+
+    // o += V^T P^T for the page whose fragments this lane reads at LDS address vaddr; with MAX, between
+    // its matrix instructions, the largest of the next page's scores n.
+    template <bool MAX>
+    __device__ __forceinline__ void mix(uint32_t vaddr, const v8 (&pf)[4], const f32x16 (&n)[2], float scale2) {
+        constexpr int NV = 4 * DB, AHEAD = 4;
+        v8 vf[NV];
+        static_for<0, AHEAD>([&](auto jc) {
+            constexpr int j = decltype(jc)::value;
+            lds_read16<((j % DB) * 4 + j / DB) * 1024>(vf[j], vaddr);
+        });
+        float mx = -INFINITY;
+        static_for<0, NV>([&](auto jc) {
+            constexpr int j = decltype(jc)::value, nx = j + AHEAD;
+            if constexpr (nx < NV) lds_read16<((nx % DB) * 4 + nx / DB) * 1024>(vf[nx], vaddr);
+            __builtin_amdgcn_s_waitcnt(0xC07F | ((nx < NV ? AHEAD : NV - 1 - j) << 8));
+            __builtin_amdgcn_sched_barrier(0);
+            o[j % DB] = mfma32(vf[j], pf[j / DB], o[j % DB]);
+            if (MAX) {
+#pragma unroll
+                for (int e = j * 32 / NV; e < (j + 1) * 32 / NV; ++e) mx = fmaxf(mx, n[e >> 4][e & 15]);
+                HERE(mx);
+            }
+            __builtin_amdgcn_sched_barrier(0);
+        });
+        if (MAX) take_max(mx, scale2);
     }
 
     __device__ __forceinline__ float total() const { return l + __shfl_xor(l, 32, WAVE); }
 };
 
-// ---------------------------------------------------------------------------
-// prefill.  A workgroup of 4 waves shares the pages of one KV head through LDS (two
-// buffers: page p+1 travels global -> registers -> LDS while page p is used).  With GW
-// query heads of a KV head packed into a workgroup (GW = 4, 2 or 1, the largest that
-// divides the group), wave w owns head w % GW and the 32-token block w / GW of the
-// workgroup's 128 / GW tokens, so every page is fetched once for up to 4 heads.
-// ---------------------------------------------------------------------------
 template <class T>
 __global__ __launch_bounds__(256, HD <= 128 ? 2 : 1) void attn_prefill_kernel(
     const T* __restrict__ q, T* __restrict__ out, CachePtrs c, const int* __restrict__ tile_seq,
@@ -203,11 +327,11 @@ __global__ __launch_bounds__(256, HD <= 128 ? 2 : 1) void attn_prefill_kernel(
     int GW) {
     typedef typename Vec<T>::v8 v8;
     constexpr int KE = PAGE * HD, VE = PAGE * DB * 32;           // elements of a head's keys / values in a page
-    constexpr int CK = (KE / 8 + 255) / 256, CV = (VE / 8 + 255) / 256;
+    constexpr int KL = KE / 512, VL = VE / 512;                  // loads of 1 KiB (a wave's) that bring them
     extern __shared__ __attribute__((aligned(16))) unsigned char smem_raw[];
-    T* smem = (T*)smem_raw;
+    T* smem = (T*)smem_raw;                                      // keys [2][KE], values [2][VE]
 
-    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int G = H / K, TT = 32 * (4 / GW);                     // tokens of this workgroup
     // A causal prompt's later token blocks read more pages.  Workgroups start in blockIdx order,
     // 256 at a time (one per CU); every other such round walks the token blocks backwards, so the
@@ -219,26 +343,26 @@ __global__ __launch_bounds__(256, HD <= 128 ? 2 : 1) void attn_prefill_kernel(
     const int kvh = blockIdx.y / (G / GW), hc = blockIdx.y % (G / GW);
     const int h = kvh * G + hc * GW + wave % GW;
     const int qlen = seq_qlen[seq], ctx = seq_ctx[seq];
-    const int q0 = tile_q0[tile] + sub * TT;                     // first token of the workgroup within the step
+    const int q0 = tile_q0[tile] + sub * TT;
     if (q0 >= qlen) return;                                      // the same for all waves
-    const int first = q0 + 32 * (wave / GW);                     // this wave's first token
+    const int first = q0 + 32 * (wave / GW);
     const bool wave_live = first < qlen;
     const int qi = first + (lane & 31);
     const bool live = qi < qlen;
-    const int base = ctx - qlen;                                 // tokens cached before this step
+    const int base = ctx - qlen;
     const int pos = live ? base + qi : -1;
     const int64_t tok = seq_qstart[seq] + qi;
-    WaveAttn<T> a;
+    PrefillWave<T> a;
     a.init(live ? q + (tok * H + h) * HD : nullptr);
     const int lo = (window > 0 && live) ? max(0, pos - window + 1) : 0;
-    // keys from lo_max to hi_min are seen by every row of the wave: pages inside need no mask
     int lo_max = lo, hi_min = pos;
 #pragma unroll
     for (int o = 32; o > 0; o >>= 1) {
         lo_max = max(lo_max, __shfl_xor(lo_max, o, WAVE));
         hi_min = min(hi_min, __shfl_xor(hi_min, o, WAVE));
     }
-    // pages of the workgroup and of this wave
+    lo_max = __builtin_amdgcn_readfirstlane(lo_max);
+    hi_min = __builtin_amdgcn_readfirstlane(hi_min);
     const int p_lo = (window > 0 ? max(0, base + q0 - window + 1) : 0) / PAGE;
     const int p_hi = (base + min(q0 + TT - 1, qlen - 1)) / PAGE;
     const int wp_lo = (window > 0 ? max(0, base + first - window + 1) : 0) / PAGE;
@@ -248,56 +372,84 @@ __global__ __launch_bounds__(256, HD <= 128 ? 2 : 1) void attn_prefill_kernel(
     const T* vbase = (const T*)c.v + (int64_t)kvh * v_head_elems(HD);
     const float scale2 = scale * LOG2E;
 
-    v8 rk[CK], rv[CV];
-    auto fetch = [&](int p) {
-        const int64_t page = (int64_t)table[p] * c.page_stride;
+    auto kbuf = [&](int p) { return smem + (p & 1) * KE; };
+    auto vbuf = [&](int p) { return smem + 2 * KE + (p & 1) * VE; };
+    const uint32_t lds_lane = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) unsigned char*)smem_raw + lane * 16;
+    auto kaddr = [&](int p) { return lds_lane + (p & 1) * (KE * 2); };            // bytes
+    auto vaddr = [&](int p) { return lds_lane + 2 * (KE * 2) + (p & 1) * (VE * 2); };
+    const uint32_t lane_at = lane * 16;                          // bytes
+    auto bring = [&](const T* src, T* dst, int n_loads) {       // a wave takes every fourth KiB; src, dst the same for all lanes
 #pragma unroll
-        for (int i = 0; i < CK; ++i) {
-            const int ch = tid + i * 256;
-            if (KE / 8 % 256 == 0 || ch < KE / 8) rk[i] = *(const v8*)(kbase + page + ch * 8);
-        }
-#pragma unroll
-        for (int i = 0; i < CV; ++i) {
-            const int ch = tid + i * 256;
-            if (VE / 8 % 256 == 0 || ch < VE / 8) rv[i] = *(const v8*)(vbase + page + ch * 8);
-        }
-    };
-    auto stash = [&](T* buf) {
-#pragma unroll
-        for (int i = 0; i < CK; ++i) {
-            const int ch = tid + i * 256;
-            if (KE / 8 % 256 == 0 || ch < KE / 8) *(v8*)(buf + ch * 8) = rk[i];
-        }
-#pragma unroll
-        for (int i = 0; i < CV; ++i) {
-            const int ch = tid + i * 256;
-            if (VE / 8 % 256 == 0 || ch < VE / 8) *(v8*)(buf + KE + ch * 8) = rv[i];
+        for (int i = 0; i < (n_loads + 3) / 4; ++i) {
+            const int j = wave + 4 * i;
+            if (n_loads % 4 == 0 || j < n_loads)
+                __builtin_amdgcn_global_load_lds(
+                    (const __attribute__((address_space(1))) void*)((const char*)(src + j * 512) + lane_at),
+                    (__attribute__((address_space(3))) void*)(dst + j * 512), 16, 0, 0);
         }
     };
-
-    fetch(p_lo);
-    stash(smem);
-    __syncthreads();
-    // Every wave walks all pages of the workgroup (p_lo..p_hi) and works on its own (wp_lo..wp_hi).
-    // Three loops, the middle one without a condition around the page's work: with one, the
-    // compiler kept the output accumulators in a second set of registers and copied all 64 back
-    // after every page.
-    auto pass = [&](int p, auto&& work) {
-        T* cur = smem + ((p - p_lo) & 1) * (KE + VE);
-        T* nxt = smem + ((p - p_lo + 1) & 1) * (KE + VE);
-        if (p < p_hi) fetch(p + 1);
-        work(cur);
-        if (p < p_hi) stash(nxt);
+    auto at_page = [&](int entry) { return (int64_t)__builtin_amdgcn_readfirstlane(entry) * c.page_stride; };
+    // Step p: the keys of page p+1 and the values of page p have arrived (everyone's: wait, then
+    // barrier), and nobody reads the keys of page p or the values of page p-1 any more, whose
+    // buffers the loads for two steps on now fill.  The page table's entry for a step is read a
+    // step before, so that it has arrived with that step's wait.
+    int entry_v = table[p_lo], entry_k = table[min(p_lo + 1, p_hi)];      // of pages p+1 and p+2
+    auto step = [&](int p) {
+        __builtin_amdgcn_s_waitcnt(0x0F70);                      // vmcnt(0)
         __syncthreads();
+        if (p + 2 <= p_hi) bring(kbase + at_page(entry_k), kbuf(p + 2), KL);
+        if (p + 1 <= p_hi) bring(vbase + at_page(entry_v), vbuf(p + 1), VL);
+        entry_v = entry_k;
+        entry_k = table[min(p + 3, p_hi)];
     };
+    auto is_masked = [&](int p) { return p * PAGE < lo_max || p * PAGE + PAGE - 1 > hi_min; };
+
+    bring(kbase + at_page(entry_v), kbuf(p_lo), KL);
+    int p = p_lo - 1;
     const int own_lo = max(p_lo, wp_lo), own_hi = min(p_hi, wp_hi);
-    int p = p_lo;
-    for (; p < own_lo && p <= p_hi; ++p) pass(p, [](T*) {});
-    for (; p <= own_hi; ++p)
-        pass(p, [&](T* cur) {
-            a.page(cur, cur + KE, p * PAGE, lo, pos, scale2, p * PAGE < lo_max || p * PAGE + PAGE - 1 > hi_min);
-        });
-    for (; p <= p_hi; ++p) pass(p, [](T*) {});
+    if (own_lo <= own_hi) {
+        f32x16 sa[2], sb[2];
+        v8 pf[4];
+        for (; p < own_lo - 1; ++p) step(p);
+        step(p);                                                 // p = own_lo - 1: the first page's scores
+        a.template scores<false>(kaddr(p + 1), sa, sa, pf, scale2);
+        if (is_masked(p + 1)) a.mask(sa, (p + 1) * PAGE, lo, pos);
+        {
+            float mx = -INFINITY;
+#pragma unroll
+            for (int e = 0; e < 32; ++e) mx = fmaxf(mx, sa[e >> 4][e & 15]);
+            a.take_max(mx, scale2);
+        }
+        ++p;
+        auto both = [&](f32x16 (&cur)[2], f32x16 (&nxt)[2]) {    // page p from cur, the scores of p+1 into nxt
+            step(p);
+            a.template scores<true>(kaddr(p + 1), nxt, cur, pf, scale2);
+            if (is_masked(p + 1)) a.mask(nxt, (p + 1) * PAGE, lo, pos);
+            a.rescale();
+            a.template mix<true>(vaddr(p), pf, nxt, scale2);
+            ++p;
+        };
+        auto last = [&](f32x16 (&cur)[2]) {
+            step(p);
+            a.softmax_only(cur, pf, scale2);
+            a.rescale();
+            a.template mix<false>(vaddr(p), pf, cur, scale2);
+            ++p;
+        };
+        // two pages a turn, so that the scores change places without copies
+        if ((own_hi - p) & 1) {
+            both(sa, sb);
+#pragma unroll
+            for (int b = 0; b < 2; ++b) sa[b] = sb[b];
+        }
+        while (p < own_hi) {
+            both(sa, sb);
+            both(sb, sa);
+        }
+        last(sa);
+    }
+    for (; p <= p_hi; ++p) step(p);
+    __builtin_amdgcn_s_waitcnt(0x0F70);                          // nothing of this workgroup's is still on its way into LDS
     const float inv = 1.f / a.total();
     if (!live) return;
     T* orow = out + (tok * H + h) * HD;
