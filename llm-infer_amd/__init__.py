@@ -24,10 +24,14 @@ def load(folder: str, dtype: str | None = None, max_tokens: int = 8192, n_slots=
     return Engine.from_folder(folder, dtype=dtype, max_tokens=max_tokens, n_slots=n_slots, kv_round=kv_round)
 
 
-def random_model(config, seed: int = 0, dtype: str | None = None, max_tokens: int = 8192, n_slots=None, kv_round=None):
-    """An engine with random weights made on the GPU from a configuration and a seed."""
+def random_model(config, seed: int = 0, dtype: str | None = None, max_tokens: int = 8192, n_slots=None, kv_round=None,
+                 same_as_folder=None):
+    """An engine with random weights from a configuration and a seed, without a folder.  Up to half a billion
+    parameters (or with ``same_as_folder=True``) the weights are those that ``write_random_model`` writes for
+    the same seed and dtype; larger models draw theirs with the GPU's generator, which is other values."""
     from .engine import Engine
-    return Engine.from_random(config, seed=seed, dtype=dtype, max_tokens=max_tokens, n_slots=n_slots, kv_round=kv_round)
+    return Engine.from_random(config, seed=seed, dtype=dtype, max_tokens=max_tokens, n_slots=n_slots, kv_round=kv_round,
+                              same_as_folder=same_as_folder)
 
 
 def write_random_model(folder: str, config, seed: int = 0, dtype: str = "bfloat16") -> None:

@@ -1,6 +1,7 @@
 """The engine: a model, its cache, and the one step function."""
 from __future__ import annotations
 
+import math
 import sys
 
 import torch
@@ -14,6 +15,10 @@ from .step import StepContext
 
 _DTYPES = {"bfloat16": torch.bfloat16, "float16": torch.float16, "float32": torch.float32,
            "bf16": torch.bfloat16, "fp16": torch.float16, "fp32": torch.float32}
+
+
+# up to this many parameters an engine with random weights draws them as a folder's writer would
+SAME_AS_FOLDER_LIMIT = 1 << 29
 
 
 def as_dtype(d):
@@ -69,15 +74,23 @@ class Engine:
 
     @classmethod
     def from_random(cls, config, seed: int = 0, dtype=None, max_tokens: int = 8192, n_slots=None,
-                    device="cuda", stored_dtype=None, kv_round=None):
-        """Random weights made on the device (no folder): matrices as ``stored_dtype`` would store them.
-        ``dtype`` None: the configuration's ``torch_dtype``, else bfloat16."""
+                    device="cuda", stored_dtype=None, kv_round=None, same_as_folder=None):
+        """Random weights without a folder: matrices as ``stored_dtype`` would store them.
+        ``dtype`` None: the configuration's ``torch_dtype``, else bfloat16.
+        ``same_as_folder``: the tensors are drawn by the CPU's generator and are those that
+        ``write_random_model`` writes for this seed and stored dtype, so that what follows a folder (a plain
+        implementation, another run) follows this engine too.  False draws them with the device's generator:
+        other values for the same seed, and seconds instead of minutes for billions of parameters.  None (the
+        default) means True up to ``SAME_AS_FOLDER_LIMIT`` parameters."""
         _require_gpu()
         dt = choose_dtype(dtype, getattr(config, "torch_dtype", None), None)
         model = DecoderModel(config.model_spec(), dt, device)
         stored = as_dtype(stored_dtype) if stored_dtype else (dt if dt != torch.float32 else torch.bfloat16)
         params = model.params()
-        model.bind(OnDemand(lambda name: place_tensor(random_tensors({name: params[name]}, seed, stored, device)[name],
+        if same_as_folder is None:
+            same_as_folder = sum(math.prod(spec.shape) for spec in params.values()) <= SAME_AS_FOLDER_LIMIT
+        drawn_on = "cpu" if same_as_folder else device
+        model.bind(OnDemand(lambda name: place_tensor(random_tensors({name: params[name]}, seed, stored, drawn_on)[name],
                                                       params[name].kind, dt, device)))
         return cls(config, model, max_tokens, n_slots, kv_round)
 

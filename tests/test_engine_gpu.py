@@ -154,3 +154,22 @@ def test_a_model_runs_in_its_own_dtype_unless_told_otherwise(model, capfd):
     assert eng.dtype == torch.bfloat16 and "three bits" in capfd.readouterr().err
     eng = llm_infer_amd.load(model.folder["float16"], dtype="float32", max_tokens=256)
     assert eng.dtype == torch.float32 and "stored" not in capfd.readouterr().err
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_random_weights_without_a_folder_are_the_folders(dtype, tmp_path):
+    """An engine made from a configuration and a seed holds what write_random_model writes for them: the same
+    logits to the bit as the engine that opens that folder.  With the device's generator they are other values."""
+    import llm_infer_amd
+    cfg = llm_infer_amd.config_from_dict(ALL["D"])
+    llm_infer_amd.write_random_model(str(tmp_path), cfg, seed=5, dtype=STORED[dtype])
+    tokens = [[3, 1, 4, 1, 5, 9, 2, 6], [5, 3]]
+    want = [[7], [0, 1]]
+    logits = []
+    for eng in (llm_infer_amd.load(str(tmp_path), dtype=dtype, max_tokens=256),
+                llm_infer_amd.random_model(cfg, seed=5, dtype=dtype, max_tokens=256),
+                llm_infer_amd.random_model(cfg, seed=5, dtype=dtype, max_tokens=256, same_as_folder=False)):
+        slots = [eng.alloc_slot() for _ in tokens]
+        logits.append(eng.step(slots, tokens, want).float().cpu())
+    assert torch.equal(logits[0], logits[1])
+    assert not torch.equal(logits[0], logits[2])
