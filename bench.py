@@ -20,6 +20,9 @@ sys.path.insert(0, ROOT)
 
 # MI355X published peaks
 HBM_BYTES_S = 8.0e12
+# what a kernel that only reads memory reaches on this chip (16 bytes a lane, 8 loads in flight, 8 GB): the
+# achievable ceiling beside the nominal one
+HBM_MEASURED_BYTES_S = 6.3e12
 PEAK_FLOPS = {"fp16": 2.5e15, "bf16": 2.5e15, "fp32": 157.3e12}
 
 # the shapes of the benchmark configurations; the default run is the Llama-3.1-8B shape
@@ -52,6 +55,10 @@ def main() -> int:
     ap.add_argument("--points", default="1,64", help="further decode batch sizes, comma separated ('' for none)")
     ap.add_argument("--no-other-shapes", action="store_true",
                     help="leave out the 1B ragged step and the 7B batch-64 decode that the default run adds to points")
+    ap.add_argument("--no-further-sizes", action="store_true",
+                    help="leave out the long contexts, batch 128 and the generation run that the default run adds to points")
+    ap.add_argument("--generate", type=int, default=0,
+                    help="also generate for this many 128-token prompts with budgets drawn from 16..512 tokens")
     args = ap.parse_args()
     if args.gpus != 1:
         print(f"bench.py: this library runs on one GPU; --gpus {args.gpus} is not supported")
@@ -78,6 +85,35 @@ def main() -> int:
                                             "8192, tied): one step of 32 prompts of 16..2048 tokens; llama-2-7b shape (32 "
                                             "layers, hidden 4096, 32/32 heads of 128, intermediate 11008, vocab 32000): "
                                             "decode batch 64 at context 4096")
+    if args.shape == "llama-3.1-8b" and not args.no_further_sizes and not args.ragged_prefill and not args.generate:
+        # further sizes of the headline shape, in engines of their own: a long context, a large batch, and
+        # generation whose batch shrinks
+        import copy
+        al = copy.copy(args)
+        al.batch, al.points, al.context, al.layers, al.steps, al.warmup = 8, "", 32768, 0, 16, 3
+        al.prefill_tokens, al.also_prefill = 32768, [8192]
+        rl = measure(al)
+        ag = copy.copy(args)
+        ag.batch, ag.points, ag.context, ag.layers, ag.steps, ag.warmup = 128, "", 2048, 0, 24, 4
+        ag.prefill_tokens, ag.generate = 0, 64
+        rg = measure(ag)
+        gen = rg["generation"]
+        line["points"].update({
+            "decode_b8_ctx32768_ms": rl["ms_per_step"], "decode_b8_ctx32768_tokens_s": rl["value"],
+            "decode_b8_ctx32768_frac_of_hbm": rl["roofline"]["frac"],
+            "prefill_32768_ms": rl["prefill"]["ms"], "prefill_32768_frac_of_peak": rl["prefill"]["frac"],
+            "prefill_8192_ms": rl["also_prefill"]["8192"]["ms"],
+            "prefill_8192_frac_of_peak": rl["also_prefill"]["8192"]["frac"],
+            "decode_b128_ctx2048_ms": rg["ms_per_step"], "decode_b128_ctx2048_tokens_s": rg["value"],
+            "decode_b128_ctx2048_frac_of_hbm": rg["roofline"]["frac"],
+            "generate_64x128_tokens_s": gen["tokens_s"], "generate_64x128_new_tokens": gen["new_tokens"],
+            "generate_64x128_decode_s": gen["decode_s"], "generate_64x128_steps_eager": gen["steps_eager"],
+            "generate_64x128_steps_recorded": gen["steps_recorded"], "generate_64x128_steps_replayed": gen["steps_replayed"],
+            "generate_64x128_replayed_frac": gen["replayed_frac"]})
+        line["config"]["also_in_points"] = (line["config"].get("also_in_points", "") + "; the headline shape again: decode "
+                                            "batch 8 at context 32768, prompts of 8192 and 32768 tokens, decode batch 128 at "
+                                            "context 2048, and generation for 64 prompts of 128 tokens with budgets uniform "
+                                            "in 16..512 (greedy, no stop token; tokens/s of the decode phase)").lstrip("; ")
     print(json.dumps(line))
     return 0
 
@@ -99,10 +135,12 @@ def measure(args) -> dict:
     cfg = llm_infer_amd.config_from_dict(raw)
     points = [int(p) for p in args.points.split(",") if p]
     batches = [args.batch] + [p for p in points if p != args.batch]
-    max_tokens = max(max(batches) * args.context, args.prefill_tokens, args.ragged_prefill * 2048) + 64 * max(batches)
+    also_prefill = list(getattr(args, "also_prefill", None) or [])
+    max_tokens = max(max(batches) * args.context, args.prefill_tokens, args.ragged_prefill * 2048,
+                     args.generate * 640, *also_prefill) + 64 * max(batches)
     t0 = time.time()
     engine = llm_infer_amd.random_model(cfg, seed=0, dtype=args.dtype, max_tokens=max_tokens,
-                                        n_slots=max(max(batches), args.ragged_prefill))
+                                        n_slots=max(max(batches), args.ragged_prefill, args.generate))
     torch.cuda.synchronize()
     print(f"[bench] model ready in {time.time() - t0:.1f} s", file=sys.stderr, flush=True)
     model, cache = engine.model, engine.cache
@@ -115,7 +153,9 @@ def measure(args) -> dict:
         for s in spec.shape:
             n *= s
         if name.startswith("model.embed_tokens"):
-            continue                                   # only the batch's rows are read
+            if cfg.tie_word_embeddings:
+                weight_bytes += n * elem               # the tied head reads the whole table
+            continue                                   # else only the batch's rows are read
         weight_bytes += n * (4 if spec.kind == "vector" else elem)
     kv_bytes_per_token = cache.bytes_per_token()
 
@@ -155,24 +195,51 @@ def measure(args) -> dict:
               f"{b * args.steps / dt:.1f} tok/s", file=sys.stderr, flush=True)
 
     # prefill of one prompt
-    T = max(1, args.prefill_tokens)
-    gen = torch.Generator().manual_seed(1)
-    prompt = torch.randint(0, cfg.vocab_size, (T,), generator=gen).tolist()
-    times = []
-    for i in range(4 if args.prefill_tokens > 0 else 2):
-        slot = engine.alloc_slot()
-        torch.cuda.synchronize()
-        t = time.perf_counter()
-        engine.step([slot], [prompt])
-        torch.cuda.synchronize()
-        times.append(time.perf_counter() - t)
-        engine.free_slot(slot)
-    prefill_s = min(times[1:])
     L, d, H, K, hd, F, V = (cfg.num_hidden_layers, cfg.hidden_size, cfg.num_attention_heads,
                             cfg.num_key_value_heads, cfg.head_dim, cfg.intermediate_size, cfg.vocab_size)
-    gemm = 2 * T * (d * (H + 2 * K) * hd + H * hd * d + 3 * d * F) * L + 2 * V * d
-    attn = 2 * H * hd * T * (T + 1) * L
-    prefill_flops = gemm + attn
+
+    def prefill_run(T, repeats):
+        gen = torch.Generator().manual_seed(1)
+        prompt = torch.randint(0, cfg.vocab_size, (T,), generator=gen).tolist()
+        times = []
+        for i in range(repeats):
+            slot = engine.alloc_slot()
+            torch.cuda.synchronize()
+            t = time.perf_counter()
+            engine.step([slot], [prompt])
+            torch.cuda.synchronize()
+            times.append(time.perf_counter() - t)
+            engine.free_slot(slot)
+        flops = 2 * T * (d * (H + 2 * K) * hd + H * hd * d + 3 * d * F) * L + 2 * V * d + 2 * H * hd * T * (T + 1) * L
+        return min(times[1:]), flops
+
+    T = max(1, args.prefill_tokens)
+    prefill_s, prefill_flops = prefill_run(T, (4 if T <= 4096 else 3) if args.prefill_tokens > 0 else 2)
+    more_prefills = {}
+    for n in also_prefill:
+        s_, f_ = prefill_run(n, 3)
+        more_prefills[str(n)] = {"value": round(n / s_, 1), "tokens": n, "ms": round(s_ * 1e3, 3),
+                                 "frac": round(f_ / s_ / PEAK_FLOPS[args.dtype], 4)}
+
+    generation = None
+    if args.generate:
+        # the generation loop itself on a batch whose sequences end at different times: prompts of 128 tokens,
+        # a budget for each request drawn from 16..512, greedy, no stop token
+        gen = torch.Generator().manual_seed(3)
+        prompts = [torch.randint(0, cfg.vocab_size, (128,), generator=gen).tolist() for _ in range(args.generate)]
+        budgets = torch.randint(16, 513, (args.generate,), generator=gen).tolist()
+        engine.generate(prompts[:2], max_new_tokens=4, temperature=0.0, stop_token_ids=())       # first-use work
+        before = dict(engine.decode_counts)
+        _, stats = engine.generate(prompts, max_new_tokens=budgets, temperature=0.0, stop_token_ids=(), return_stats=True)
+        did = {k: engine.decode_counts[k] - before[k] for k in before}
+        steps = max(1, sum(did.values()))
+        # the first token of every request comes out of the prefill step; the decode phase makes the others
+        decoded = stats.generated_tokens - len(prompts)
+        generation = {"prompts": len(prompts), "new_tokens": stats.generated_tokens, "decode_s": round(stats.decode_s, 4),
+                      "prefill_s": round(stats.prefill_s, 4), "tokens_s": round(decoded / stats.decode_s, 1),
+                      "steps_eager": did["eager"], "steps_recorded": did["recorded"], "steps_replayed": did["replayed"],
+                      "replayed_frac": round(did["replayed"] / steps, 4), "mean_batch": round(decoded / steps, 2)}
+        print(f"[bench] generation: {generation}", file=sys.stderr, flush=True)
 
     ragged = None
     if args.ragged_prefill:
@@ -216,11 +283,17 @@ def measure(args) -> dict:
         "prefill": {"value": round(T / prefill_s, 1), "tokens": T, "ms": round(prefill_s * 1e3, 3),
                     "frac": round(prefill_flops / prefill_s / PEAK_FLOPS[args.dtype], 4)},
         "roofline": {"bound": "hbm", "achieved": round(achieved / 1e9, 1), "peak": HBM_BYTES_S / 1e9,
-                     "unit": "GB/s", "frac": round(achieved / HBM_BYTES_S, 4)},
+                     "unit": "GB/s", "frac": round(achieved / HBM_BYTES_S, 4),
+                     "measured_peak": HBM_MEASURED_BYTES_S / 1e9,
+                     "frac_of_measured": round(achieved / HBM_MEASURED_BYTES_S, 4)},
         "points": {f"decode_b{b}": round(b * args.steps / results[b][0], 2) for b in batches if b != args.batch},
     }
     if ragged:
         line["ragged_prefill"] = ragged
+    if more_prefills:
+        line["also_prefill"] = more_prefills
+    if generation:
+        line["generation"] = generation
     del engine, model, cache
     gc.collect()
     torch.cuda.empty_cache()

@@ -9,6 +9,12 @@ which the attention kernels feed the matrix cores.  Pages are zeroed when handed
 out, so nothing of an earlier sequence can be read.  A group with a window gives
 pages back once all their tokens have left the window.
 
+One row more than there are slots lies behind every per-slot table (page tables, lengths, sampling state,
+state groups): the scratch slot, ``Cache.scratch_slot``, which is never handed out.  Its page-table entries
+all point at the null page and its length stays 0.  A recorded decode step that runs more rows than there
+are live sequences (its batch size rounded up to a bucket) lets the idle rows work on that slot: they write
+and read the null page, which no live sequence ever reads, and change nothing else.
+
 The reference keeps one contiguous cache per layer for a single sequence
 (src/model/block.cpp:71-74) and has no per-sequence state beyond the position the
 caller passes (src/model/model.cpp:66-68).
@@ -68,7 +74,8 @@ class KVGroup:
         self._views = {}
         if device is not None:
             self.storage = Tensor.zeros((n_pages, self.page_elems), dtype, device)
-            self.page_table = Tensor.zeros((n_slots, self.max_pages), torch.int32, device)
+            # (one row more: the scratch slot's, all null pages)
+            self.page_table = Tensor.zeros((n_slots + 1, self.max_pages), torch.int32, device)
         else:
             self.storage = self.page_table = None
 
@@ -120,6 +127,16 @@ class KVGroup:
                 self.table_host[slot, p] = NULL_PAGE
             dirty.add(slot)
 
+    def release_from(self, slot: int, length: int, dirty: set) -> None:
+        """Gives back the pages that a sequence of ``length`` tokens does not reach."""
+        have = self.pages_of[slot]
+        gone = [p for p in have if p * PAGE >= length]
+        if gone:
+            self.pool.free([have.pop(p) for p in gone])
+            for p in gone:
+                self.table_host[slot, p] = NULL_PAGE
+            dirty.add(slot)
+
     def release(self, slot: int) -> None:
         have = self.pages_of[slot]
         self.pool.free(list(have.values()))
@@ -145,7 +162,7 @@ class StateGroup:
         dtype = getattr(torch, spec.dtype)
         self.storage = None
         if device is not None:
-            self.storage = Tensor.zeros((len(self.entries), n_slots) + tuple(spec.shape), dtype, device)
+            self.storage = Tensor.zeros((len(self.entries), n_slots + 1) + tuple(spec.shape), dtype, device)
 
     def view(self, entry: int) -> StateView:
         return StateView(self.storage[self.entries.index(entry)], self.spec)
@@ -171,6 +188,7 @@ class Cache:
         self.n_slots = n_slots or max(1, min(self.n_pages - 1, 4096))
         self.device, self.dtype = device, dtype
         self.slots = SlotAllocator(self.n_slots)
+        self.scratch_slot = self.n_slots          # behind the last slot in every per-slot table; never handed out
         self.lens = [0] * self.n_slots
         self.groups = []
         self._group_of = {}
@@ -189,9 +207,9 @@ class Cache:
             for e in entries:
                 self._group_of[e] = g
         if device is not None:
-            self.lens_dev = Tensor.zeros((self.n_slots,), torch.int32, device)
+            self.lens_dev = Tensor.zeros((self.n_slots + 1,), torch.int32, device)
             # fixed-size state of every sequence: key and counter of its sampling generator
-            self.seq_state = Tensor.zeros((self.n_slots, 2), torch.int64, device)
+            self.seq_state = Tensor.zeros((self.n_slots + 1, 2), torch.int64, device)
         else:
             self.lens_dev = self.seq_state = None
 
@@ -237,6 +255,22 @@ class Cache:
         if sync_lens and self.lens_dev is not None and slots:
             idx = torch.tensor(list(slots), dtype=torch.int64, device=self.device)
             self.lens_dev.index_copy_(0, idx, torch.tensor(list(new_lens), dtype=torch.int32, device=self.device))
+
+    def truncate(self, slots, lens) -> None:
+        """Takes sequences back to earlier lengths (a step that failed after ``grow``): the lengths are
+        restored and the pages beyond them given back, so that a later step finds them cleared or fills
+        them itself.  State groups are not restored: what a mixer has already written into its state stays."""
+        for g in self.groups:
+            if isinstance(g, KVGroup):
+                dirty = set()
+                for slot, n in zip(slots, lens):
+                    g.release_from(slot, n, dirty)
+                g.flush(dirty, [])
+        for slot, n in zip(slots, lens):
+            self.lens[slot] = n
+        if self.lens_dev is not None and slots:
+            idx = torch.tensor(list(slots), dtype=torch.int64, device=self.device)
+            self.lens_dev.index_copy_(0, idx, torch.tensor(list(lens), dtype=torch.int32, device=self.device))
 
     def trim_windows(self, slots) -> None:
         for g in self.groups:

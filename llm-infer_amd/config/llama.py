@@ -156,6 +156,11 @@ class LlamaConfig:
                 return f"blk.{layer}.{parts[rest]}.weight"
         return name
 
+    # Tensors that a GGUF file of this architecture may hold without the model using them: the frequency
+    # factors of a rotation scaling that other tools export beside the weights.  The reference binds
+    # tensors by name and never looks at them (src/model/model.cpp:25-38), and applies no such scaling.
+    gguf_ignorable = ("rope_freqs.weight",)
+
     @classmethod
     def from_folder(cls, folder: str) -> "LlamaConfig":
         with open(os.path.join(folder, "config.json")) as f:

@@ -77,6 +77,17 @@ __device__ __forceinline__ float block_max(float v, float* scratch) {
     return t;
 }
 
+// A power of two near 1 / (8 rms) for a row whose root mean square is `rms`: what the rows of a residual
+// stream are multiplied by before they are rounded to float16 on their way from one product to the norm
+// inside the next (gemm.hip, RowsOut), so that they lie in the middle of that type's range whatever the
+// model's own scale.  An element is at most sqrt(width) times the rms, so a row that has grown a hundredfold
+// since the rms was taken still fits.
+__device__ __forceinline__ float row_scale_for(float rms) {
+    int e;
+    frexpf(fminf(fmaxf(rms, 1e-30f), 1e30f), &e);        // rms = m 2^e, 0.5 <= m < 1
+    return ldexpf(0.125f, -e);
+}
+
 // The gate's activation: silu(x) = x / (1 + exp(-x)) (include/kernels_cpu.hpp:186) or the tanh form of
 // gelu that the reference computes, 0.5 x (1 + tanh(sqrt(2 / pi) (x + 0.044715 x^3)))
 // (include/kernels_cpu.hpp:179-184).

@@ -34,9 +34,12 @@ extern "C" int li_embed(const void* table, int table_dt, const int* tokens, floa
 // out[r, :] = x[row(r), :] / sqrt(mean(x^2) + eps) * w     (include/kernels_cpu.hpp:43-54)
 // Sum of squares, root and scaling in float32; `rows` (may be null) picks rows.
 // ---------------------------------------------------------------------------
+// `row_scale` (may be null): row_scale_for(rms) of the first 16 rows, for a product that will add into these
+// rows and hand them on in float16 (gemm.hip, RowsOut).
 template <class TO>
 __global__ void rmsnorm_kernel(const float* __restrict__ x, const float* __restrict__ w,
-                               const int* __restrict__ rows, TO* __restrict__ out, int d, float eps) {
+                               const int* __restrict__ rows, TO* __restrict__ out, int d, float eps,
+                               float* __restrict__ row_scale) {
     __shared__ float scratch[16];
     const int r = blockIdx.x;
     const float* xr = x + (int64_t)(rows ? rows[r] : r) * d;
@@ -45,6 +48,7 @@ __global__ void rmsnorm_kernel(const float* __restrict__ x, const float* __restr
     for (int i = threadIdx.x; i < d; i += blockDim.x) { const float v = xr[i]; ss += v * v; }
     ss = block_sum(ss, scratch);
     const float rms = sqrtf(ss / (float)d + eps);
+    if (row_scale && threadIdx.x == 0 && r < 16) row_scale[r] = row_scale_for(rms);
     for (int i = threadIdx.x; i < d; i += blockDim.x) o[i] = from_f32<TO>(xr[i] / rms * w[i]);
 }
 
@@ -52,7 +56,8 @@ __global__ void rmsnorm_kernel(const float* __restrict__ x, const float* __restr
 // pointers): the row and its weights are read once, in 16-byte pieces that stay in registers.
 template <class TO, int V>
 __global__ void rmsnorm_vec_kernel(const float* __restrict__ x, const float* __restrict__ w,
-                                   const int* __restrict__ rows, TO* __restrict__ out, int d, float eps) {
+                                   const int* __restrict__ rows, TO* __restrict__ out, int d, float eps,
+                                   float* __restrict__ row_scale) {
     struct alignas(4 * sizeof(TO)) Out4 { TO v[4]; };
     __shared__ float scratch[16];
     const int r = blockIdx.x, n4 = d >> 2;
@@ -77,6 +82,7 @@ __global__ void rmsnorm_vec_kernel(const float* __restrict__ x, const float* __r
         for (int q = 0; q < 4; ++q) ss += xv[j][q] * xv[j][q];
     ss = block_sum(ss, scratch);
     const float rms = sqrtf(ss / (float)d + eps);
+    if (row_scale && threadIdx.x == 0 && r < 16) row_scale[r] = row_scale_for(rms);
 #pragma unroll
     for (int j = 0; j < V; ++j) {
         const int i = threadIdx.x + j * blockDim.x;
@@ -90,7 +96,7 @@ __global__ void rmsnorm_vec_kernel(const float* __restrict__ x, const float* __r
 }
 
 extern "C" int li_rmsnorm(const float* x, const float* w, const int* rows, void* out, int out_dt,
-                          int n_rows, int d, float eps, hipStream_t stream) {
+                          int n_rows, int d, float eps, float* row_scale, hipStream_t stream) {
     if (n_rows <= 0) return LI_OK;
     if (d <= 0) return LI_BAD_ARG;
     if (out_dt != DT_F32 && out_dt != DT_F16 && out_dt != DT_BF16) return LI_BAD_ARG;
@@ -102,16 +108,16 @@ extern "C" int li_rmsnorm(const float* x, const float* w, const int* rows, void*
         const bool two = n4 <= 2 * threads;
 #define GO(TO)                                                                                             \
     do {                                                                                                   \
-        if (two) rmsnorm_vec_kernel<TO, 2><<<grid, threads, 0, stream>>>(x, w, rows, (TO*)out, d, eps);    \
-        else rmsnorm_vec_kernel<TO, 4><<<grid, threads, 0, stream>>>(x, w, rows, (TO*)out, d, eps);        \
+        if (two) rmsnorm_vec_kernel<TO, 2><<<grid, threads, 0, stream>>>(x, w, rows, (TO*)out, d, eps, row_scale); \
+        else rmsnorm_vec_kernel<TO, 4><<<grid, threads, 0, stream>>>(x, w, rows, (TO*)out, d, eps, row_scale);     \
     } while (0)
         if (out_dt == DT_F32) GO(float); else if (out_dt == DT_F16) GO(f16); else GO(bf16);
 #undef GO
     } else {
         dim3 block(d >= 2048 ? 512 : (d >= 512 ? 256 : 64));
-        if (out_dt == DT_F32) rmsnorm_kernel<float><<<grid, block, 0, stream>>>(x, w, rows, (float*)out, d, eps);
-        else if (out_dt == DT_F16) rmsnorm_kernel<f16><<<grid, block, 0, stream>>>(x, w, rows, (f16*)out, d, eps);
-        else rmsnorm_kernel<bf16><<<grid, block, 0, stream>>>(x, w, rows, (bf16*)out, d, eps);
+        if (out_dt == DT_F32) rmsnorm_kernel<float><<<grid, block, 0, stream>>>(x, w, rows, (float*)out, d, eps, row_scale);
+        else if (out_dt == DT_F16) rmsnorm_kernel<f16><<<grid, block, 0, stream>>>(x, w, rows, (f16*)out, d, eps, row_scale);
+        else rmsnorm_kernel<bf16><<<grid, block, 0, stream>>>(x, w, rows, (bf16*)out, d, eps, row_scale);
     }
     LI_CHECK_LAUNCH();
     return LI_OK;
@@ -225,22 +231,40 @@ extern "C" int li_rope_table(const float* inv_freq, const int* pos, float* out, 
 // ---------------------------------------------------------------------------
 // Bookkeeping of one decode step, on the device so that a captured step can be
 // replayed: each sequence's new token gets the position lens[slot], the
-// sequence's context grows by one.
+// sequence's context grows by one.  A row on `scratch_slot` is an idle row of a
+// step that runs more rows than there are live sequences: position 0, a context
+// of one token, and no length is changed.  With `cos_sin` (may be null) the same
+// kernel fills the table of rotation angles of the step, [n, n_freq, 2] = cos and
+// sin of pos * inv_freq as rope_table_kernel does, so that a step needs no
+// second small kernel before its first layer.
 // ---------------------------------------------------------------------------
 __global__ void decode_prepare_kernel(const int* __restrict__ seq_slot, int* __restrict__ lens,
-                                      int* __restrict__ pos, int* __restrict__ ctx, int n) {
-    const int i = blockIdx.x * blockDim.x + threadIdx.x;
-    if (i >= n) return;
+                                      int* __restrict__ pos, int* __restrict__ ctx, int n, int scratch_slot,
+                                      const float* __restrict__ inv_freq, float* __restrict__ cos_sin, int n_freq) {
+    // one workgroup a row: thread 0 does the bookkeeping, all threads the row's angles
+    const int i = blockIdx.x;
     const int s = seq_slot[i];
-    const int l = lens[s];
-    pos[i] = l;
-    ctx[i] = l + 1;
-    lens[s] = l + 1;
+    const int l = s == scratch_slot ? 0 : lens[s];
+    __syncthreads();                                  // every thread has read the length before it changes
+    if (threadIdx.x == 0) {
+        pos[i] = l;
+        ctx[i] = l + 1;
+        if (s != scratch_slot) lens[s] = l + 1;
+    }
+    if (cos_sin)
+        for (int j = threadIdx.x; j < n_freq; j += blockDim.x) {
+            float sn, cs;
+            sincosf((float)l * inv_freq[j], &sn, &cs);
+            cos_sin[2 * ((int64_t)i * n_freq + j)] = cs;
+            cos_sin[2 * ((int64_t)i * n_freq + j) + 1] = sn;
+        }
 }
 
-extern "C" int li_decode_prepare(const int* seq_slot, int* lens, int* pos, int* ctx, int n, hipStream_t stream) {
+extern "C" int li_decode_prepare(const int* seq_slot, int* lens, int* pos, int* ctx, int n, int scratch_slot,
+                                 const float* inv_freq, float* cos_sin, int n_freq, hipStream_t stream) {
     if (n <= 0) return LI_OK;
-    decode_prepare_kernel<<<(n + 255) / 256, 256, 0, stream>>>(seq_slot, lens, pos, ctx, n);
+    if (cos_sin && (!inv_freq || n_freq <= 0)) return LI_BAD_ARG;
+    decode_prepare_kernel<<<n, 64, 0, stream>>>(seq_slot, lens, pos, ctx, n, scratch_slot, inv_freq, cos_sin, n_freq);
     LI_CHECK_LAUNCH();
     return LI_OK;
 }

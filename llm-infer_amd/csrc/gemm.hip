@@ -297,18 +297,24 @@ __global__ void tile_weight_kernel(const T* __restrict__ W, T* __restrict__ out,
 // x next (RowsOut).  The next product takes `xw` as its X and multiplies its sums by
 // 1 / (scale * sqrt(mean(x^2) + eps)) from the partial sums (RowScale): together  W . (x / rms * w),
 // the norm of include/kernels_cpu.hpp:43-54 in another order of rounding.  `scale` keeps x * w inside
-// float16's range.
+// float16's range: one power of two for each row, near 1 / (8 rms) of the row as it was when a norm was last
+// taken of it (`row_scale`, written by the norm kernel or by the product that finished that norm:
+// row_scale_for in common.h), so that the rounding is as fine for a model whose residual stream is of the
+// order of 0.01 or 1000 as for one of the order of 1; without it the fixed `scale`.
 struct RowsOut {
     float* ss;               // [gridDim.x, 16]
     void* xw;                // [M, N] in the product's 16-bit type
     const float* w;          // [N] weight of the next norm
     float scale;
+    const float* row_scale;  // [16] or null
 };
 struct RowScale {
     const float* ss;         // [P, 16]
     int P;
     float eps;               // of the norm
     float inv_scale;         // 1 / RowsOut.scale
+    const float* row_scale;  // [16] the scales RowsOut used, or null (then inv_scale)
+    float* next_scale;       // [16] or null: row_scale_for(rms) of these rows, for the product that adds into them next
 };
 
 template <class T, int NT, int MT, int KW>
@@ -405,7 +411,9 @@ __global__ __launch_bounds__(64 * KW) void gemv_tiled_kernel(const T* __restrict
         // this lane's row: the waves' sums in wave order, then 1 / (scale * rms)
         float ss = ss_wave[0][r];
         for (int w = 1; w < KW; ++w) ss += ss_wave[w][r];
-        const float f = rsc.inv_scale / sqrtf(ss / (float)K + rsc.eps);
+        const float rms = sqrtf(ss / (float)K + rsc.eps);
+        const float f = (rsc.row_scale ? 1.f / rsc.row_scale[r] : rsc.inv_scale) / rms;
+        if (rsc.next_scale && blockIdx.x == 0 && g == 0) rsc.next_scale[r] = row_scale_for(rms);
 #pragma unroll
         for (int t = 0; t < NT; ++t)
 #pragma unroll
@@ -418,6 +426,7 @@ __global__ __launch_bounds__(64 * KW) void gemv_tiled_kernel(const T* __restrict
         for (int j = 0; j < MT; ++j) {
             sq[j] = 0.f;
             const int m = 16 * j + r;
+            const float scale = ro.row_scale ? ro.row_scale[m & 15] : ro.scale;
 #pragma unroll
             for (int t = 0; t < NT; ++t) {
                 const int n = (tile0 + t) * 16 + 4 * g;
@@ -430,7 +439,7 @@ __global__ __launch_bounds__(64 * KW) void gemv_tiled_kernel(const T* __restrict
                     for (int q = 0; q < 4; ++q) {
                         o[q] += acc[t][j][q];
                         sq[j] = fmaf(o[q], o[q], sq[j]);
-                        xw[q] = from_f32<T>(o[q] * wv[q] * ro.scale);
+                        xw[q] = from_f32<T>(o[q] * wv[q] * scale);
                     }
                     *(f32x4*)c = o;
                     *(typename Vec<T>::v4*)((T*)ro.xw + (int64_t)m * e.N + n) = xw;

@@ -50,12 +50,27 @@ class _GraphContext(StepShared):
 MAX_RECORDED_STEPS = 48        # recorded steps an engine keeps; the least recently used goes first
 
 
+def batch_bucket(n: int, limit: int) -> int:
+    """The number of rows a recorded step runs for ``n`` live sequences: the next of 1, 2, 4, 8, 12, 16, 24,
+    32, 48, 64, 96, ... (powers of two and the sizes half-way between them), at most ``limit``; the rows beyond
+    ``n`` are idle rows on the cache's scratch slot.  A batch that shrinks from 64 sequences to 1 so meets ten
+    sizes instead of 64, each of them often enough to be worth recording."""
+    b = 1
+    while b < n:
+        b = b * 2 if b < 8 else (b // 2 * 3 if b & (b - 1) == 0 else b // 3 * 4)
+    return max(n, min(b, limit))
+
+
 class GraphDecodeRunner:
     """Replays a recorded step while the set of live sequences stays the same; when it
     changes, the slots and tokens are uploaded anew and the graph of the new size is used.
-    A step is run eagerly the first time its (batch size, bucket of context lengths, sampling mode)
-    is seen and recorded the second time; the temperature is read from the device, so it is no part
-    of the key.  An engine keeps at most MAX_RECORDED_STEPS recorded steps."""
+    A step is keyed by (rows, bucket of context lengths, sampling mode): the rows are the number of live
+    sequences rounded up to a ``batch_bucket`` (idle rows run on the cache's scratch slot and their tokens
+    are dropped); the temperature is read from the device, so it is no part of the key.  The first step of an
+    engine is run eagerly (whatever is built or loaded at first use must not happen while a graph is being
+    recorded) and recorded when its key comes again; every later key is recorded when it is first seen.  An
+    engine keeps at most MAX_RECORDED_STEPS recorded steps and counts what it did in ``engine.decode_counts``
+    (steps run eagerly, steps recorded, steps replayed)."""
 
     def __init__(self, engine, sampler):
         self.engine, self.sampler = engine, sampler
@@ -64,59 +79,72 @@ class GraphDecodeRunner:
         dev = engine.device
         self.bufs = engine._graph_bufs
         if self.bufs is None:
-            self.bufs = {k: torch.zeros((n,), dtype=torch.int32, device=dev)
-                         for k in ("tokens", "slots", "pos", "ctx", "next")}
+            self.bufs = {k: torch.zeros((n,), dtype=torch.int32, device=dev) for k in ("tokens", "slots", "pos", "ctx")}
             self.bufs["rows"] = torch.arange(n, dtype=torch.int32, device=dev)
             self.bufs["temperature"] = torch.ones((1,), dtype=torch.float32, device=dev)
             # where the tokens of the steps in flight arrive on the host
             self.bufs["host"] = [Tensor.pinned((n,), torch.int32) for _ in range(3)]
             self.bufs["done"] = [torch.cuda.Event() for _ in range(3)]
             engine._graph_bufs = self.bufs
-        self.current = None            # the slots now in the buffers
+        self.current = None            # the rows' slots now in the buffers
         self._ahead = None             # a step enqueued before its predecessor's tokens were read
         self._fed = None               # slot -> the token that step was fed on the device
         self._host, self._done = self.bufs["host"], self.bufs["done"]
         self._turn = 0
+        # one table of rotation angles for the whole model: the bookkeeping kernel fills it
+        wanted = [p.step_table() for p in engine.model.positions.values() if hasattr(p, "step_table")]
+        wanted = [w for w in wanted if w is not None]
+        self._table = wanted[0] if len(wanted) == 1 else None
 
     def _body(self, n, bucket):
         eng, b = self.engine, self.bufs
-        ops.decode_prepare(b["slots"], eng.cache.lens_dev, b["pos"], b["ctx"], n)
         ctx = _GraphContext(b, n, bucket)
+        table = ops.decode_prepare(b["slots"], eng.cache.lens_dev, b["pos"], b["ctx"], n, eng.cache.scratch_slot,
+                                   self._table[1] if self._table else None)
+        if table is not None:
+            ctx.shared(self._table[0], lambda: table)
         logits = eng.model.forward(ctx, eng.cache)
-        self.sampler.sample(logits, b["slots"][:n], eng.cache, out=b["next"], temperature_dev=b["temperature"])
-        b["tokens"][:n].copy_(b["next"][:n])
+        # the sampled tokens go where the next step reads its tokens (the copy to the host is enqueued
+        # between the two steps)
+        self.sampler.sample(logits, b["slots"][:n], eng.cache, out=b["tokens"], temperature_dev=b["temperature"])
 
     def _launch(self, slots, tokens):
         """Enqueues one step for ``slots`` and the copy of its tokens to pinned host memory.
         ``tokens`` None: the tokens the step before left on the device are fed."""
         eng, cache, b = self.engine, self.engine.cache, self.bufs
         n = len(slots)
+        rows = batch_bucket(n, cache.n_slots)
         new_lens = [cache.lens[s] + 1 for s in slots]
         cache.grow(slots, new_lens, sync_lens=False)
-        if self.current != list(slots):
+        padded = list(slots) + [cache.scratch_slot] * (rows - n)
+        if self.current != padded:
             if tokens is None:
                 raise RuntimeError("a new set of sequences needs its tokens")
-            b["slots"][:n].copy_(torch.tensor(slots, dtype=torch.int32))
-            b["tokens"][:n].copy_(torch.tensor(tokens, dtype=torch.int32))
-            self.current = list(slots)
+            b["slots"][:rows].copy_(torch.tensor(padded, dtype=torch.int32))
+            b["tokens"][:rows].copy_(torch.tensor(list(tokens) + [0] * (rows - n), dtype=torch.int32))
+            self.current = padded
         bucket = split_bucket(max(new_lens))
         hot = self.sampler.temperature > 0.0
         if hot and b.get("temperature_value") != self.sampler.temperature:
             b["temperature"].fill_(self.sampler.temperature)
             b["temperature_value"] = self.sampler.temperature
-        key = (n, bucket, hot)
-        graphs = eng._graphs
+        key = (rows, bucket, hot)
+        graphs, counts = eng._graphs, eng.decode_counts
         entry = graphs.pop(key, None)            # taken out and put back: the dict is in order of last use
-        if entry is None:
-            self._body(n, bucket)
+        if entry is None and not graphs:
+            self._body(rows, bucket)             # the engine's first decode step
             entry = "seen"
+            counts["eager"] += 1
         else:
-            if entry == "seen":
+            if entry is None or entry == "seen":
                 g = torch.cuda.CUDAGraph()
                 torch.cuda.synchronize()
                 with torch.cuda.graph(g):
-                    self._body(n, bucket)
+                    self._body(rows, bucket)
                 entry = g
+                counts["recorded"] += 1
+            else:
+                counts["replayed"] += 1
             entry.replay()
         graphs[key] = entry
         while len(graphs) > MAX_RECORDED_STEPS:
@@ -126,7 +154,7 @@ class GraphDecodeRunner:
             del graphs[old]
         self._turn = (self._turn + 1) % len(self._host)
         host, done = self._host[self._turn], self._done[self._turn]
-        host[:n].copy_(b["next"][:n], non_blocking=True)
+        host[:n].copy_(b["tokens"][:n], non_blocking=True)
         done.record()
         return list(slots), host, done
 

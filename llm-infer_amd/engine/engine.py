@@ -55,6 +55,7 @@ class Engine:
                            as_dtype(kv_round) if kv_round else None)
         self._graphs = {}
         self._graph_bufs = None
+        self.decode_counts = {"eager": 0, "recorded": 0, "replayed": 0}      # what the recorded-step runner did
 
     # -- construction ----------------------------------------------------------
     @classmethod
@@ -120,7 +121,13 @@ class Engine:
         want[i]: places among these tokens whose logits are returned (default: the last).
         Returns float32 [sum(len(want[i])), vocab] in the order of the sequences and of want."""
         ctx = self.prepare(slots, tokens, want)
-        logits = self.model.forward(ctx, self.cache)
+        try:
+            logits = self.model.forward(ctx, self.cache)
+        except Exception:
+            # a kernel refused its operands: the sequences are as long as before the step, and the pages
+            # the step took are given back
+            self.cache.truncate(slots, ctx.host_lens_before)
+            raise
         self.cache.trim_windows(slots)
         return logits
 

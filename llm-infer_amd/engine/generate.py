@@ -18,17 +18,28 @@ class RequestError(ValueError):
     pass
 
 
-def plan_batches(prompt_lens, max_new_tokens: int, max_batch: int, capacity_tokens: int, max_positions: int):
+def per_request(value, n: int, what: str = "max_new_tokens") -> list:
+    """One number for every request, or a list with one for each."""
+    if isinstance(value, (list, tuple)):
+        if len(value) != n:
+            raise RequestError(f"{what}: {len(value)} values for {n} requests")
+        return [int(v) for v in value]
+    return [int(value)] * n
+
+
+def plan_batches(prompt_lens, max_new_tokens, max_batch: int, capacity_tokens: int, max_positions: int):
     """Cuts the requests, in their order, into batches that fit the slots and the cache.
-    A request holds room for its prompt and all it may generate, rounded up to whole pages."""
+    A request holds room for its prompt and all it may generate (``max_new_tokens``: one number, or one for
+    each request), rounded up to whole pages."""
     batches, cur, used = [], [], 0
+    budget = per_request(max_new_tokens, len(prompt_lens))
     for i, n in enumerate(prompt_lens):
         if n <= 0:
             raise RequestError(f"request {i} has an empty prompt")
         if n >= max_positions:
             # tools/infer.cpp:262-265
             raise RequestError(f"Prompt too long: {n} tokens (max: {max_positions})")
-        need = -(-min(n + max_new_tokens, max_positions) // PAGE) * PAGE
+        need = -(-min(n + budget[i], max_positions) // PAGE) * PAGE
         if need > capacity_tokens:
             raise RequestError(f"request {i} needs room for {need} tokens, the cache holds {capacity_tokens}")
         if cur and (len(cur) >= max_batch or used + need > capacity_tokens):
@@ -51,9 +62,10 @@ class BatchTracker:
 
     def __init__(self, prompt_lens, max_new_tokens, stop_token_ids, max_positions):
         self.prompt_lens = list(prompt_lens)
-        self.max_new, self.stop, self.max_positions = max_new_tokens, set(stop_token_ids or ()), max_positions
+        self.max_new = per_request(max_new_tokens, len(self.prompt_lens))     # a budget for each request
+        self.stop, self.max_positions = set(stop_token_ids or ()), max_positions
         self.outputs = [[] for _ in prompt_lens]
-        self.finished = [max_new_tokens <= 0 for _ in prompt_lens]
+        self.finished = [m <= 0 for m in self.max_new]
         self.reason = ["length" if f else None for f in self.finished]
 
     def live(self):
@@ -61,7 +73,7 @@ class BatchTracker:
 
     def will_go_on(self, live) -> bool:
         """True if every live request goes on after its next token unless that is a stop token."""
-        return all(len(self.outputs[i]) + 1 < self.max_new and
+        return all(len(self.outputs[i]) + 1 < self.max_new[i] and
                    self.prompt_lens[i] + len(self.outputs[i]) + 1 <= self.max_positions for i in live)
 
     def accept(self, live, sampled):
@@ -73,7 +85,7 @@ class BatchTracker:
                 self.finished[i], self.reason[i] = True, "stop"
                 continue
             self.outputs[i].append(int(t))
-            if len(self.outputs[i]) >= self.max_new:
+            if len(self.outputs[i]) >= self.max_new[i]:
                 self.finished[i], self.reason[i] = True, "length"
             elif self.prompt_lens[i] + len(self.outputs[i]) > self.max_positions:
                 self.finished[i], self.reason[i] = True, "context"
@@ -92,10 +104,11 @@ class GenerationStats:
     finish_reasons: list = field(default_factory=list)
 
 
-def generate(engine, prompts, max_new_tokens: int = 256, temperature: float = 1.0, seed: int = 0,
+def generate(engine, prompts, max_new_tokens=256, temperature: float = 1.0, seed: int = 0,
              stop_token_ids=None, max_batch: int | None = None, return_stats: bool = False,
              use_graph: bool = True):
-    """Generates for every prompt (a list of token ids); returns the new tokens of each, in order."""
+    """Generates for every prompt (a list of token ids); returns the new tokens of each, in order.
+    ``max_new_tokens``: one budget for all requests, or a list with one for each."""
     if stop_token_ids is None:
         stop_token_ids = engine.model.spec.stop_token_ids
     cache = engine.cache
@@ -104,15 +117,18 @@ def generate(engine, prompts, max_new_tokens: int = 256, temperature: float = 1.
         if len(p) and (min(p) < 0 or max(p) >= engine.vocab_size):
             raise RequestError(f"request {i}: token id outside [0, {engine.vocab_size})")
     capacity = (cache.n_pages - 1) * PAGE
+    max_new_tokens = per_request(max_new_tokens, len(prompts))
     batches = plan_batches([len(p) for p in prompts], max_new_tokens, max_batch, capacity, engine.max_positions)
     sampler = Sampler(temperature, seed)
     outputs = [None] * len(prompts)
     stats = GenerationStats(finish_reasons=[None] * len(prompts))
     for batch in batches:
-        slots = [engine.alloc_slot() for _ in batch]
+        slots = []
         try:
-            tracker = BatchTracker([len(prompts[r]) for r in batch], max_new_tokens, stop_token_ids,
-                                   engine.max_positions)
+            for _ in batch:                      # inside the try: a slot that cannot be had leaks none of the others
+                slots.append(engine.alloc_slot())
+            tracker = BatchTracker([len(prompts[r]) for r in batch], [max_new_tokens[r] for r in batch],
+                                   stop_token_ids, engine.max_positions)
             sampler.start(cache, slots, batch)
             live = tracker.live()
             if live:

@@ -54,7 +54,7 @@ def describe(path: str, n_list: int = 12, out=sys.stdout) -> int:
         say(f"  ... and {len(names) - n_list} more")
     status = 0
     try:
-        check_tensors(needed, ckpt, model.ignorable_names() + ["rope_freqs.weight"])
+        check_tensors(needed, ckpt, model.ignorable_names() + list(getattr(config, "gguf_ignorable", ())))
         say("The tensors fit the model.")
     except (WeightError, ValueError) as e:
         say(str(e))

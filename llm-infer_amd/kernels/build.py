@@ -99,7 +99,10 @@ def _run(cmd, what):
 
 # Kernels that count their own loads in flight (waits placed by hand): a register spilled by the compiler
 # would be a load that they do not count, so a build in which they use scratch memory is refused.
-NO_SCRATCH = {"gemm_prefill.hip": "gemm_wreg_kernel"}
+# (gemm_wreg: W into a ring of registers by global_load_dwordx4; attn_prefill: the fragments of a page out of
+# LDS by ds_read_b128; both written as instructions whose results the compiler knows nothing about until the
+# hand-counted wait.)
+NO_SCRATCH = {"gemm_prefill.hip": "gemm_wreg_kernel", "attention.hip": "attn_prefill_kernel"}
 
 
 def _check_no_scratch(report: str, kernel: str, src: str) -> None:

@@ -96,17 +96,25 @@ def rmsnorm(x: torch.Tensor, w: torch.Tensor, eps: float, out_dtype, rows: torch
     else:
         n = x.shape[0]
     out = torch.empty((n, x.shape[1]), dtype=out_dtype, device=x.device)
+    # for the few rows of a decode step in float16: a power of two near 1 / (8 rms) of each row, for the product
+    # that adds into these rows next and hands them on in 16 bits (see LazyNorm)
+    row_scale = None
+    if rows is None and n <= 16 and out_dtype == torch.float16:
+        row_scale = torch.empty((16,), dtype=torch.float32, device=x.device)
     _check(core().li_rmsnorm(_ptr(x), _ptr(w), _ptr(rows), _ptr(out), DT[out_dtype], n, x.shape[1],
-                             c_float(eps), _stream()), "rmsnorm")
+                             c_float(eps), _ptr(row_scale), _stream()), "rmsnorm")
+    if row_scale is not None:
+        x._li_row_scale = row_scale
     return out
 
 
 class _RowsOut(ctypes.Structure):
-    _fields_ = [("ss", c_void_p), ("xw", c_void_p), ("w", c_void_p), ("scale", c_float)]
+    _fields_ = [("ss", c_void_p), ("xw", c_void_p), ("w", c_void_p), ("scale", c_float), ("row_scale", c_void_p)]
 
 
 class _RowScale(ctypes.Structure):
-    _fields_ = [("ss", c_void_p), ("P", c_int), ("eps", c_float), ("inv_scale", c_float)]
+    _fields_ = [("ss", c_void_p), ("P", c_int), ("eps", c_float), ("inv_scale", c_float), ("row_scale", c_void_p),
+                ("next_scale", c_void_p)]
 
 
 class LazyNorm:
@@ -114,11 +122,18 @@ class LazyNorm:
     last added into the float32 rows ``x`` also left ``xw`` = x * weight * scale in the 16-bit type and
     the rows' sums of squares as partial sums ``ss`` [P, 16]; the product that reads the norm takes
     ``xw`` as its X and multiplies its sums by 1 / (scale * rms).  ``linear`` does that where its kernel
-    can (up to 16 rows against a tiled weight); everywhere else ``tensor()`` runs the norm kernel."""
+    can (up to 16 rows against a tiled weight); everywhere else ``tensor()`` runs the norm kernel.
 
-    def __init__(self, x, weight, eps, dtype, xw, ss, scale):
+    ``scale`` keeps x * weight inside float16's range (bfloat16 has float32's and takes 1).  A fixed factor
+    cannot: a residual stream of the order of 0.01 under norm weights of 0.02 would fall below float16's
+    normal numbers, one of the order of 1000 above its largest.  So in float16 each row has a power of two of its
+    own, ``row_scales`` [16]: near 1 / (8 rms) of the row when a norm was last taken of it (by the norm kernel, or
+    by the product that finished the norm before this one, which leaves the next one's scales on the residual
+    tensor as ``_li_row_scale``); rows about which nothing is known take the fixed ``scale``."""
+
+    def __init__(self, x, weight, eps, dtype, xw, ss, scale, row_scales=None):
         self.x, self.weight, self.eps, self.dtype = x, weight, float(eps), dtype
-        self.xw, self.ss, self.scale = xw, ss, float(scale)
+        self.xw, self.ss, self.scale, self.row_scales = xw, ss, float(scale), row_scales
         self.shape, self.device = x.shape, x.device
 
     def dim(self):
@@ -138,10 +153,15 @@ def expect_norm(x: torch.Tensor, weight, eps: float | None = None) -> None:
 
 
 def _drop_row_stats(x) -> None:
-    if x is not None and getattr(x, "_li_rows", None) is not None:
-        x._li_rows = None
-    if x is not None and getattr(x, "_li_normed", None) is not None:
-        x._li_normed = None
+    """Whatever a kernel of this library is about to write into ``x``, what was prepared for a norm of its rows
+    is void: on ``x`` itself and, if ``x`` is a view (``out=rows[:n]``), on the tensor it is a view of, whose
+    ``_version`` a write through ctypes does not move."""
+    while x is not None:
+        if getattr(x, "_li_rows", None) is not None:
+            x._li_rows = None
+        if getattr(x, "_li_normed", None) is not None:
+            x._li_normed = None
+        x = getattr(x, "_base", None)
 
 
 def prepared_rmsnorm(x: torch.Tensor, w: torch.Tensor, eps: float, out_dtype):
@@ -165,10 +185,10 @@ def lazy_rmsnorm(x: torch.Tensor, w: torch.Tensor, eps: float, out_dtype):
     rec = getattr(x, "_li_rows", None)
     if rec is None:
         return None
-    xw, ss, scale, weight, version = rec
+    xw, ss, scale, weight, version, row_scales = rec
     if weight is not w or version != x._version or xw.dtype != out_dtype or xw.shape != x.shape:
         return None
-    return LazyNorm(x, w, eps, out_dtype, xw, ss, scale)
+    return LazyNorm(x, w, eps, out_dtype, xw, ss, scale, row_scales)
 
 
 class _NormAfter(ctypes.Structure):
@@ -276,14 +296,22 @@ def linear(x: torch.Tensor, w, mode: int = EPI_STORE, out: torch.Tensor | None =
                 ss = torch.empty((lib.li_gemv_tiled_blocks(m, n, k, 0, 0), 16), dtype=torch.float32, device=x.device)
                 xw = torch.empty((m, n), dtype=x.dtype, device=x.device)
                 scale = 0.125 if x.dtype == torch.float16 else 1.0        # x * w stays inside float16's range
-                ro = _RowsOut(ss.data_ptr(), xw.data_ptr(), nxt.data_ptr(), scale)
+                row_scales = getattr(out, "_li_row_scale", None) if x.dtype == torch.float16 else None
+                ro = _RowsOut(ss.data_ptr(), xw.data_ptr(), nxt.data_ptr(), scale,
+                              row_scales.data_ptr() if row_scales is not None else None)
             if lazy is not None:
-                rsc = _RowScale(lazy.ss.data_ptr(), lazy.ss.shape[0], lazy.eps, 1.0 / lazy.scale)
+                # in float16 the kernel also leaves the scales for the product that adds into these rows next
+                nxt_scale = torch.empty((16,), dtype=torch.float32, device=x.device) if x.dtype == torch.float16 else None
+                rsc = _RowScale(lazy.ss.data_ptr(), lazy.ss.shape[0], lazy.eps, 1.0 / lazy.scale,
+                                lazy.row_scales.data_ptr() if lazy.row_scales is not None else None,
+                                nxt_scale.data_ptr() if nxt_scale is not None else None)
+                if nxt_scale is not None:
+                    lazy.x._li_row_scale = nxt_scale
             _check(lib.li_gemv_tiled(_ptr(x), _ptr(wd), DT[x.dtype], _ptr(out), out_dt, mode, m, n, k, 0, 0, rs,
                                      ctypes.byref(ro) if ro is not None else None,
                                      ctypes.byref(rsc) if rsc is not None else None, _stream()), "gemv_tiled")
             if ro is not None:
-                out._li_rows = (xw, ss, scale, nxt, out._version)
+                out._li_rows = (xw, ss, scale, nxt, out._version, row_scales)
             return out
         _need(lazy is None, "a norm is finished by gemv_tiled alone")
         if force is None and m * k * 2 < (1 << 32):
@@ -465,12 +493,23 @@ def linear_rope_store(x, w, inv_freq, rotary_dim, pos, tok_slot, page_table, pag
     return q
 
 
-def decode_prepare(seq_slot, lens, pos, ctx, n):
-    _dev(seq_slot, lens, pos, ctx)
+def decode_prepare(seq_slot, lens, pos, ctx, n, scratch_slot: int = -1, inv_freq=None):
+    """The bookkeeping of a decode step on the device: row i's token gets position lens[seq_slot[i]], its
+    context is one more, the length grows by one; a row on ``scratch_slot`` (an idle row) gets position 0 and
+    changes no length.  With ``inv_freq`` the kernel also fills and returns the step's table of angles
+    (what ``rope_table`` computes from these positions)."""
+    _dev(seq_slot, lens, pos, ctx, inv_freq)
     for a in (seq_slot, lens, pos, ctx):
         _need(a.dtype == torch.int32, "decode_prepare: int32 arrays")
     _need(seq_slot.numel() >= n and pos.numel() >= n and ctx.numel() >= n, "decode_prepare: arrays too short")
-    _check(core().li_decode_prepare(_ptr(seq_slot), _ptr(lens), _ptr(pos), _ptr(ctx), n, _stream()), "decode_prepare")
+    table = None
+    if inv_freq is not None:
+        _need(inv_freq.dtype == torch.float32 and inv_freq.numel() > 0, "decode_prepare: float32 frequencies")
+        table = torch.empty((n, inv_freq.numel(), 2), dtype=torch.float32, device=inv_freq.device)
+    _check(core().li_decode_prepare(_ptr(seq_slot), _ptr(lens), _ptr(pos), _ptr(ctx), n, int(scratch_slot),
+                                    _ptr(inv_freq), _ptr(table), inv_freq.numel() if inv_freq is not None else 0,
+                                    _stream()), "decode_prepare")
+    return table
 
 
 # ---------------------------------------------------------------------------

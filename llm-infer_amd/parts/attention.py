@@ -45,9 +45,13 @@ class Attention(Part):
         return {"q_proj.weight": ParamSpec((h * hd, d)), "k_proj.weight": ParamSpec((k * hd, d)),
                 "v_proj.weight": ParamSpec((k * hd, d)), "o_proj.weight": ParamSpec((d, h * hd))}
 
-    def _pad_rows(self, w, heads):
-        """[heads * hd, d] -> [heads * padded, d]: zero rows after each head's own."""
+    def _pad_rows(self, w, heads, order=None):
+        """[heads * hd, d] -> [heads * padded, d]: the rows of each head in ``order`` (the position part's
+        wish for q and k heads, see ``RotaryPosition.head_row_order``), zero rows after each head's own."""
         hd, pad = self.head_dim, self.padded_head_dim
+        if order is not None:
+            index = torch.as_tensor(order, dtype=torch.long, device=w.device)
+            w = w.view(heads, hd, w.shape[1])[:, index].reshape(heads * hd, w.shape[1])
         if pad == hd:
             return w
         out = torch.zeros((heads, pad, w.shape[1]), dtype=w.dtype, device=w.device)
@@ -56,7 +60,10 @@ class Attention(Part):
 
     def bind(self, tensors):
         H, K, hd, pad = self.n_heads, self.n_kv_heads, self.head_dim, self.padded_head_dim
-        wqkv = torch.cat([self._pad_rows(tensors["q_proj.weight"], H), self._pad_rows(tensors["k_proj.weight"], K),
+        wants = getattr(self.position, "head_row_order", None)
+        order = wants(hd) if wants else None
+        wqkv = torch.cat([self._pad_rows(tensors["q_proj.weight"], H, order),
+                          self._pad_rows(tensors["k_proj.weight"], K, order),
                           self._pad_rows(tensors["v_proj.weight"], K)], 0)
         self.wqkv = ops.prepare_weight(wqkv)
         self.wq = self.wqkv.prefix(H * pad) if ops.is_tiled(self.wqkv) else self.wqkv[:H * pad]

@@ -1,7 +1,7 @@
 """Reader (and a writer for tests and the random-weights mode) for GGUF files with
 unquantized tensors.
 
-Layout (docs/gguf.md of the reference; its reader is src/gguf.cpp:171-330): the magic
+Layout (docs/gguf.md of the reference; its reader is src/gguf.cpp:8-85 and 173-257): the magic
 ``GGUF``, a u32 version (2 or 3), the u64 numbers of tensors and of metadata pairs;
 then the pairs, each a string key (u64 length + bytes), a u32 value type and the
 value; then for each tensor its name, a u32 number of dimensions, the u64 dimensions

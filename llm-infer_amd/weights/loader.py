@@ -207,9 +207,7 @@ def load_into(model, folder: str, config=None, ckpt=None) -> None:
         ckpt = read_checkpoint(folder, needed, config)
     ignorable = list(model.ignorable_names())
     if isinstance(ckpt, GGUFCheckpoint):
-        # exported beside the weights by other tools; the reference binds tensors by name and never
-        # looks at it (frequency factors of a rotation scaling that neither it nor this library applies)
-        ignorable.append("rope_freqs.weight")
+        ignorable += list(getattr(config, "gguf_ignorable", ()))     # the configuration class names them
     check_tensors(needed, ckpt, ignorable)
     model.bind(OnDemand(lambda name: place_tensor(ckpt.tensor(name), needed[name].kind, model.dtype, model.device)))
 

@@ -43,6 +43,9 @@ def sizes(cfg: dict) -> dict:
         # absent: silu, the Llama decoder's activation and what the reference's GGUF constructor fixes
         # (config.cpp:163); its HF constructor would default to gelu (config.cpp:97), a departure on purpose
         act=cfg.get("hidden_act", "silu"),
+        # which two dimensions of a head form a rotated pair: (2j, 2j+1) as the reference rotates them, or
+        # (j, j + rotary/2) for checkpoints whose rows were not permuted for it (docs/gguf.md:487-493)
+        pairing=cfg.get("rope_pairing", "adjacent"),
     )
 
 
@@ -68,21 +71,29 @@ def linear(x: torch.Tensor, w: torch.Tensor) -> torch.Tensor:
     return x @ w.t()
 
 
-def rope(v: torch.Tensor, positions: torch.Tensor, theta: float, rotary_dim: int) -> torch.Tensor:
+def rope(v: torch.Tensor, positions: torch.Tensor, theta: float, rotary_dim: int,
+         pairing: str = "adjacent") -> torch.Tensor:
     """Rotate adjacent pairs (i, i+1), i even < rotary_dim, by pos * theta^(-i/rotary_dim).
 
     v is [n, heads, head_dim]; include/kernels_cpu.hpp:82-100.  Dimensions at or
-    beyond rotary_dim stay as they are.
+    beyond rotary_dim stay as they are.  ``pairing`` "half" pairs dimension j with
+    j + rotary_dim/2 instead, pair j keeping the angle of the adjacent pair j: the order of a
+    checkpoint before the row permutation that the reference's files carry (docs/gguf.md:487-493,
+    which maps row j of the first half to 2j and row j of the second half to 2j+1).
     """
     out = v.clone()
     i = torch.arange(0, rotary_dim, 2, dtype=v.dtype)
     freq = 1.0 / torch.pow(torch.tensor(theta, dtype=v.dtype), i / rotary_dim)   # hpp:87
     ang = positions.to(v.dtype)[:, None] * freq[None, :]                          # hpp:88
     cos, sin = torch.cos(ang)[:, None, :], torch.sin(ang)[:, None, :]
-    v0 = v[..., 0:rotary_dim:2]
-    v1 = v[..., 1:rotary_dim:2]
-    out[..., 0:rotary_dim:2] = v0 * cos - v1 * sin                                # hpp:96
-    out[..., 1:rotary_dim:2] = v0 * sin + v1 * cos                                # hpp:97
+    if pairing == "half":
+        first, second = slice(0, rotary_dim // 2), slice(rotary_dim // 2, rotary_dim)
+    else:
+        first, second = slice(0, rotary_dim, 2), slice(1, rotary_dim, 2)
+    v0 = v[..., first]
+    v1 = v[..., second]
+    out[..., first] = v0 * cos - v1 * sin                                         # hpp:96
+    out[..., second] = v0 * sin + v1 * cos                                        # hpp:97
     return out
 
 
@@ -141,8 +152,9 @@ def attention_part(x, w, prefix, s, positions, window=None, act_dtype=None, kv_d
     q = linear(x, w[prefix + "q_proj.weight"]).view(n, s["n_heads"], s["hd"])
     k = linear(x, w[prefix + "k_proj.weight"]).view(n, s["n_kv"], s["hd"])
     v = linear(x, w[prefix + "v_proj.weight"]).view(n, s["n_kv"], s["hd"])
-    q = _r(rope(q, positions, s["theta"], s["rotary"]), act_dtype)          # block.cpp:141
-    k = _r(rope(k, positions, s["theta"], s["rotary"]), act_dtype)          # block.cpp:142
+    pairing = s.get("pairing", "adjacent")
+    q = _r(rope(q, positions, s["theta"], s["rotary"], pairing), act_dtype)          # block.cpp:141
+    k = _r(rope(k, positions, s["theta"], s["rotary"], pairing), act_dtype)          # block.cpp:142
     k, v = _r(k, kv_dtype), _r(v, kv_dtype)               # the cache holds float16 (block.cpp:145-148)
     a = attention(q, k, _r(v, act_dtype), window, act_dtype).reshape(n, s["n_heads"] * s["hd"])
     return linear(_r(a, act_dtype), w[prefix + "o_proj.weight"])            # block.cpp:167

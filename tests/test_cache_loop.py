@@ -96,6 +96,25 @@ def test_cache_groups_lengths_and_page_accounting():
     assert kv_full.pool.n_free == 10 and not kv_full.pool.held() and c.slots.n_free == 4
 
 
+def test_a_failed_step_gives_its_pages_back():
+    """``truncate`` undoes ``grow``: lengths as before, the pages beyond them free again (and so cleared or
+    wholly filled when they are next handed out), the page a sequence still reaches kept."""
+    c = _cache([KVSpec(2, 16), KVSpec(2, 16, window=100)])
+    full = c.groups[0]
+    s0, s1 = c.alloc_slot(), c.alloc_slot()
+    c.grow([s0, s1], [70, 64])
+    free_before, pages_before = full.pool.n_free, dict(full.pages_of[s0])
+    c.grow([s0, s1], [200, 65], filled=True)
+    c.truncate([s0, s1], [70, 64])
+    assert c.lens[s0] == 70 and c.lens[s1] == 64
+    assert full.pool.n_free == free_before and full.pages_of[s0] == pages_before
+    assert sorted(full.pages_of[s1]) == [0] and full.table_host[s1, 1] == 0 and full.table_host[s0, 2] == 0
+    held = [p for s in (s0, s1) for p in full.pages_of[s].values()]
+    assert set(held) == full.pool.held()
+    c.grow([s0], [200])                                   # and the sequence grows again as if nothing had been
+    assert len(full.pages_of[s0]) == 4
+
+
 def test_random_sequences_never_share_a_page():
     c = _cache([KVSpec(1, 16)], max_tokens=64 * 40, max_pos=64 * 12, slots=6)
     g = c.groups[0]
@@ -177,6 +196,26 @@ def test_the_loop_decisions():
     assert t.live() == [] and t.reason == ["length"]
 
 
+def test_a_budget_for_each_request_and_the_rows_of_a_recorded_step():
+    from llm_infer_amd.engine.decode import batch_bucket
+    from llm_infer_amd.engine.generate import per_request
+    t = BatchTracker([3, 3, 3], max_new_tokens=[1, 3, 0], stop_token_ids=(), max_positions=100)
+    assert t.live() == [0, 1] and t.reason[2] == "length"
+    assert not t.will_go_on([0, 1]) and t.will_go_on([1])
+    assert t.accept([0, 1], [4, 5]) == [1] and t.reason[0] == "length"
+    assert t.accept([1], [6]) == [1] and t.accept([1], [7]) == [] and t.outputs == [[4], [5, 6, 7], []]
+    assert plan_batches([60, 60, 60], [10, 200, 4], 8, 448, 1000) == [[0, 1], [2]]      # 128 + 320, then 64
+    with pytest.raises(RequestError, match="2 values for 3 requests"):
+        per_request([1, 2], 3)
+    # a shrinking batch meets few sizes: every size at least the live sequences, at most the slots, and at
+    # most a third of its rows idle
+    sizes = [batch_bucket(n, 4096) for n in range(1, 300)]
+    assert sizes[:17] == [1, 2, 4, 4, 8, 8, 8, 8, 12, 12, 12, 12, 16, 16, 16, 16, 24]
+    assert len(set(sizes[:64])) == 10 and all(b >= n for n, b in zip(range(1, 300), sizes))
+    assert all(b - n <= b // 3 + 1 for n, b in zip(range(1, 300), sizes))
+    assert batch_bucket(5, 6) == 6 and batch_bucket(7, 7) == 7 and batch_bucket(64, 64) == 64
+
+
 def test_the_loop_knows_beforehand_whether_all_go_on():
     """will_go_on is what lets a step be enqueued before the tokens of the step before are read:
     it must say exactly whether tokens that are no stop tokens keep every live request going."""
@@ -245,7 +284,7 @@ def test_a_build_whose_hand_counted_kernel_spills_is_refused():
         build._check_no_scratch(ok.replace("lane]: 0", "lane]: 16"), "gemm_wreg_kernel", "x.hip")
     with pytest.raises(build.BuildError, match="no resource usage"):
         build._check_no_scratch("", "gemm_wreg_kernel", "x.hip")
-    assert build.NO_SCRATCH == {"gemm_prefill.hip": "gemm_wreg_kernel"}
+    assert build.NO_SCRATCH == {"gemm_prefill.hip": "gemm_wreg_kernel", "attention.hip": "attn_prefill_kernel"}
 
 
 def test_build_folder_is_the_same_for_builds_that_run_side_by_side(tmp_path, monkeypatch):

@@ -15,7 +15,7 @@ from tiny_configs import ALL
 pytestmark = pytest.mark.gpu
 
 LENGTHS = {"A": [40, 7, 100, 1, 64, 65, 33, 127], "B": [200, 1, 4, 9, 16, 31, 130, 255], "C": [300, 70, 5, 640, 129],
-           "D": [150, 2, 64, 33, 190], "E": [90, 1, 65, 300]}
+           "D": [150, 2, 64, 33, 190], "E": [90, 1, 65, 300], "F": [120, 3, 64, 159, 31]}
 
 
 def make_weights(cfg, seed, matrix_dtype=torch.bfloat16):
@@ -139,6 +139,44 @@ def test_step_direct_and_generate(model, dtype):
                     break                                     # a near tie: either token is right
                 assert t == int(ref.argmax()), (model.name, dtype, use_graph)
                 toks.append(t)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_half_paired_model_is_the_adjacent_model_with_dealt_out_rows(dtype, tmp_path):
+    """"rope_pairing": "half" is served by ordering the rows of every q and k head when the weights are bound:
+    the same checkpoint with those rows dealt out by hand (j -> 2j, j + rotary/2 -> 2j+1) and adjacent pairing
+    gives the same logits to the bit, prompt and decoded tokens, and both run the fused kernels."""
+    import llm_infer_amd
+    cfg = dict(ALL["F"], torch_dtype=STORED[dtype])
+    s = P.sizes(cfg)
+    weights = make_weights(cfg, seed=11, matrix_dtype=TORCH[STORED[dtype]])
+    order = list(range(s["hd"]))
+    for j in range(s["rotary"] // 2):
+        order[2 * j], order[2 * j + 1] = j, j + s["rotary"] // 2
+    dealt = dict(weights)
+    for name, w in weights.items():
+        if "q_proj" in name or "k_proj" in name:
+            heads = w.shape[0] // s["hd"]
+            dealt[name] = w.view(heads, s["hd"], -1)[:, order].reshape(w.shape).contiguous()
+    P.write_model(str(tmp_path / "half"), cfg, weights)
+    P.write_model(str(tmp_path / "adjacent"), dict(cfg, rope_pairing="adjacent"), dealt)
+    tokens = [[5, 300, 17, 2, 250, 99, 1], [8] * 70]
+    out = []
+    for folder in ("half", "adjacent"):
+        eng = llm_infer_amd.load(str(tmp_path / folder), dtype=dtype, max_tokens=512)
+        slots = [eng.alloc_slot() for _ in tokens]
+        first = eng.step(slots, tokens, [list(range(len(t))) for t in tokens])
+        second = eng.step(slots, [[3], [4]])
+        out.append(torch.cat([first, second]).cpu())
+    assert torch.equal(out[0], out[1])
+    # and they are the plain implementation's, which pairs (j, j + rotary/2) itself
+    ref = P.forward(weights, cfg, tokens[0], torch.float64)
+    err = (out[0][:len(tokens[0])].double() - ref).abs().max().item()
+    own = (P.forward(weights, cfg, tokens[0], torch.float64, None if dtype == "float32" else TORCH[dtype]) - ref).abs().max().item()
+    own = max(own, (P.forward(weights, cfg, tokens[0], torch.float32).double() - ref).abs().max().item())
+    assert err < 3 * own + 1e-6 * ref.std().item(), (err, own)
+    wrong = P.forward(weights, dict(cfg, rope_pairing="adjacent"), tokens[0], torch.float64)
+    assert (wrong - ref).abs().max().item() > 10 * (3 * own + 1e-6)       # the pairing matters on this model
 
 
 def test_a_model_runs_in_its_own_dtype_unless_told_otherwise(model, capfd):

@@ -311,6 +311,46 @@ def test_recorded_steps_replay_like_eager_steps(lib, folders, dtype):
     assert eng.cache.slots.n_free == eng.cache.n_slots and eng.cache.tokens_free() == (eng.cache.n_pages - 1) * 64
 
 
+@pytest.mark.parametrize("dtype", ["bfloat16", "float32"])
+def test_recorded_steps_at_bucket_edges_other_temperatures_and_after_eviction(lib, folders, dtype, monkeypatch):
+    """What a recorded step is keyed by, each edge crossed: the bucket of context lengths (193 and 449 tokens
+    are where the split count may change), the rows of the step (a batch that shrinks through the sizes 8,
+    4, 2, 1 with idle rows in between), the temperature (read from the device: one recorded step, two
+    temperatures), and a table of recorded steps so small that a step is dropped and recorded again."""
+    from llm_infer_amd.engine import decode
+    eng = lib.load(folder_for(folders, "C", dtype), dtype=dtype, max_tokens=16384)
+    g = torch.Generator().manual_seed(11)
+    prompts = [torch.randint(0, 331, (n,), generator=g).tolist() for n in (185, 440, 60, 189, 7, 445, 100, 3)]
+    budgets = [16, 14, 3, 12, 5, 9, 7, 2]                       # the batch shrinks 8 -> 1, crossing both edges on the way
+    eager = eng.generate(prompts, max_new_tokens=budgets, temperature=0.0, use_graph=False)
+    assert [len(o) for o in eager] == budgets
+    assert eng.decode_counts == {"eager": 0, "recorded": 0, "replayed": 0}
+    first = eng.generate(prompts, max_new_tokens=budgets, temperature=0.0, use_graph=True)
+    counts = dict(eng.decode_counts)
+    again = eng.generate(prompts, max_new_tokens=budgets, temperature=0.0, use_graph=True)
+    assert first == eager and again == eager
+    assert counts["eager"] == 1 and counts["recorded"] >= 4 and counts["replayed"] >= 1
+    assert eng.decode_counts["recorded"] == counts["recorded"]            # the second time every step was there
+    rows = sorted({k[0] for k in eng._graphs})
+    assert rows == [1, 2, 4, 8], rows                                     # 7, 6, 5 and 3 live sequences ran as 8, 8, 8 and 4 rows
+    # two temperatures through the same recorded steps, against the eager runner with the same seeds
+    for temperature in (0.7, 1.6):
+        cold = eng.generate(prompts, max_new_tokens=budgets, temperature=temperature, seed=3, use_graph=False)
+        warm = eng.generate(prompts, max_new_tokens=budgets, temperature=temperature, seed=3, use_graph=True)
+        assert cold == warm, temperature
+    recorded_hot = eng.decode_counts["recorded"]
+    assert eng.generate(prompts, max_new_tokens=budgets, temperature=0.9, seed=3, use_graph=True) == \
+        eng.generate(prompts, max_new_tokens=budgets, temperature=0.9, seed=3, use_graph=False)
+    assert eng.decode_counts["recorded"] == recorded_hot                 # a third temperature recorded nothing
+    # a table of two: steps are dropped while the batch shrinks and recorded again when they come back
+    monkeypatch.setattr(decode, "MAX_RECORDED_STEPS", 2)
+    before = eng.decode_counts["recorded"]
+    for _ in range(2):
+        assert eng.generate(prompts, max_new_tokens=budgets, temperature=0.0, use_graph=True) == eager
+    assert len(eng._graphs) <= 2 and eng.decode_counts["recorded"] >= before + 6
+    assert eng.cache.slots.n_free == eng.cache.n_slots and eng.cache.tokens_free() == (eng.cache.n_pages - 1) * 64
+
+
 # ---------------------------------------------------------------------------
 # slots and pages used again, batch composition
 # ---------------------------------------------------------------------------

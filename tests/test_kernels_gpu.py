@@ -215,6 +215,49 @@ def test_norm_split_over_two_products(ops, M, d, K2, N2, dt):
         assert ops.lazy_rmsnorm(big, wn, eps, dt) is None                   # more than 16 rows: the norm kernel
 
 
+@pytest.mark.parametrize("dt", F16S)
+@pytest.mark.parametrize("rms,wscale", [(1e-2, 0.02), (1e3, 0.02), (1e3, 4.0), (3.0, 1.0)])
+def test_norm_split_over_two_products_at_a_models_own_scale(ops, rms, wscale, dt):
+    """The rows that travel in 16 bits between the two products are x * weight; a checkpoint's residual stream
+    may be of the order of 0.01 or of 1000 and its norm weights of 0.02.  In float16 each row is scaled by a
+    power of two taken from the norm before (left by the norm kernel, then by each product that finishes a
+    norm), so the split norm is as exact as norm kernel + product at every scale, down a chain of layers in
+    which the rows grow; a view of the rows that a kernel writes through voids the preparation too."""
+    M, d, K2, N2 = 7, 1024, 512, 768
+    g = torch.Generator().manual_seed(3)
+    x0 = torch.randn(M, d, generator=g) * rms
+    x0[2, 5] = 40 * rms                                            # a row with one large element
+    wn = (wscale * (1 + 0.3 * torch.randn(d, generator=g))).to(DEV)
+    # (the product's own operands stay of moderate size in 16 bits: what it adds is of the order of rms 3^layer)
+    wo = (torch.randn(d, K2, generator=g) * 0.05 * rms / 34).to(dt)
+    w2 = (torch.randn(N2, d, generator=g) * 0.05).to(dt)
+    wot, w2t = ops.tile_weight(wo.to(DEV)), ops.tile_weight(w2.to(DEV))
+    eps = 1e-6
+    x = x0.to(DEV)
+    ops.rmsnorm(x, wn, eps, dt)                                    # the norm before: in float16 it leaves the rows' scales
+    assert (getattr(x, "_li_row_scale", None) is not None) == (dt == torch.float16)
+    for layer in range(3):                                         # the rows grow by a factor of about 3 a layer
+        a = (torch.randn(M, K2, generator=g) * 30 * 3 ** layer).to(dt)
+        ops.expect_norm(x, wn)
+        ops.linear(a.to(DEV), wot, ops.EPI_ADD, out=x)
+        ln = ops.lazy_rmsnorm(x, wn, eps, dt)
+        assert ln is not None and (ln.row_scales is not None) == (dt == torch.float16)
+        assert torch.isfinite(ln.xw.float()).all()
+        fused = ops.linear(ln, w2t, out_dtype=torch.float32)
+        xd = x.double().cpu()
+        ref = (xd / torch.sqrt((xd ** 2).mean(1, keepdim=True) + eps) * wn.double().cpu()) @ w2.double().t()
+        plain = ops.linear(ops.rmsnorm(x.clone(), wn, eps, dt), w2t, out_dtype=torch.float32)
+        own = (plain.double().cpu() - ref).abs().max().item()
+        err = (fused.double().cpu() - ref).abs().max().item()
+        assert err < 1.5 * own + 1e-6 * ref.abs().max().item(), (layer, err, own)
+    # a kernel that writes through a view of the rows voids what was prepared for the rows themselves
+    ops.expect_norm(x, wn)
+    ops.linear(a.to(DEV), wot, ops.EPI_ADD, out=x)
+    assert ops.lazy_rmsnorm(x, wn, eps, dt) is not None
+    ops.linear(a.to(DEV)[:4].contiguous(), wot, ops.EPI_ADD, out=x[:4])
+    assert ops.lazy_rmsnorm(x, wn, eps, dt) is None
+
+
 def test_gate_activation_alone(ops):
     """act(gate) * up on interleaved columns, for a product that was stored unactivated."""
     g = torch.Generator().manual_seed(3)

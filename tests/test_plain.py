@@ -78,6 +78,34 @@ def test_rope_scores_depend_on_distance_only():
     assert not torch.allclose(score(5, 2), score(5, 3), atol=1e-6)
 
 
+def test_rope_half_pairing_is_a_complex_product_and_a_permutation_of_the_adjacent_one():
+    """Half pairing: dimension j and j + rotary/2 are the real and imaginary part of a number that is
+    multiplied by exp(i pos theta^(-2j/rotary)) (a library routine), and the same rotation as the adjacent
+    one on a head whose dimensions were dealt out (first half to the even places, second half to the odd
+    ones: the permutation of docs/gguf.md:487-493).  A wrong sign, a pair (j, j+1) or frequencies counted
+    over the half fail one of the two."""
+    rot, hd = 24, 32
+    v = torch.randn(5, 2, hd, dtype=F64)
+    pos = torch.tensor([0, 1, 7, 300, 4097])
+    out = P.rope(v, pos, 20000.0, rot, "half")
+    z = torch.complex(v[..., :rot // 2], v[..., rot // 2:rot])
+    ang = pos.to(F64)[:, None] * 20000.0 ** (-torch.arange(0, rot, 2, dtype=F64) / rot)[None, :]
+    w = z * torch.polar(torch.ones_like(ang), ang)[:, None, :]
+    assert torch.allclose(out[..., :rot // 2], w.real, atol=1e-12)
+    assert torch.allclose(out[..., rot // 2:rot], w.imag, atol=1e-12)
+    assert torch.equal(out[..., rot:], v[..., rot:]) and torch.equal(out[0], v[0])
+    # dealt out: new dimension 2j <- j, 2j+1 <- j + rot/2; the adjacent rotation of that is the half one, dealt out
+    order = list(range(hd))
+    for j in range(rot // 2):
+        order[2 * j], order[2 * j + 1] = j, j + rot // 2
+    assert torch.allclose(P.rope(v[..., order], pos, 20000.0, rot), out[..., order], atol=1e-12)
+    assert not torch.allclose(P.rope(v, pos, 20000.0, rot), out, atol=1e-3)
+    # scores depend on the distance alone here too
+    q, k = v[:1], v[1:2]
+    s = lambda m, n: (P.rope(q, torch.tensor([m]), 1e4, rot, "half") * P.rope(k, torch.tensor([n]), 1e4, rot, "half")).sum(-1)
+    assert torch.allclose(s(9, 4), s(209, 204), atol=1e-10)
+
+
 def _library_attention(q, k, v):
     n, H, hd = q.shape
     g = H // k.shape[1]

@@ -41,4 +41,14 @@ TINY_E = {
     "max_position_embeddings": 320, "tie_word_embeddings": False, "hidden_act": "silu",
 }
 
-ALL = {"A": TINY_A, "B": TINY_B, "C": TINY_C, "D": TINY_D, "E": TINY_E}
+# rotated pairs (j, j + 12) of a 32-wide head instead of adjacent ones (a checkpoint in the row order the
+# reference's files are permuted from): GQA 6/3, explicit head size, three quarters of it rotated
+TINY_F = {
+    "architectures": ["LlamaForCausalLM"], "model_type": "llama",
+    "num_hidden_layers": 2, "hidden_size": 88, "num_attention_heads": 6, "num_key_value_heads": 3, "head_dim": 32,
+    "intermediate_size": 120, "vocab_size": 301, "rope_theta": 5000.0, "rms_norm_eps": 3e-6,
+    "partial_rotary_factor": 0.75, "rope_pairing": "half",
+    "max_position_embeddings": 160, "tie_word_embeddings": False, "hidden_act": "silu",
+}
+
+ALL = {"A": TINY_A, "B": TINY_B, "C": TINY_C, "D": TINY_D, "E": TINY_E, "F": TINY_F}
