@@ -64,7 +64,11 @@ def main() -> int:
         print(f"bench.py: this library runs on one GPU; --gpus {args.gpus} is not supported")
         return 2
 
+    if args.shape == "llama-3.1-8b" and not args.no_further_sizes and args.prefill_tokens == 2048:
+        args.also_prefill = [16, 128]                      # short prompts, which run as recorded steps
     line = measure(args)
+    for n, r in line.pop("also_prefill", {}).items():
+        line["points"][f"prefill_{n}_ms"] = r["ms"]
     if args.shape == "llama-3.1-8b" and not args.no_other_shapes and not args.ragged_prefill:
         # the other two benchmark shapes, each in an engine of its own, into the same line
         import copy
@@ -217,7 +221,7 @@ def measure(args) -> dict:
     prefill_s, prefill_flops = prefill_run(T, (4 if T <= 4096 else 3) if args.prefill_tokens > 0 else 2)
     more_prefills = {}
     for n in also_prefill:
-        s_, f_ = prefill_run(n, 3)
+        s_, f_ = prefill_run(n, 5 if n <= 512 else 3)      # (a short prompt is run eagerly, recorded, then replayed)
         more_prefills[str(n)] = {"value": round(n / s_, 1), "tokens": n, "ms": round(s_ * 1e3, 3),
                                  "frac": round(f_ / s_ / PEAK_FLOPS[args.dtype], 4)}
 

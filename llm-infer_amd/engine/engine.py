@@ -56,6 +56,9 @@ class Engine:
         self._graphs = {}
         self._graph_bufs = None
         self.decode_counts = {"eager": 0, "recorded": 0, "replayed": 0}      # what the recorded-step runner did
+        # short prompts are recorded too (engine/prefill.py); False runs every prefill step eagerly
+        self.record_prefill = True
+        self._prefill = None
 
     # -- construction ----------------------------------------------------------
     @classmethod
@@ -120,9 +123,18 @@ class Engine:
         """slots[i]: a held slot; tokens[i]: that sequence's next tokens (at least one);
         want[i]: places among these tokens whose logits are returned (default: the last).
         Returns float32 [sum(len(want[i])), vocab] in the order of the sequences and of want."""
-        ctx = self.prepare(slots, tokens, want)
+        ctx = self.prepare(slots, tokens, want, upload=False)
         try:
-            logits = self.model.forward(ctx, self.cache)
+            logits = None
+            if self.record_prefill:
+                if self._prefill is None:
+                    from .prefill import PrefillRecorder
+                    self._prefill = PrefillRecorder(self)
+                if self._prefill.takes(ctx):
+                    logits = self._prefill.run(ctx)          # None the first time a size is seen
+            if logits is None:
+                ctx.upload()
+                logits = self.model.forward(ctx, self.cache)
         except Exception:
             # a kernel refused its operands: the sequences are as long as before the step, and the pages
             # the step took are given back
@@ -131,7 +143,7 @@ class Engine:
         self.cache.trim_windows(slots)
         return logits
 
-    def prepare(self, slots, tokens, want=None) -> StepContext:
+    def prepare(self, slots, tokens, want=None, upload: bool = True) -> StepContext:
         if len(slots) != len(tokens) or len(set(slots)) != len(slots):
             raise ValueError("step: one token list for each slot, each slot once")
         if want is None:
@@ -146,4 +158,4 @@ class Engine:
         before = [self.cache.lens[s] for s in slots]
         # every mixer writes all of the step's tokens into its cache before anything reads it
         self.cache.grow(slots, [b + len(t) for b, t in zip(before, tokens)], filled=True)
-        return StepContext(self.device, slots, tokens, before, want)
+        return StepContext(self.device, slots, tokens, before, want, upload)

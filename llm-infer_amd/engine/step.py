@@ -28,9 +28,11 @@ class StepContext(StepShared):
                   seq_qlen (tokens in this step), seq_ctx (context length after the step)
     want_rows   : rows of the step whose logits are asked for
     The host keeps ``host_slots``, ``host_qlens`` and ``host_lens_before`` for parts that plan on the host.
+    ``upload=False`` leaves the device arrays out until ``upload()`` is called (a step that is replayed from a
+    recording reads them from the recording's own buffer).
     """
 
-    def __init__(self, device, slots, tokens, lens_before, want):
+    def __init__(self, device, slots, tokens, lens_before, want, upload: bool = True):
         self.n_seqs = len(slots)
         qlens = [len(t) for t in tokens]
         self.n_tokens = sum(qlens)
@@ -44,10 +46,17 @@ class StepContext(StepShared):
         want_rows = [int(qstart[i]) + w for i, ws in enumerate(want) for w in ws]
         self.n_want = len(want_rows)
         self.device = device
-        fields = [("token_ids", flat), ("pos", pos), ("tok_slot", tok_slot), ("seq_slot", slots),
-                  ("seq_qstart", qstart), ("seq_qlen", qlens),
-                  ("seq_ctx", [l + q for l, q in zip(lens_before, qlens)]),
-                  ("want_rows", want_rows)]
+        self.host_tokens, self.host_want_rows = flat, want_rows
+        self._fields = [("token_ids", flat), ("pos", pos), ("tok_slot", tok_slot), ("seq_slot", slots),
+                        ("seq_qstart", qstart), ("seq_qlen", qlens),
+                        ("seq_ctx", [l + q for l, q in zip(lens_before, qlens)]),
+                        ("want_rows", want_rows)]
+        if upload:
+            self.upload()
+
+    def upload(self) -> None:
+        """The index arrays onto the device, with one copy."""
+        fields, device = self._fields, self.device
         sizes = [len(v) for _, v in fields]
         offs = np.concatenate([[0], np.cumsum([(s + 3) // 4 * 4 for s in sizes])])
         packed = np.zeros(int(offs[-1]) + 4, dtype=np.int32)

@@ -535,19 +535,30 @@ def _check_pages(k_pages, v_pages, page_table, n_kv_heads, head_dim, dtype):
 Q_TILE = 128            # tokens of one workgroup of the prefill attention kernel
 
 
+PREFILL_TILES_KEY = ("attention_prefill_tiles", Q_TILE)      # under this key a step shares the list of tiles
+
+
+def prefill_tiles(qlens) -> tuple:
+    """The tiles of attention_prefill for sequences that bring ``qlens`` tokens: one for every Q_TILE tokens
+    of every sequence, as (sequence of the tile, first token of the tile within its sequence's tokens)."""
+    tile_seq, tile_q0 = [], []
+    for i, n in enumerate(qlens):
+        for q0 in range(0, n, Q_TILE):
+            tile_seq.append(i)
+            tile_q0.append(q0)
+    return tile_seq, tile_q0
+
+
 def prefill_meta(ctx) -> dict:
     """The index arrays of attention_prefill for a step: the per-sequence arrays of the step and the
-    kernel's own list of tiles (one for every Q_TILE tokens of every sequence), which is made and
-    uploaded once per step, by the first attention layer that runs."""
+    kernel's own list of tiles, which is made and uploaded once per step, by the first attention layer that
+    runs (a recorded step brings it along under the same key, padded with tiles that begin beyond their
+    sequence's tokens)."""
     def tiles():
-        tile_seq, tile_q0 = [], []
-        for i, n in enumerate(ctx.host_qlens):
-            for q0 in range(0, n, Q_TILE):
-                tile_seq.append(i)
-                tile_q0.append(q0)
+        tile_seq, tile_q0 = prefill_tiles(ctx.host_qlens)
         both = torch.tensor([tile_seq, tile_q0], dtype=torch.int32).to(ctx.device)
         return {"tile_seq": both[0], "tile_q0": both[1], "n_tiles": len(tile_seq)}
-    return dict(ctx.shared(("attention_prefill_tiles", Q_TILE), tiles), seq_slot=ctx.seq_slot,
+    return dict(ctx.shared(PREFILL_TILES_KEY, tiles), seq_slot=ctx.seq_slot,
                 seq_qstart=ctx.seq_qstart, seq_qlen=ctx.seq_qlen, seq_ctx=ctx.seq_ctx)
 
 

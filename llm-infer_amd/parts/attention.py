@@ -27,6 +27,8 @@ class Attention(Part):
     """
 
     takes_lazy_norm = True      # the normed input goes to ops.linear as it comes
+    prefill_recordable = True   # nothing here is planned on the host from a step's lengths but the tile list,
+                                # which a recorded step brings along (ops.PREFILL_TILES_KEY)
 
     def __init__(self, *, hidden_size, n_heads, n_kv_heads, head_dim, scale, window=None, position=None,
                  prefix, dtype, device):
