@@ -461,6 +461,148 @@ __global__ __launch_bounds__(64 * KW) void gemv_tiled_kernel(const T* __restrict
 }
 
 // ===========================================================================
+// gemm_rows: the products of 17 to 128 rows of X against a tiled weight (a decode step of a larger batch, a
+// short prompt).  gemv_tiled's structure, for more rows: a workgroup owns NT tiles of 16 rows of W for the
+// WHOLE of K, its KW waves take shares of K and sum their partial tiles through LDS in wave order, so every
+// epilogue (residual sum, activation, rotation and cache write) is the product's own: no partial sums in
+// memory, no second kernel.  W comes from HBM once, straight into operand A.  The rows of X are fetched by
+// every workgroup (from L2): a wave brings its share, 64 of K at a time, into LDS of its own by
+// global_load_lds in units of 8 rows x 128 bytes (whole lines; lanes that read the operand's own 16 rows x
+// 64 bytes from memory fetch half lines, and that was three times slower) and reads the fragments back in
+// operand order, the units placed with the exclusive-or of gemm_wreg so that the reads are free of bank
+// conflicts.  No barrier in the loop: a wave waits for its own loads only, D stages of 64 of K in flight,
+// by count.  A step past a wave's share takes its W from a KiB of zeros and adds nothing.
+// ===========================================================================
+static __device__ __attribute__((aligned(1024))) unsigned char zero_kib[1024];      // never written
+
+template <class T, int NT, int MT, int KW, int D>
+__global__ __launch_bounds__(64 * KW) void gemm_rows_kernel(const T* __restrict__ X, const T* __restrict__ Wt,
+                                                            int K, int ldx, Epilogue e) {
+    typedef typename Vec<T>::v8 v8;
+    constexpr int UNITS = 2 * MT, STAGE = UNITS * 1024, REGION = D * STAGE;     // bytes of LDS: a stage, a wave's stages
+    static_assert(REGION >= NT * MT * 1024, "a wave's partial tiles lie in its own stages");
+    extern __shared__ __attribute__((aligned(1024))) unsigned char rows_smem[];
+    const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int r = lane & 15, g = lane >> 4;
+    const int tile0 = blockIdx.x * NT;
+    const int n_tiles = (e.N + 15) >> 4;
+    const int steps = K >> 5, doubles = (steps + 1) >> 1;            // 32 and 64 of K
+    const int per = (doubles + KW - 1) / KW;
+    const int d_begin = wave * per, d_end = min(doubles, d_begin + per);
+    const int n = d_end - d_begin;                      // this wave's steps of 64 of K (none for a short K)
+    unsigned char* region = rows_smem + wave * REGION;
+    f32x4 acc[NT][MT];
+#pragma unroll
+    for (int t = 0; t < NT; ++t)
+#pragma unroll
+        for (int j = 0; j < MT; ++j) acc[t][j] = f32x4{0.f, 0.f, 0.f, 0.f};
+    if (n > 0) {
+        // W: tile t, step s (32 of K) is 1 KiB at ((tile0 + t) steps + s) KiB, lane l its 16 bytes at 16 l; the
+        // base is the wave's (scalar registers), the lane's offset never changes.
+        const unsigned char* wbase[NT];
+#pragma unroll
+        for (int t = 0; t < NT; ++t)
+            wbase[t] = (const unsigned char*)Wt + (int64_t)min(tile0 + t, n_tiles - 1) * steps * 1024;
+        const uint32_t woff = lane * 16;
+        // X: lane 8 p + c of unit q brings chunk c ^ p (8 of K) of row 8 q + p (rows beyond M: row M - 1 again;
+        // the epilogue drops them).  If K ends half way through a step of 64, the lanes of the second half
+        // fetch the first half again in that step (the row ends there) and W's second half is the zeros.
+        const int p = lane >> 3, chunk = (lane & 7) ^ p;
+        uint32_t xoff[UNITS];
+#pragma unroll
+        for (int q = 0; q < UNITS; ++q) xoff[q] = ((uint32_t)min(8 * q + p, e.M - 1) * (uint32_t)ldx + 8 * chunk) * 2;
+        const uint32_t odd_back = ((steps & 1) && chunk >= 4) ? 64 : 0;
+        const unsigned char* xbase = (const unsigned char*)X;
+        v8 a[D][2][NT];
+        auto fetch = [&](int u, int i) {
+            const bool in = i < n;
+            const int dd = d_begin + min(i, n - 1);
+            const uint32_t back = dd == doubles - 1 ? odd_back : 0;
+#pragma unroll
+            for (int q = 0; q < UNITS; ++q)
+                __builtin_amdgcn_global_load_lds(
+                    (const __attribute__((address_space(1))) void*)(xbase + (int64_t)dd * 128 + (xoff[q] - back)),
+                    (__attribute__((address_space(3))) void*)(region + u * STAGE + q * 1024), 16, 0, 0);
+#pragma unroll
+            for (int h = 0; h < 2; ++h)
+#pragma unroll
+                for (int t = 0; t < NT; ++t) {
+                    const int step = 2 * dd + h;
+                    const unsigned char* from = (in && step < steps) ? wbase[t] + (int64_t)step * 1024
+                                                                     : (const unsigned char*)zero_kib;
+                    asm volatile("global_load_dwordx4 %0, %1, %2" : "=v"(a[u][h][t]) : "v"(woff), "s"(from) : "memory");
+                }
+        };
+        // where lane (r, g) finds row r, chunk 4 h + g of fragment 0 in a stage: unit r / 8, place
+        // 8 (r % 8) + ((4 h + g) ^ r % 8); fragment j lies 2 KiB on
+        const uint32_t lds_base = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) unsigned char*)region +
+                                  (r >> 3) * 1024 + (r & 7) * 128;
+        const uint32_t lds_h0 = lds_base + (g ^ (r & 7)) * 16, lds_h1 = lds_base + ((4 + g) ^ (r & 7)) * 16;
+        constexpr int PER_STAGE = UNITS + 2 * NT, AHEAD = (D - 1) * PER_STAGE;
+        static_assert(AHEAD <= 63, "the wait's count");
+#pragma unroll
+        for (int u = 0; u < D; ++u) fetch(u, u);
+        for (int i0 = 0; i0 < n; i0 += D) {
+#pragma unroll
+            for (int u = 0; u < D; ++u) {
+                // the oldest stage in flight has landed (its rows of X in LDS, its W in registers)
+                __builtin_amdgcn_s_waitcnt(0x0F70 | (AHEAD & 15) | ((AHEAD >> 4) << 14));     // vmcnt(AHEAD) only
+                __builtin_amdgcn_sched_barrier(0);
+                v8 b[2][MT];
+#pragma unroll
+                for (int j = 0; j < MT; ++j) {
+                    asm volatile("ds_read_b128 %0, %1 offset:%2" : "=v"(b[0][j]) : "v"(lds_h0 + u * STAGE), "n"(j * 2048) : "memory");
+                    asm volatile("ds_read_b128 %0, %1 offset:%2" : "=v"(b[1][j]) : "v"(lds_h1 + u * STAGE), "n"(j * 2048) : "memory");
+                }
+                __builtin_amdgcn_s_waitcnt(0xC07F);                                            // lgkmcnt(0) only
+                __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+                for (int h = 0; h < 2; ++h)
+#pragma unroll
+                    for (int t = 0; t < NT; ++t)
+#pragma unroll
+                        for (int j = 0; j < MT; ++j) acc[t][j] = mfma16(a[u][h][t], b[h][j], acc[t][j]);
+                __builtin_amdgcn_sched_barrier(0);
+                fetch(u, i0 + u + D);                    // the stage is free: its fragments are in registers
+                __builtin_amdgcn_sched_barrier(0);
+            }
+        }
+        // loads past the last step are still in flight (into this wave's LDS and its ring of registers) and the
+        // compiler does not know of them: wait, then name the registers, so that none of them is handed to
+        // another value before the wait
+        __builtin_amdgcn_s_waitcnt(0x0F70);
+#pragma unroll
+        for (int u = 0; u < D; ++u)
+#pragma unroll
+            for (int h = 0; h < 2; ++h)
+#pragma unroll
+                for (int t = 0; t < NT; ++t) asm volatile("" ::"v"(a[u][h][t]));
+        __builtin_amdgcn_sched_barrier(0);
+    }
+    // the partial tiles of a wave go into its own stages (nothing is in flight into them any more)
+    float* mine = (float*)region;
+#pragma unroll
+    for (int t = 0; t < NT; ++t)
+#pragma unroll
+        for (int j = 0; j < MT; ++j) *(f32x4*)(mine + ((t * MT + j) * 64 + lane) * 4) = acc[t][j];
+    __syncthreads();
+    // the tiles are dealt to the waves: each sums its tiles over the waves in wave order and runs the epilogue
+#pragma unroll
+    for (int t = 0; t < NT; ++t)
+#pragma unroll
+        for (int j = 0; j < MT; ++j) {
+            if ((t * MT + j) % KW != wave) continue;
+            f32x4 v = *(const f32x4*)((const float*)rows_smem + ((t * MT + j) * 64 + lane) * 4);
+            for (int w = 1; w < KW; ++w) {
+                const f32x4 pw = *(const f32x4*)((const float*)(rows_smem + w * REGION) + ((t * MT + j) * 64 + lane) * 4);
+                v[0] += pw[0]; v[1] += pw[1]; v[2] += pw[2]; v[3] += pw[3];
+            }
+            const float vv[4] = {v[0], v[1], v[2], v[3]};
+            epilogue4(e, 16 * j + r, (tile0 + t) * 16 + 4 * g, vv);
+        }
+}
+
+// ===========================================================================
 // C interface
 // ===========================================================================
 extern "C" int li_gemm_fma(const void* X, int x_dt, const void* W, int w_dt, void* C, int out_dt, int mode,
@@ -636,3 +778,57 @@ extern "C" int li_gemv_tiled(const void* X, const void* Wt, int dt, void* C, int
     return LI_OK;
 }
 
+
+// 17 to 128 rows of X against a tiled weight, every epilogue its own (gemm_rows).  nt: 1 or 2 tiles of 16 rows
+// of W a workgroup, kw: 4 or 8 waves that share K (8: up to 64 rows of X) (0: chosen here); ldx: elements from
+// one row of X to the next.
+extern "C" int li_gemm_rows(const void* X, const void* Wt, int dt, void* C, int out_dt, int mode,
+                            int M, int N, int K, int ldx, int nt, int kw, const RopeStore* rs, hipStream_t stream) {
+    int rc = check_common(X, Wt, C, M, N, K, mode, out_dt);
+    if (rc) return rc;
+    if (dt != DT_F16 && dt != DT_BF16) return LI_BAD_ARG;
+    if (M > 128 || ldx < K || ldx % 8 != 0) return LI_BAD_ARG;
+    if (K % 32 != 0 || ((uintptr_t)X & 15) || ((uintptr_t)Wt & 15)) return LI_UNSUPPORTED;
+    if (M == 0) return LI_OK;
+    Epilogue e;
+    rc = make_epilogue(e, C, mode, out_dt, M, N, rs);
+    if (rc) return rc;
+    const int mt = M <= 32 ? 2 : (M <= 64 ? 4 : (M <= 96 ? 6 : 8));
+    const int tiles = (N + 15) / 16;
+    if (nt <= 0) nt = tiles >= 1024 ? 2 : 1;          // enough workgroups for 256 CUs either way
+    if (kw <= 0) kw = 4;
+    if ((nt != 1 && nt != 2) || (kw != 4 && kw != 8) || (kw == 8 && mt > 4)) return LI_BAD_ARG;
+    const int blocks = (tiles + nt - 1) / nt;
+    // stages of 64 of K a wave: what 128 KiB of LDS hold for the workgroup's waves
+#define GO(T, NT, MT, KW, D)                                                                              \
+    do {                                                                                                  \
+        auto kfn = gemm_rows_kernel<T, NT, MT, KW, D>;                                                    \
+        const size_t lds = (size_t)KW * D * 2 * MT * 1024;                                                \
+        static bool allowed = false;               /* more than 64 KiB of LDS is asked for once */       \
+        if (!allowed) {                                                                                   \
+            if (hipFuncSetAttribute((const void*)kfn, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds) != hipSuccess) \
+                return LI_HIP_ERROR;                                                                      \
+            allowed = true;                                                                               \
+        }                                                                                                 \
+        kfn<<<blocks, 64 * KW, lds, stream>>>((const T*)X, (const T*)Wt, K, ldx, e);                      \
+    } while (0)
+#define BY_MT(T, NT)                                            \
+    do {                                                        \
+        if (mt == 2 && kw == 4) GO(T, NT, 2, 4, 6);             \
+        else if (mt == 2) GO(T, NT, 2, 8, 4);                   \
+        else if (mt == 4 && kw == 4) GO(T, NT, 4, 4, 4);        \
+        else if (mt == 4) GO(T, NT, 4, 8, 2);                   \
+        else if (mt == 6) GO(T, NT, 6, 4, 2);                   \
+        else GO(T, NT, 8, 4, 2);                                \
+    } while (0)
+#define PICK(T)                                   \
+    do {                                          \
+        if (nt == 1) BY_MT(T, 1); else BY_MT(T, 2); \
+    } while (0)
+    if (dt == DT_F16) PICK(f16); else PICK(bf16);
+#undef PICK
+#undef BY_MT
+#undef GO
+    LI_CHECK_LAUNCH();
+    return LI_OK;
+}

@@ -9,11 +9,32 @@ CUDA graph per token in the same spirit (src/model/model.cu:11-22).
 """
 from __future__ import annotations
 
+import contextlib
+import gc
+
 import torch
 
 from ..kernels import ops
 from ..tensor import Tensor
 from .step import StepShared, decode_splits, split_bucket
+
+
+@contextlib.contextmanager
+def recording(graph):
+    """What runs inside is recorded into ``graph`` (a HIP graph) instead of being run.  The garbage collector
+    is run before and kept off meanwhile: an object that it frees in the middle of a recording (the recorded
+    steps of an engine that is no longer used, say) calls into the runtime, which refuses such calls while a
+    stream is being recorded, and the process ends."""
+    torch.cuda.synchronize()
+    gc.collect()
+    was_enabled = gc.isenabled()
+    gc.disable()
+    try:
+        with torch.cuda.graph(graph):
+            yield
+    finally:
+        if was_enabled:
+            gc.enable()
 
 
 class PlainDecodeRunner:
@@ -138,8 +159,7 @@ class GraphDecodeRunner:
         else:
             if entry is None or entry == "seen":
                 g = torch.cuda.CUDAGraph()
-                torch.cuda.synchronize()
-                with torch.cuda.graph(g):
+                with recording(g):
                     self._body(rows, bucket)
                 entry = g
                 counts["recorded"] += 1

@@ -129,9 +129,9 @@ class Engine:
             if self.record_prefill:
                 if self._prefill is None:
                     from .prefill import PrefillRecorder
-                    self._prefill = PrefillRecorder(self)
-                if self._prefill.takes(ctx):
-                    logits = self._prefill.run(ctx)          # None the first time a size is seen
+                    self._prefill = PrefillRecorder()
+                if self._prefill.takes(self, ctx):
+                    logits = self._prefill.run(self, ctx)    # None the first time a size is seen
             if logits is None:
                 ctx.upload()
                 logits = self.model.forward(ctx, self.cache)

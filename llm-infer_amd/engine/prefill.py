@@ -21,7 +21,7 @@ import numpy as np
 import torch
 
 from ..kernels import ops
-from .decode import batch_bucket
+from .decode import batch_bucket, recording
 from .step import StepShared
 
 MAX_TOKENS = 512          # a longer step keeps the device busy longer than the host needs to enqueue it
@@ -40,20 +40,22 @@ class _RecordedContext(StepShared):
 
 
 class PrefillRecorder:
-    def __init__(self, engine):
-        self.engine = engine
+    """The recorded prefill steps of one engine (which is handed in with every call: the engine holds this
+    object, and a reference back would keep both alive until the garbage collector finds the cycle)."""
+
+    def __init__(self):
         self.graphs = {}                   # key -> "seen" | (graph, logits)
         self.counts = {"eager": 0, "recorded": 0, "replayed": 0}
         self._buffers = {}                 # key -> (device buffer, layout)
 
     # -- which steps ---------------------------------------------------------------
-    def takes(self, ctx) -> bool:
+    def takes(self, eng, ctx) -> bool:
         """A step of whole prompts (or chunks of them) that is small enough, on a model whose parts can all
         be recorded."""
         if ctx.is_decode or ctx.n_want == 0 or ctx.n_tokens > MAX_TOKENS or ctx.n_seqs > MAX_SEQS:
             return False
         if getattr(self, "_model_ok", None) is None:
-            model = self.engine.model
+            model = eng.model
             mixers = [m for ms in model.layer_mixers for m in ms]
             self._model_ok = model.recordable() and all(getattr(m, "prefill_recordable", False) for m in mixers)
         return self._model_ok
@@ -70,9 +72,9 @@ class PrefillRecorder:
             at += (n + 3) // 4 * 4
         return layout, at
 
-    def _fill(self, ctx, layout, total):
+    @staticmethod
+    def _fill(ctx, layout, total, scratch):
         """The step's index arrays with their padding, as one int32 array."""
-        scratch = self.engine.cache.scratch_slot
         packed = np.zeros(total, dtype=np.int32)
 
         def put(name, values, pad):
@@ -95,10 +97,9 @@ class PrefillRecorder:
         return packed
 
     # -- the step --------------------------------------------------------------------
-    def run(self, ctx):
+    def run(self, eng, ctx):
         """The logits of the step [n_want, vocab], or None if this step is to be run eagerly (the first time
         its key is seen)."""
-        eng = self.engine
         rows = batch_bucket(ctx.n_tokens, MAX_TOKENS)
         seqs = batch_bucket(ctx.n_seqs, MAX_SEQS)
         wants = batch_bucket(ctx.n_want, rows)
@@ -113,13 +114,12 @@ class PrefillRecorder:
         if key not in self._buffers:
             self._buffers[key] = torch.zeros((total,), dtype=torch.int32, device=eng.device)
         buf = self._buffers[key]
-        buf.copy_(torch.from_numpy(self._fill(ctx, layout, total)))
+        buf.copy_(torch.from_numpy(self._fill(ctx, layout, total, eng.cache.scratch_slot)))
         if entry == "seen":
             fields = {name: buf[at:at + n] for name, (at, n) in layout.items()}
             tiles = {"tile_seq": fields.pop("tile_seq"), "tile_q0": fields.pop("tile_q0"), "n_tiles": layout["tile_seq"][1]}
             graph = torch.cuda.CUDAGraph()
-            torch.cuda.synchronize()
-            with torch.cuda.graph(graph):
+            with recording(graph):
                 rec = _RecordedContext(fields, rows, seqs, wants, eng.device)
                 rec.shared(ops.PREFILL_TILES_KEY, lambda: tiles)
                 logits = eng.model.forward(rec, eng.cache)

@@ -314,8 +314,22 @@ def linear(x: torch.Tensor, w, mode: int = EPI_STORE, out: torch.Tensor | None =
                 out._li_rows = (xw, ss, scale, nxt, out._version, row_scales)
             return out
         _need(lazy is None, "a norm is finished by gemv_tiled alone")
-        if force is None and m * k * 2 < (1 << 32):
+        if force is None and m <= 128:
+            # 17 to 128 rows: all of K in one workgroup and every epilogue the product's own (gemm_rows), where
+            # that is estimated faster than the tiled GEMM with K split and its second kernel
+            norm_rides = mode == EPI_ADD and getattr(out, "_li_next_norm", None) is not None
+            nt = _rows_plan(m, n, k, norm_rides)
+            if nt:
+                kind = f"rows:{nt}"
+        if force is None and kind != "fma" and not kind.startswith("rows") and m * k * 2 < (1 << 32):
             kind = "wreg"
+    if kind.startswith("rows"):                                # "rows[:<tiles of W a workgroup>]" (a test's choice)
+        _need(tiled and fast_ok and m <= 128, "gemm_rows: a tiled weight, at most 128 rows of X")
+        parts = kind.split(":")
+        _check(lib.li_gemm_rows(_ptr(x), _ptr(wd), DT[x.dtype], _ptr(out), out_dt, mode, m, n, k, x.stride(0),
+                                int(parts[1]) if len(parts) > 1 else 0, int(parts[2]) if len(parts) > 2 else 0,
+                                rs, _stream()), "gemm_rows")
+        return out
     if kind.startswith("wreg"):                                # "wreg[:<tile>[:<splits>]]" (a test's choice)
         _need(tiled and fast_ok and m * k * 2 < (1 << 32), "gemm_wreg: a tiled weight, X below 4 GiB")
         parts = kind.split(":")
@@ -403,6 +417,32 @@ def _wreg_plan(m: int, n: int, k: int) -> tuple[int, int]:
     read; the narrower tiles are for products whose tiles would leave much of the last round empty."""
     options = [(t, s) for t in (0, 1, 2) for s in (1, 2, 3, 4, 6, 8, 12, 16) if s == 1 or k // s >= 1024]
     return min(options, key=lambda o: (_wreg_cost(o[0], o[1], m, n, k), o[1], o[0]))
+
+
+def _rows_cost(nt: int, m: int, n: int, k: int) -> float:
+    """Estimated microseconds of one gemm_rows launch, fitted to measurements on MI355X (24 to 128 rows against
+    the matrices of the 8B shape): W streamed once (at the rate of 256 workgroups, slower with fewer), plus the
+    rows of X, which every workgroup fetches from L2 in blocks of 16, plus a launch."""
+    blocks16 = 2 if m <= 32 else (4 if m <= 64 else (6 if m <= 96 else 8))
+    groups = -(-(-(-n // 16)) // nt)
+    w_mb, x_mb = n * k * 2 / 1e6, groups * blocks16 * 16 * k * 2 / 1e6
+    # one workgroup a CU at a time (its stages fill the LDS): a last round that is not full runs as long as a full one
+    uneven = -(-groups // 256) * 256 / groups
+    return 2.5 + (w_mb / 6.2 + x_mb / 22.0) * uneven
+
+
+@functools.lru_cache(maxsize=4096)
+def _rows_plan(m: int, n: int, k: int, norm_rides: bool = False) -> int:
+    """Tiles of 16 rows of W a workgroup (1 or 2) if gemm_rows is the faster kernel for this product of 17 to
+    128 rows, else 0 (the tiled GEMM).  ``norm_rides``: the product adds into the residual stream and the
+    norm that follows is known; with K split, the tiled GEMM's second kernel takes that norm along, gemm_rows
+    leaves it to the norm kernel."""
+    rows, nt = min((_rows_cost(t, m, n, k), t) for t in (1, 2))
+    tile, splits = _wreg_plan(m, n, k)
+    other = _wreg_cost(tile, splits, m, n, k)
+    if norm_rides:
+        rows += 4.5 if splits > 1 else 0.0
+    return nt if rows < other else 0
 
 
 def _big_tile(m: int, n: int) -> int:

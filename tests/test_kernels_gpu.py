@@ -108,7 +108,7 @@ def test_linear_all_kernels_and_epilogues(ops, M, N, K, dt):
 
 
 TILED_CASES = [(1, 64, 64), (3, 172, 96), (16, 40, 4096), (9, 16400, 256), (17, 100, 64), (64, 256, 512),
-               (33, 4100, 2048), (48, 72, 8192), (50, 6144, 4096),
+               (33, 4100, 2048), (48, 72, 8192), (50, 6144, 4096), (65, 48, 32), (97, 200, 14336), (30, 520, 96), (128, 16, 160),
                (70, 200, 1024), (96, 1000, 416), (128, 136, 2048), (129, 384, 320), (256, 520, 2048), (384, 512, 192), (300, 1000, 96)]
 
 
@@ -126,6 +126,8 @@ def test_linear_tiled_weights(ops, M, N, K, dt):
     kinds = [None, "mfma:0:1", "mfma:1:2", "mfma:2:1", "big:0", "big:1", "big:0:2", "big:1:5"] + (["gemv_mfma"] if M <= 16 else [])
     # W into registers (tiles of 256, 192, 128 rows of W): the planner's choice and every tile, K whole and split
     kinds += ["wreg", "wreg:0", "wreg:1", "wreg:2", "wreg:0:2", "wreg:1:5", "wreg:2:3"]
+    # all of K in one workgroup, the rows of X through LDS of each wave's own (up to 128 rows): one and two tiles of W
+    kinds += ["rows", "rows:1", "rows:2"] if M <= 128 else []
     for kind in kinds:
         for mode in (0, 1, 2, 4):
             if mode in (2, 4) and N % 2:
@@ -306,7 +308,8 @@ def test_norm_taken_by_the_sum_of_split_products(ops, M, d, K2, dt):
     ops.linear(a, wot, ops.EPI_ADD, out=z)
     ready = ops.prepared_rmsnorm(z, wn, eps, dt)
     assert ready is None or torch.equal(ready, ops.rmsnorm(z, wn, eps, dt))
-    assert M < 64 or ops._wreg_plan(M, d, K2)[1] == 1 or ready is not None
+    # (where the product runs as gemm_rows, all of K in a workgroup, there is no second kernel to take the norm)
+    assert M < 64 or ops._wreg_plan(M, d, K2)[1] == 1 or ops._rows_plan(M, d, K2, True) or ready is not None
 
 
 @pytest.mark.parametrize("M,N,K", [(2048, 8560, 736), (5000, 4048, 736), (1300, 12288, 4096)])
