@@ -36,7 +36,10 @@ Options:
   --random-weights      Ignore the model's tensors: random weights from --seed-weights
   --seed-weights <int>  Seed of the random weights (default: 0)
   --config <json>       With --random-weights: the configuration file (the model argument is not opened)
-  --no-graph            Launch every decode step kernel by kernel"""
+  --no-graph            Launch every decode step kernel by kernel
+
+A folder whose q and k rows are in the original Hugging Face order (rotated pairs j and j + rotary_dim/2,
+never permuted for adjacent pairs as GGUF files are) needs "rope_pairing": "half" in its config.json."""
 
 
 def parse_ids(text: str) -> list:

@@ -496,6 +496,39 @@ __global__ __launch_bounds__(64 * KW) void gemm_rows_kernel(const T* __restrict_
     for (int t = 0; t < NT; ++t)
 #pragma unroll
         for (int j = 0; j < MT; ++j) acc[t][j] = f32x4{0.f, 0.f, 0.f, 0.f};
+    // What the epilogue reads from memory is fetched now, so that it has arrived when the sums are ready: the
+    // tiles are dealt to the waves (tile i to wave i % KW), a lane finishes row 16 j + r, columns n .. n + 3 of
+    // its tiles.  Residual sum: the four values it adds to.  Rotation: the row's position, its cache page, and
+    // the angles of the quad's two pairs (from the table if there is one).
+    constexpr int MINE = (NT * MT + KW - 1) / KW;
+    const bool quads = (e.N & 3) == 0;
+    f32x4 res[MINE];
+    int row_p[MINE];
+    int64_t row_page[MINE];
+    f32x2 ang[MINE][2];
+    if (e.mode == EPI_ADD || e.mode == EPI_ROPE) {
+#pragma unroll
+        for (int i = 0; i < MINE; ++i) {
+            const int id = wave + i * KW, t = id / MT, j = id % MT;
+            const int m = 16 * j + r, col = (tile0 + t) * 16 + 4 * g;
+            res[i] = f32x4{0.f, 0.f, 0.f, 0.f};
+            row_p[i] = 0;
+            row_page[i] = 0;
+            ang[i][0] = ang[i][1] = f32x2{1.f, 0.f};
+            if (id < NT * MT && m < e.M && col < e.N) {
+                if (e.mode == EPI_ADD) {
+                    if (quads) res[i] = *(const f32x4*)((const float*)e.C + (int64_t)m * e.N + col);
+                } else {
+                    const RopeStore& rs = e.rs;
+                    const int head = col / rs.hd, d = col - head * rs.hd;
+                    const int pp = rs.pos[m];
+                    row_p[i] = pp;
+                    if (head >= rs.H) row_page[i] = rs.page_table[(int64_t)rs.tok_slot[m] * rs.max_pages + pp / PAGE];
+                    if (rs.cos_sin) rope_angles(rs, m, pp, head, d, ang[i], true);
+                }
+            }
+        }
+    }
     if (n > 0) {
         // W: tile t, step s (32 of K) is 1 KiB at ((tile0 + t) steps + s) KiB, lane l its 16 bytes at 16 l; the
         // base is the wave's (scalar registers), the lane's offset never changes.
@@ -586,20 +619,34 @@ __global__ __launch_bounds__(64 * KW) void gemm_rows_kernel(const T* __restrict_
 #pragma unroll
         for (int j = 0; j < MT; ++j) *(f32x4*)(mine + ((t * MT + j) * 64 + lane) * 4) = acc[t][j];
     __syncthreads();
-    // the tiles are dealt to the waves: each sums its tiles over the waves in wave order and runs the epilogue
+    // each wave sums its tiles over the waves in wave order and runs the epilogue
 #pragma unroll
-    for (int t = 0; t < NT; ++t)
-#pragma unroll
-        for (int j = 0; j < MT; ++j) {
-            if ((t * MT + j) % KW != wave) continue;
-            f32x4 v = *(const f32x4*)((const float*)rows_smem + ((t * MT + j) * 64 + lane) * 4);
-            for (int w = 1; w < KW; ++w) {
-                const f32x4 pw = *(const f32x4*)((const float*)(rows_smem + w * REGION) + ((t * MT + j) * 64 + lane) * 4);
-                v[0] += pw[0]; v[1] += pw[1]; v[2] += pw[2]; v[3] += pw[3];
-            }
-            const float vv[4] = {v[0], v[1], v[2], v[3]};
-            epilogue4(e, 16 * j + r, (tile0 + t) * 16 + 4 * g, vv);
+    for (int i = 0; i < MINE; ++i) {
+        const int id = wave + i * KW;
+        if (id >= NT * MT) break;
+        const int t = id / MT, j = id % MT;
+        f32x4 v = *(const f32x4*)((const float*)rows_smem + (id * 64 + lane) * 4);
+        for (int w = 1; w < KW; ++w) {
+            const f32x4 pw = *(const f32x4*)((const float*)(rows_smem + w * REGION) + (id * 64 + lane) * 4);
+            v[0] += pw[0]; v[1] += pw[1]; v[2] += pw[2]; v[3] += pw[3];
         }
+        const int m = 16 * j + r, col = (tile0 + t) * 16 + 4 * g;
+        const float vv[4] = {v[0], v[1], v[2], v[3]};
+        if (e.mode == EPI_ADD && quads) {
+            if (m < e.M && col < e.N) {
+                f32x4 o = res[i];
+                o[0] += v[0]; o[1] += v[1]; o[2] += v[2]; o[3] += v[3];
+                *(f32x4*)((float*)e.C + (int64_t)m * e.N + col) = o;
+            }
+        } else if (e.mode == EPI_ROPE && e.rs.cos_sin) {
+            if (m < e.M && col < e.N) {
+                const int head = col / e.rs.hd;
+                rope_store4(e.rs, m, head, col - head * e.rs.hd, vv, row_p[i], row_page[i], ang[i]);
+            }
+        } else {
+            epilogue4(e, m, col, vv);
+        }
+    }
 }
 
 // ===========================================================================

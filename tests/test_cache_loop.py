@@ -263,6 +263,46 @@ def test_the_prefill_product_plan():
     assert _wreg_plan(2048, 6144, 4096)[0] == 1           # 512 tiles of 192 x 128: two on every CU
 
 
+def test_the_plan_for_products_of_a_few_dozen_rows():
+    """17 to 128 rows: all of K in one workgroup (gemm_rows, no second kernel) where its estimate beats the tiled
+    GEMM's; it fetches the rows of X once per workgroup, so it wins against the small matrices and loses against
+    the wide ones, and two tiles of W a workgroup are for matrices with tiles enough for 256 CUs."""
+    from llm_infer_amd.kernels import ops
+    for m in (17, 32, 64, 128):
+        assert ops._rows_plan(m, 4096, 4096, True) in (1, 2)            # attention output, 34 MB
+        assert ops._rows_plan(m, 6144, 4096) in (1, 2)                  # q/k/v, 50 MB
+        assert ops._rows_plan(m, 28672, 4096) == 0                      # gate and up, 235 MB: the tiled GEMM
+    assert ops._rows_plan(64, 6144, 4096) == 2 and ops._rows_plan(64, 4096, 4096, True) == 1
+    assert ops._rows_plan(96, 4096, 14336, True) == 0                   # down: K split and the norm taken along
+    # more rows of X cost more, more tiles a workgroup cost fewer fetches of X
+    assert ops._rows_cost(1, 128, 4096, 4096) > ops._rows_cost(1, 64, 4096, 4096) > ops._rows_cost(1, 32, 4096, 4096)
+    assert ops._rows_cost(2, 64, 28672, 4096) < ops._rows_cost(1, 64, 28672, 4096)
+    # the norm that would have ridden on the tiled GEMM's second kernel counts against gemm_rows
+    assert any(ops._rows_plan(m, n, k, False) and not ops._rows_plan(m, n, k, True)
+               for m in (24, 48, 96) for n, k in ((2048, 8192), (4096, 11008), (4096, 14336)))
+
+
+def test_the_index_arrays_of_a_recorded_prefill_step():
+    """A recorded prefill step reads its step from one buffer of fixed layout; what the step does not fill is
+    padding that belongs to no sequence: tokens on the scratch slot, sequences without tokens, tiles that begin
+    beyond their sequence, wanted places that repeat row 0."""
+    from llm_infer_amd.engine.prefill import PrefillRecorder
+    from llm_infer_amd.engine.step import StepContext
+    ctx = StepContext(None, [3, 1], [[5, 6, 7], [8] * 130], [10, 0], [[2], [0, 129]], upload=False)
+    layout, total = PrefillRecorder._layout(192, 2, 4)
+    assert [layout[k][1] for k in ("token_ids", "seq_slot", "want_rows", "tile_seq")] == [192, 2, 4, 4]
+    packed = PrefillRecorder._fill(ctx, layout, total, scratch=9)
+    get = lambda name: packed[layout[name][0]:layout[name][0] + layout[name][1]].tolist()
+    assert get("token_ids")[:4] == [5, 6, 7, 8] and get("token_ids")[133:] == [0] * 59
+    assert get("pos")[:5] == [10, 11, 12, 0, 1] and get("pos")[132] == 129
+    assert get("tok_slot")[:4] == [3, 3, 3, 1] and set(get("tok_slot")[133:]) == {9}
+    assert get("seq_slot") == [3, 1] and get("seq_qstart") == [0, 3] and get("seq_qlen") == [3, 130] and get("seq_ctx") == [13, 130]
+    assert get("want_rows") == [2, 3, 132, 0]
+    assert get("tile_seq") == [0, 1, 1, 0] and get("tile_q0") == [0, 0, 128, 1 << 30]
+    # every array starts at a multiple of four elements (16 bytes)
+    assert all(at % 4 == 0 for at, _ in layout.values()) and total % 4 == 0
+
+
 def test_cache_rounding_option_is_for_a_float32_cache():
     with pytest.raises(CacheError, match="kv_round"):
         Cache([KVSpec(1, 16)], 256, 128, torch.bfloat16, None, 2, kv_round=torch.float16)
