@@ -223,13 +223,18 @@ __global__ __launch_bounds__(256) void gemm_big_kernel(const T* __restrict__ X, 
 // epilogue, chosen at run time.
 // The loop counts its own loads and LDS reads in flight (s_waitcnt by hand), so the compiler must add none:
 // no spills (the build checks that the kernel uses no scratch memory).
-template <class T, int NI, int MODE>
+// MJ: the tile's rows of X in blocks of 16 (8: 128 rows; 4: 64 rows, for products of up to 64 rows, which then
+// fetch and multiply no rows that are not there).  A: how many steps ahead of their use the loads of W are
+// issued (2, or 4 for products of few rows, where one workgroup a CU has to keep enough of W in flight by itself:
+// 8 NI KiB a wave instead of 4 NI).
+template <class T, int NI, int MODE, int MJ = 8, int A = 2>
 __global__ __launch_bounds__(256) void gemm_wreg_kernel(const T* __restrict__ X, const T* __restrict__ Wt,
                                                         int K, int k_per_split, float* __restrict__ ws, Epilogue e) {
     typedef typename Vec<T>::v8 v8;
     // A step is 64 of K: two halves of 32, each one matrix instruction deep.
     // MJ: fragments of X (16 rows each) per wave and half step; every wave takes all the tile's rows of X
-    constexpr int MJ = 8, BN = 64 * NI, BM = 16 * MJ, XBUFS = 3, SLOTS = 4;
+    constexpr int BN = 64 * NI, BM = 16 * MJ, XBUFS = A + 1, SLOTS = 2 * A;
+    static_assert(MJ == 4 || MJ == 8, "the groups of a half are written out for 4 and 8 fragments");
     constexpr int XU = BM / 8, PER_WAVE = XU / 4;       // 1 KiB units of X per stage (8 rows x 64 of K each), and per wave
     constexpr int STAGE = XU * 1024;
     extern __shared__ __attribute__((aligned(16))) unsigned char smem_raw[];
@@ -325,51 +330,52 @@ __global__ __launch_bounds__(256) void gemm_wreg_kernel(const T* __restrict__ X,
         __builtin_amdgcn_sched_barrier(0);                                                 \
     }
 #define WREG_EIGHT(F, ...) F(0, __VA_ARGS__) F(1, __VA_ARGS__) F(2, __VA_ARGS__) F(3, __VA_ARGS__) \
-                           F(4, __VA_ARGS__) F(5, __VA_ARGS__) F(6, __VA_ARGS__) F(7, __VA_ARGS__)
+    if constexpr (MJ == 8) { F(4, __VA_ARGS__) F(5, __VA_ARGS__) F(6, __VA_ARGS__) F(7, __VA_ARGS__) }
 #define WREG_HALF(A, NEXT)                                                                 \
     {                                                                                      \
         const uint32_t next_ = (NEXT);                                                     \
         WREG_EIGHT(WREG_GROUP, A, next_)                                                   \
     }
-    static_assert(MJ == 8, "the groups of a half are written out");
 
     // (The host gives every split of K at least one step.  Without this line the compiler builds a path
     // for no steps on which the ring's registers are written while the first loads are in flight.)
     if (n_steps <= 0) return;
-    // In flight, in order: at the head of step s the loads of X of step s + 2 are issued, in its middle
-    // those of W's first half of step s + 2, at its end those of the second half.  Step s needs X of step
-    // s + 1 (its second half reads ahead into it) and its own W: all but the 2 NI loads issued last.
+    // In flight, in order: at the head of step s the loads of X of step s + A are issued, in its middle
+    // those of W's first half of step s + A, at its end those of the second half.  Step s needs X of step
+    // s + 1 (its second half reads ahead into it) and its own W: everything up to the loads of X of step s + 1,
+    // i.e. all but the 2 NI loads that followed them in their step and the A - 2 whole steps issued since.
     v8 ring[SLOTS][NI];
-    static_assert(PER_WAVE + 2 * NI <= 15, "the waits' counts");
-    fill(0, 0);
-    fetch_w(0, ring[0]);
-    fetch_w(1, ring[1]);
-    fill(1, STAGE);
-    fetch_w(2, ring[2]);
-    fetch_w(3, ring[3]);
-    // X of step 0 has landed
-    __builtin_amdgcn_s_waitcnt(0x0F70 | (PER_WAVE + 2 * NI));
+    constexpr int PER_STEP = PER_WAVE + 2 * NI, AHEAD = 2 * NI + (A - 2) * PER_STEP;
+    static_assert((A - 1) * PER_STEP <= 63 && AHEAD <= 63, "the waits' counts");
+#pragma unroll
+    for (int a = 0; a < A; ++a) {
+        fill(a, a * STAGE);
+        fetch_w(2 * a, ring[2 * a]);
+        fetch_w(2 * a + 1, ring[2 * a + 1]);
+    }
+    // X of step 0 has landed (and W of step 0 with it)
+    __builtin_amdgcn_s_waitcnt(0x0F70 | (((A - 1) * PER_STEP) & 15) | ((((A - 1) * PER_STEP) >> 4) << 14));
     __builtin_amdgcn_s_barrier();
     WREG_EIGHT(WREG_READ, lds_lane)
     int cur = 0;                                                   // byte offset of the buffer of step s
-    for (int s = 0; s < n_steps; s += 2) {
+    for (int s = 0; s < n_steps; s += A) {
 #pragma unroll
-        for (int u = 0; u < 2; ++u) {                              // two steps a turn of the ring
+        for (int u = 0; u < A; ++u) {                              // A steps a turn of the ring
             if (s + u < n_steps) {
                 const int nxt = cur == (XBUFS - 1) * STAGE ? 0 : cur + STAGE;
-                const int free_buf = nxt == (XBUFS - 1) * STAGE ? 0 : nxt + STAGE;
-                // X of step s + 1 and W of step s have landed (all but the 2 NI loads issued last), and this
-                // wave's reads of the buffer that is filled next are done (all but the MJ issued last, which
-                // read the buffer of this step); the barrier publishes the one and frees the other
-                __builtin_amdgcn_s_waitcnt(0x0070 | (MJ << 8) | (2 * NI));
+                const int free_buf = cur == 0 ? (XBUFS - 1) * STAGE : cur - STAGE;      // of the step before this one
+                // X of step s + 1 and W of step s have landed, and this wave's reads of the buffer that is filled
+                // next are done (all but the MJ issued last, which read the buffer of this step); the barrier
+                // publishes the one and frees the other
+                __builtin_amdgcn_s_waitcnt(0x0070 | (MJ << 8) | (AHEAD & 15) | ((AHEAD >> 4) << 14));
                 __builtin_amdgcn_s_barrier();
-                fill(s + u + 2, free_buf);
+                fill(s + u + A, free_buf);
                 __builtin_amdgcn_sched_barrier(0);
                 WREG_HALF(ring[2 * u], lds_lane2 + cur)
-                fetch_w(2 * (s + u + 2), ring[2 * u]);
+                fetch_w(2 * (s + u + A), ring[2 * u]);
                 __builtin_amdgcn_sched_barrier(0);
                 if (2 * (s + u) + 1 < n_halves) WREG_HALF(ring[2 * u + 1], lds_lane + nxt)
-                fetch_w(2 * (s + u + 2) + 1, ring[2 * u + 1]);
+                fetch_w(2 * (s + u + A) + 1, ring[2 * u + 1]);
                 __builtin_amdgcn_sched_barrier(0);
                 cur = nxt;
             }
@@ -559,44 +565,58 @@ extern "C" int li_gemm_big(const void* X, const void* W, int tiled, int dt, void
 // X below 4 GiB (the kernel addresses it with 32-bit offsets); ws: splits * M * N floats when K is split.
 // `na` (or null): with K split and the residual sum as epilogue, the kernel that adds the partial sums also
 // takes the norm of the finished rows; it must fit (norm_after_fits), the caller has checked the same.
+// few_rows (tile 2 only): 1 = the tile has 64 rows of X, 2 = 128 rows; either way W is fetched four steps ahead
+// instead of two (for products of up to 128 rows, where a workgroup has a CU to itself); 0 = neither.
 extern "C" int li_gemm_wreg(const void* X, const void* Wt, int dt, void* C, int out_dt, int mode,
                             int M, int N, int K, int tile, int splits, float* ws, const RopeStore* rs,
-                            const NormAfter* na, hipStream_t stream) {
+                            const NormAfter* na, int few_rows, hipStream_t stream) {
     int rc = check_common(X, Wt, C, M, N, K, mode, out_dt);
     if (rc) return rc;
     if (dt != DT_F16 && dt != DT_BF16) return LI_BAD_ARG;
     if (K % 32 != 0 || ((uintptr_t)X & 15) || ((uintptr_t)Wt & 15)) return LI_UNSUPPORTED;
-    if (tile < 0 || tile > 2) return LI_BAD_ARG;
+    if (tile < 0 || tile > 2 || few_rows < 0 || few_rows > 2 || (few_rows && tile != 2)) return LI_BAD_ARG;
     if ((int64_t)M * K * 2 >= ((int64_t)1 << 32)) return LI_UNSUPPORTED;
     if (splits < 1 || (splits > 1 && !ws)) return LI_BAD_ARG;
     if (M == 0) return LI_OK;
     Epilogue e;
     rc = make_epilogue(e, C, mode, out_dt, M, N, rs);
     if (rc) return rc;
-    const int bn = 256 - 64 * tile, bm = 128, bk = 32;
+    const int bn = 256 - 64 * tile, bm = few_rows == 1 ? 64 : 128, bk = 32, ahead = few_rows ? 4 : 2;
     int k_per_split = ((K + splits - 1) / splits + bk - 1) / bk * bk;
     splits = (K + k_per_split - 1) / k_per_split;
     if (na && !(splits > 1 && norm_after_fits(na, e, ws))) return LI_BAD_ARG;
     dim3 grid((M + bm - 1) / bm, (N + bn - 1) / bn, splits), block(256);
-    // three stages of X (a step is 64 of K); the epilogue stages two strips of 16 x (bn / 4 + 4) floats a wave
+    // ahead + 1 stages of X (a step is 64 of K); the epilogue stages two strips of 16 x (bn / 4 + 4) floats a wave
     // in the same LDS, and behind both lie a position and a page for each of the tile's rows
-    const size_t stages = (size_t)3 * 2 * (bm / 16) * 1024, strips = (size_t)4 * 2 * 16 * (bn / 4 + 4) * 4;
+    const size_t stages = (size_t)(ahead + 1) * 2 * (bm / 16) * 1024, strips = (size_t)4 * 2 * 16 * (bn / 4 + 4) * 4;
     const size_t lds = (stages > strips ? stages : strips) + (size_t)2 * bm * 4;
     // the kernels of one epilogue: the residual sum into float32 with whole quads of columns; the
     // rotation with a table of angles
     const int one = splits > 1 ? -1 : (mode == EPI_ADD && N % 4 == 0) ? EPI_ADD : (mode == EPI_ROPE && e.rs.cos_sin) ? EPI_ROPE : -1;
-#define GO(T, NI, MODE) gemm_wreg_kernel<T, NI, MODE><<<grid, block, lds, stream>>>((const T*)X, (const T*)Wt, K, k_per_split, ws, e)
-#define BY_MODE(T, NI)                              \
-    do {                                            \
-        if (one == EPI_ADD) GO(T, NI, EPI_ADD);     \
-        else if (one == EPI_ROPE) GO(T, NI, EPI_ROPE); \
-        else GO(T, NI, -1);                         \
+#define GO(T, NI, MODE, MJ, A)                                                                            \
+    do {                                                                                                  \
+        auto kfn = gemm_wreg_kernel<T, NI, MODE, MJ, A>;                                                  \
+        if (lds > 64 * 1024) {                                                                            \
+            static bool allowed = false;           /* more than 64 KiB of LDS is asked for once */       \
+            if (!allowed && hipFuncSetAttribute((const void*)kfn, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds) != hipSuccess) \
+                return LI_HIP_ERROR;                                                                      \
+            allowed = true;                                                                               \
+        }                                                                                                 \
+        kfn<<<grid, block, lds, stream>>>((const T*)X, (const T*)Wt, K, k_per_split, ws, e);              \
     } while (0)
-#define LAUNCH(T)                            \
-    do {                                     \
-        if (tile == 0) BY_MODE(T, 4);        \
-        else if (tile == 1) BY_MODE(T, 3);   \
-        else BY_MODE(T, 2);                  \
+#define BY_MODE(T, NI, MJ, A)                             \
+    do {                                                  \
+        if (one == EPI_ADD) GO(T, NI, EPI_ADD, MJ, A);    \
+        else if (one == EPI_ROPE) GO(T, NI, EPI_ROPE, MJ, A); \
+        else GO(T, NI, -1, MJ, A);                        \
+    } while (0)
+#define LAUNCH(T)                                       \
+    do {                                                \
+        if (tile == 0) BY_MODE(T, 4, 8, 2);             \
+        else if (tile == 1) BY_MODE(T, 3, 8, 2);        \
+        else if (few_rows == 1) BY_MODE(T, 2, 4, 4);    \
+        else if (few_rows == 2) BY_MODE(T, 2, 8, 4);    \
+        else BY_MODE(T, 2, 8, 2);                       \
     } while (0)
     if (dt == DT_F16) LAUNCH(f16); else LAUNCH(bf16);
 #undef LAUNCH

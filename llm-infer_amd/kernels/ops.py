@@ -330,12 +330,17 @@ def linear(x: torch.Tensor, w, mode: int = EPI_STORE, out: torch.Tensor | None =
                                 int(parts[1]) if len(parts) > 1 else 0, int(parts[2]) if len(parts) > 2 else 0,
                                 rs, _stream()), "gemm_rows")
         return out
-    if kind.startswith("wreg"):                                # "wreg[:<tile>[:<splits>]]" (a test's choice)
+    if kind.startswith("wreg"):                                # "wreg[:<tile>[:<splits>[:<few rows>]]]" (a test's choice)
         _need(tiled and fast_ok and m * k * 2 < (1 << 32), "gemm_wreg: a tiled weight, X below 4 GiB")
         parts = kind.split(":")
         tile, splits = _wreg_plan(m, n, k)
+        # up to 64 rows against the narrowest tile: a tile of 64 rows of X (none fetched or multiplied that is not
+        # there) with W four steps ahead (measured at 64 rows: gate/up 53.9 -> 46.0 us, down 35.9 -> 35.0 and 29.5
+        # with K in 8; the same depth with 128 rows of X gained 2% at 128 rows and is not used)
+        few_rows = 1 if (tile == 2 and m <= 64) else 0
         if len(parts) > 1:
             tile, splits = int(parts[1]), int(parts[2]) if len(parts) > 2 else 1
+            few_rows = int(parts[3]) if len(parts) > 3 else 0
         ws = _workspace(splits * m * n, x.device) if splits > 1 else None
         # with K split, the kernel that adds the partial sums to the residual also takes the norm that reads
         # the finished rows next, if the block has said which one that is
@@ -348,7 +353,8 @@ def linear(x: torch.Tensor, w, mode: int = EPI_STORE, out: torch.Tensor | None =
             normed = torch.empty((m, n), dtype=x.dtype, device=x.device)
             na = _NormAfter(nxt.data_ptr(), normed.data_ptr(), DT[x.dtype], eps)
         _check(lib.li_gemm_wreg(_ptr(x), _ptr(wd), DT[x.dtype], _ptr(out), out_dt, mode, m, n, k, tile, splits,
-                                _ptr(ws), rs, ctypes.byref(na) if na is not None else None, _stream()), "gemm_wreg")
+                                _ptr(ws), rs, ctypes.byref(na) if na is not None else None, few_rows, _stream()),
+               "gemm_wreg")
         if na is not None:
             out._li_normed = (normed, nxt, eps, out._version)
         return out
@@ -405,7 +411,11 @@ def _wreg_cost(tile: int, splits: int, m: int, n: int, k: int) -> float:
     us = 0.0
     for count, (a, c) in ((full, times[-1]), (1 if rest else 0, times[-(-rest // 256) - 1])):
         us += count * (a * k_split / 4096 + c)
-    main = max(us, n * k * 2 / 5.5e6)
+    # W streams at 5.5 TB/s when every CU has a workgroup, at less with fewer workgroups
+    groups = -(-m // bm) * -(-n // bn) * splits
+    main = max(us, n * k * 2 / (5.5e6 * min(1.0, groups / 256)))
+    if tile == 2 and m <= 64:
+        main *= 0.87                                  # the 64-row tile of X with W four steps ahead
     reduce = 2.5 + 2 * splits * m * n * 4 / 3.0e6 if splits > 1 else 0.0
     return main + 5.5 + reduce
 

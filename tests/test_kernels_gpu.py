@@ -126,6 +126,8 @@ def test_linear_tiled_weights(ops, M, N, K, dt):
     kinds = [None, "mfma:0:1", "mfma:1:2", "mfma:2:1", "big:0", "big:1", "big:0:2", "big:1:5"] + (["gemv_mfma"] if M <= 16 else [])
     # W into registers (tiles of 256, 192, 128 rows of W): the planner's choice and every tile, K whole and split
     kinds += ["wreg", "wreg:0", "wreg:1", "wreg:2", "wreg:0:2", "wreg:1:5", "wreg:2:3"]
+    # the narrowest tile with W four steps ahead, with 64 rows of X (:1) and with 128 (:2), K whole and split
+    kinds += ["wreg:2:1:1", "wreg:2:3:1", "wreg:2:1:2", "wreg:2:4:2"]
     # all of K in one workgroup, the rows of X through LDS of each wave's own (up to 128 rows): one and two tiles of W
     kinds += ["rows", "rows:1", "rows:2"] if M <= 128 else []
     for kind in kinds:
