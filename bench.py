@@ -6,6 +6,9 @@
 A step is one decode step of the generation loop's own runner (bookkeeping, the
 model's forward pass from the cache, sampling, tokens back to the host) for a
 batch of 8 sequences whose contexts end at the benchmark's context length.  The
+runner replays recorded steps; the window of positions is walked once untimed
+first, so that no step is recorded inside the timed ones (`warmup` counts all
+untimed steps).  The
 line printed also holds the prefill of one 2,048-token prompt, the decode step's
 share of the HBM roofline, and decode throughput at batch 1 and 64.
 """
@@ -163,9 +166,12 @@ def measure(args) -> dict:
         weight_bytes += n * (4 if spec.kind == "vector" else elem)
     kv_bytes_per_token = cache.bytes_per_token()
 
-    def decode_run(batch, steps, warmup):
+    def decode_run(batch, steps, warmup, timed=True):
         """Fills `batch` sequences to just below the context length with random keys and values,
-        then times `steps` decode steps."""
+        then times `steps` decode steps.  The runner records a step the first time it meets its size and its
+        bucket of context lengths, and the window of positions crosses a bucket's edge (8,128 tokens at a
+        context of 8,192); `timed=False` walks the window once beforehand so that the timed steps are all
+        replays, as every step of a long generation is."""
         start = args.context - steps - warmup - 2            # warm-up enqueues one step more than it returns
         slots = [engine.alloc_slot() for _ in range(batch)]
         cache.grow(slots, [start] * batch)
@@ -193,7 +199,10 @@ def measure(args) -> dict:
 
     results = {}
     for b in batches:
+        decode_run(b, args.steps, args.warmup, timed=False)
+        recorded = engine.decode_counts["recorded"]
         dt, ctx_mid = decode_run(b, args.steps, args.warmup)
+        assert engine.decode_counts["recorded"] == recorded, "a step was recorded inside the timed steps"
         results[b] = (dt, ctx_mid)
         print(f"[bench] decode batch {b}: {dt / args.steps * 1e3:.3f} ms/step, "
               f"{b * args.steps / dt:.1f} tok/s", file=sys.stderr, flush=True)
@@ -273,7 +282,8 @@ def measure(args) -> dict:
     line = {
         "metric": f"decode tokens/s, {args.shape} shape, batch {args.batch}, context {args.context}",
         "value": round(args.batch * args.steps / dt, 2), "unit": "tokens/s", "n_gpus": 1,
-        "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(ms, 4),
+        # (untimed: a first walk over the same positions, in which the steps are recorded, then the warm-up)
+        "steps": args.steps, "warmup": 2 * args.warmup + args.steps, "ms_per_step": round(ms, 4),
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": args.dtype,
         "data": "synthetic: random weights N(0, 0.02), uniform random token ids, cache filled with random "
                 "keys and values up to the context length",
