@@ -229,7 +229,8 @@ __global__ __launch_bounds__(256) void gemm_big_kernel(const T* __restrict__ X, 
 // 8 NI KiB a wave instead of 4 NI).
 template <class T, int NI, int MODE, int MJ = 8, int A = 2>
 __global__ __launch_bounds__(256) void gemm_wreg_kernel(const T* __restrict__ X, const T* __restrict__ Wt,
-                                                        int K, int k_per_split, float* __restrict__ ws, Epilogue e) {
+                                                        int K, int k_per_split, float* __restrict__ ws, Epilogue e,
+                                                        int wg_blocks) {
     typedef typename Vec<T>::v8 v8;
     // A step is 64 of K: two halves of 32, each one matrix instruction deep.
     // MJ: fragments of X (16 rows each) per wave and half step; every wave takes all the tile's rows of X
@@ -244,7 +245,11 @@ __global__ __launch_bounds__(256) void gemm_wreg_kernel(const T* __restrict__ X,
     const int wn = wave;
     int bx, by, bz;
     tile_of_workgroup(8, bx, by, bz);
-    const int m0 = bx * BM, n0 = by * BN;
+    // wg_blocks: the blocks of 16 rows of W that a workgroup takes of its 4 NI (fewer: more workgroups, for a
+    // product whose full tiles would leave CUs without one); a wave whose block lies beyond them fetches and
+    // multiplies the workgroup's last block again and stores nothing of it
+    const int m0 = bx * BM, n0 = by * 16 * wg_blocks;
+    const int n_end = min(e.N, n0 + 16 * wg_blocks);
     const int kb = bz * k_per_split, ke = min(K, kb + k_per_split);
     // a share of K that is 32 more than a multiple of 64 ends with a step of one half
     const int n_halves = (ke - kb) >> 5, n_steps = (n_halves + 1) >> 1;
@@ -254,7 +259,7 @@ __global__ __launch_bounds__(256) void gemm_wreg_kernel(const T* __restrict__ X,
     const T* wsrc[NI];
 #pragma unroll
     for (int i = 0; i < NI; ++i) {
-        const int blk = min(n0 / 16 + wn * NI + i, w_blocks - 1);
+        const int blk = min(n0 / 16 + min(wn * NI + i, wg_blocks - 1), w_blocks - 1);
         wsrc[i] = Wt + (((int64_t)blk * steps + (kb >> 5)) * 64 + lane) * 8;
     }
     // This wave's share of a stage of X.  A 1 KiB unit holds 8 rows x 64 of K, so that the 8 lanes of a row
@@ -439,7 +444,7 @@ __global__ __launch_bounds__(256) void gemm_wreg_kernel(const T* __restrict__ X,
 #pragma unroll
             for (int it = 0; it < NI; ++it) {
                 const int m = m0 + 16 * j + row_of[it];
-                if (m < e.M && col_of[it] < e.N) c[it] = *(const f32x4*)(C + (int64_t)m * e.N + col_of[it]);
+                if (m < e.M && col_of[it] < n_end) c[it] = *(const f32x4*)(C + (int64_t)m * e.N + col_of[it]);
             }
         };
         fetch(0, res[0]);
@@ -451,7 +456,7 @@ __global__ __launch_bounds__(256) void gemm_wreg_kernel(const T* __restrict__ X,
 #pragma unroll
             for (int it = 0; it < NI; ++it) {
                 const int m = m0 + 16 * j + row_of[it];
-                if (m < e.M && col_of[it] < e.N) {
+                if (m < e.M && col_of[it] < n_end) {
                     f32x4 o = res[j & 1][it];
                     const f32x4 v = *(const f32x4*)(stage + row_of[it] * SLD + (col_of[it] - nb));
                     o[0] += v[0]; o[1] += v[1]; o[2] += v[2]; o[3] += v[3];
@@ -481,7 +486,7 @@ __global__ __launch_bounds__(256) void gemm_wreg_kernel(const T* __restrict__ X,
             int row, n;
             place_of(lane, row, n);
             if constexpr (MODE == EPI_ROPE) {
-                if (mb + row < e.M && n < e.N) rope_angles(rs, mb + row, 0, n / rs.hd, n % rs.hd, ang, true);
+                if (mb + row < e.M && n < n_end) rope_angles(rs, mb + row, 0, n / rs.hd, n % rs.hd, ang, true);
             }
 #pragma unroll 1
             for (int q = lane; q < 2 * 16 * QUADS; q += 64) {
@@ -492,14 +497,15 @@ __global__ __launch_bounds__(256) void gemm_wreg_kernel(const T* __restrict__ X,
                     const f32x2 now[2] = {ang[0], ang[1]};
                     if (q + 64 < 2 * 16 * QUADS) {
                         place_of(q + 64, row, n);
-                        if (mb + row < e.M && n < e.N) rope_angles(rs, mb + row, 0, n / rs.hd, n % rs.hd, ang, true);
+                        if (mb + row < e.M && n < n_end) rope_angles(rs, mb + row, 0, n / rs.hd, n % rs.hd, ang, true);
                     }
-                    if (m < e.M && col < e.N) {
+                    if (m < e.M && col < n_end) {
                         const int head = col / rs.hd;
                         rope_store4(rs, m, head, col - head * rs.hd, vv, row_pos[m - m0], row_page[m - m0], now);
                     }
                 } else {
                     if (q + 64 < 2 * 16 * QUADS) place_of(q + 64, row, n);
+                    if (col >= n_end) continue;
                     if (gridDim.z == 1) epilogue4(e, m, col, vv);
                     else if (m < e.M) {
                         float* p = ws + ((int64_t)bz * e.M + m) * e.N + col;
@@ -567,9 +573,11 @@ extern "C" int li_gemm_big(const void* X, const void* W, int tiled, int dt, void
 // takes the norm of the finished rows; it must fit (norm_after_fits), the caller has checked the same.
 // few_rows (tile 2 only): 1 = the tile has 64 rows of X, 2 = 128 rows; either way W is fetched four steps ahead
 // instead of two (for products of up to 128 rows, where a workgroup has a CU to itself); 0 = neither.
+// wg_blocks: blocks of 16 rows of W a workgroup, from 1 to the tile's own number (0: that number); fewer make
+// more workgroups of a product whose full tiles would leave CUs without one.
 extern "C" int li_gemm_wreg(const void* X, const void* Wt, int dt, void* C, int out_dt, int mode,
                             int M, int N, int K, int tile, int splits, float* ws, const RopeStore* rs,
-                            const NormAfter* na, int few_rows, hipStream_t stream) {
+                            const NormAfter* na, int few_rows, int wg_blocks, hipStream_t stream) {
     int rc = check_common(X, Wt, C, M, N, K, mode, out_dt);
     if (rc) return rc;
     if (dt != DT_F16 && dt != DT_BF16) return LI_BAD_ARG;
@@ -582,10 +590,12 @@ extern "C" int li_gemm_wreg(const void* X, const void* Wt, int dt, void* C, int 
     rc = make_epilogue(e, C, mode, out_dt, M, N, rs);
     if (rc) return rc;
     const int bn = 256 - 64 * tile, bm = few_rows == 1 ? 64 : 128, bk = 32, ahead = few_rows ? 4 : 2;
+    if (wg_blocks == 0) wg_blocks = bn / 16;
+    if (wg_blocks < 1 || wg_blocks > bn / 16) return LI_BAD_ARG;
     int k_per_split = ((K + splits - 1) / splits + bk - 1) / bk * bk;
     splits = (K + k_per_split - 1) / k_per_split;
     if (na && !(splits > 1 && norm_after_fits(na, e, ws))) return LI_BAD_ARG;
-    dim3 grid((M + bm - 1) / bm, (N + bn - 1) / bn, splits), block(256);
+    dim3 grid((M + bm - 1) / bm, ((N + 15) / 16 + wg_blocks - 1) / wg_blocks, splits), block(256);
     // ahead + 1 stages of X (a step is 64 of K); the epilogue stages two strips of 16 x (bn / 4 + 4) floats a wave
     // in the same LDS, and behind both lie a position and a page for each of the tile's rows
     const size_t stages = (size_t)(ahead + 1) * 2 * (bm / 16) * 1024, strips = (size_t)4 * 2 * 16 * (bn / 4 + 4) * 4;
@@ -602,7 +612,7 @@ extern "C" int li_gemm_wreg(const void* X, const void* Wt, int dt, void* C, int 
                 return LI_HIP_ERROR;                                                                      \
             allowed = true;                                                                               \
         }                                                                                                 \
-        kfn<<<grid, block, lds, stream>>>((const T*)X, (const T*)Wt, K, k_per_split, ws, e);              \
+        kfn<<<grid, block, lds, stream>>>((const T*)X, (const T*)Wt, K, k_per_split, ws, e, wg_blocks);   \
     } while (0)
 #define BY_MODE(T, NI, MJ, A)                             \
     do {                                                  \

@@ -336,11 +336,14 @@ def linear(x: torch.Tensor, w, mode: int = EPI_STORE, out: torch.Tensor | None =
         tile, splits = _wreg_plan(m, n, k)
         # up to 64 rows against the narrowest tile: a tile of 64 rows of X (none fetched or multiplied that is not
         # there) with W four steps ahead (measured at 64 rows: gate/up 53.9 -> 46.0 us, down 35.9 -> 35.0 and 29.5
-        # with K in 8; the same depth with 128 rows of X gained 2% at 128 rows and is not used)
+        # with K in 8; the same depth with 128 rows of X: by itself gate/up at 128 rows 61.5 -> 53.6 us, in a decode
+        # step at batch 128 nothing (11.41 and 11.47 ms), and is not used)
         few_rows = 1 if (tile == 2 and m <= 64) else 0
-        if len(parts) > 1:
+        wg_blocks = _wreg_blocks(tile, splits, m, n)
+        if len(parts) > 1:                                     # "wreg:<tile>:<splits>:<few rows>:<blocks of W>"
             tile, splits = int(parts[1]), int(parts[2]) if len(parts) > 2 else 1
             few_rows = int(parts[3]) if len(parts) > 3 else 0
+            wg_blocks = int(parts[4]) if len(parts) > 4 else 0
         ws = _workspace(splits * m * n, x.device) if splits > 1 else None
         # with K split, the kernel that adds the partial sums to the residual also takes the norm that reads
         # the finished rows next, if the block has said which one that is
@@ -353,7 +356,8 @@ def linear(x: torch.Tensor, w, mode: int = EPI_STORE, out: torch.Tensor | None =
             normed = torch.empty((m, n), dtype=x.dtype, device=x.device)
             na = _NormAfter(nxt.data_ptr(), normed.data_ptr(), DT[x.dtype], eps)
         _check(lib.li_gemm_wreg(_ptr(x), _ptr(wd), DT[x.dtype], _ptr(out), out_dt, mode, m, n, k, tile, splits,
-                                _ptr(ws), rs, ctypes.byref(na) if na is not None else None, few_rows, _stream()),
+                                _ptr(ws), rs, ctypes.byref(na) if na is not None else None, few_rows, wg_blocks,
+                                _stream()),
                "gemm_wreg")
         if na is not None:
             out._li_normed = (normed, nxt, eps, out._version)
@@ -400,19 +404,34 @@ _WREG_ROUND_US = {0: ((53.0, 9.0), (103.0, 5.0)), 1: ((35.0, 13.0), (73.0, 12.0)
                   2: ((31.4, 3.4), (57.1, 3.8), (89.0, 0.0))}
 
 
+def _wreg_blocks(tile: int, splits: int, m: int, n: int) -> int:
+    """Blocks of 16 rows of W that a workgroup of gemm_wreg takes: all of its tile's, or, for a product of up to
+    64 rows against the narrowest tile (one workgroup a CU at a time, one tile of X), as few as make the rounds of
+    256 workgroups times the blocks of each the least (28,672 rows of W: 224 workgroups of 8 blocks leave 32 CUs
+    idle, 256 workgroups of 7 none; measured at 64 rows: 49.3 -> 46.8 us, and 22,016 rows of W with 6 blocks
+    44.8 -> 37.5).  With the 128-row tile of X the same measured no gain, and where K is split the splits are what
+    fills the CUs."""
+    full = _WREG_TILES[tile][0] // 16
+    if tile != 2 or m > 64 or splits > 1:
+        return full
+    blocks16 = -(-n // 16)
+    return min(range(full, full // 2, -1), key=lambda b: -(-(-(-blocks16 // b) * splits) // 256) * b)
+
+
 def _wreg_cost(tile: int, splits: int, m: int, n: int, k: int) -> float:
     """Estimated microseconds of one gemm_wreg launch (and its split-K reduction): rounds of workgroups
     at the measured time of a round, not below the time to stream W once; a fixed cost for the launch,
     the first tiles and the epilogue; the partial sums written and read back."""
     bn, bm = _WREG_TILES[tile]
     times = _WREG_ROUND_US[tile]
-    full, rest = divmod(-(-m // bm) * -(-n // bn) * splits, 256 * len(times))
+    wg_blocks = _wreg_blocks(tile, splits, m, n)
+    groups = -(-m // bm) * -(-(-(-n // 16)) // wg_blocks) * splits
+    full, rest = divmod(groups, 256 * len(times))
     k_split = -(-(-(-k // splits)) // 32) * 32
     us = 0.0
     for count, (a, c) in ((full, times[-1]), (1 if rest else 0, times[-(-rest // 256) - 1])):
-        us += count * (a * k_split / 4096 + c)
+        us += count * (a * wg_blocks * 16 / bn * k_split / 4096 + c)
     # W streams at 5.5 TB/s when every CU has a workgroup, at less with fewer workgroups
-    groups = -(-m // bm) * -(-n // bn) * splits
     main = max(us, n * k * 2 / (5.5e6 * min(1.0, groups / 256)))
     if tile == 2 and m <= 64:
         main *= 0.87                                  # the 64-row tile of X with W four steps ahead

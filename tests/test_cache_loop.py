@@ -282,6 +282,21 @@ def test_the_plan_for_products_of_a_few_dozen_rows():
                for m in (24, 48, 96) for n, k in ((2048, 8192), (4096, 11008), (4096, 14336)))
 
 
+def test_blocks_of_w_a_workgroup_for_products_whose_tiles_leave_cus_idle():
+    """Up to 64 rows of X, K whole, the narrowest tile: a workgroup takes as few of its tile's eight blocks of 16 rows
+    of W as make (rounds of 256 workgroups) x (blocks) least; everything else takes the whole tile."""
+    from llm_infer_amd.kernels import ops
+    assert ops._wreg_blocks(2, 1, 64, 28672) == 7            # 1,792 blocks: 224 workgroups of 8, 256 of 7
+    assert ops._wreg_blocks(2, 1, 64, 22016) == 6            # 1,376 blocks: 172 of 8, 230 of 6
+    assert ops._wreg_blocks(2, 1, 64, 4096 * 8) == 8         # 2,048 blocks: 256 of 8 already
+    assert ops._wreg_blocks(2, 8, 64, 4096) == 8             # K split: the splits fill the CUs
+    assert ops._wreg_blocks(2, 1, 128, 28672) == 8 and ops._wreg_blocks(0, 1, 64, 28672) == 16
+    for n in range(16, 40000, 1008):
+        b = ops._wreg_blocks(2, 1, 33, n)
+        groups = lambda blocks: -(-(-(-n // 16)) // blocks)
+        assert 5 <= b <= 8 and -(-groups(b) // 256) * b <= -(-groups(8) // 256) * 8
+
+
 def test_the_index_arrays_of_a_recorded_prefill_step():
     """A recorded prefill step reads its step from one buffer of fixed layout; what the step does not fill is
     padding that belongs to no sequence: tokens on the scratch slot, sequences without tokens, tiles that begin
