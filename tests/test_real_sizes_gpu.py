@@ -103,3 +103,41 @@ def test_three_schedules_at_real_sizes(case, dtype, tmp_path):
                     worst, worst_key = e, (rid, p)
         assert seen == {(r, p) for r, t in requests.items() for p in range(len(t))}, what
         assert worst < tol, f"{case.name} {what} {dtype}: first look at {worst_key}: error {worst:.3e}, allowed {tol:.3e}"
+
+
+def test_recorded_decode_steps_at_real_sizes(tmp_path):
+    """Greedy generation through recorded steps at the 8B layer's sizes: twenty sequences that end at different
+    times, so the recorded steps run 24, 16, 12, 8, 4, 2 and 1 rows (idle rows on the scratch slot) through the
+    kernels for 17 to 128 rows and for up to 16, the prompts through recorded prefill steps the second time.
+    The tokens are those of the eager steps, and where the plain implementation's two best logits lie further
+    apart than the engine may err, they are the plain implementation's choice."""
+    import llm_infer_amd as lib
+    cfg = CONFIGS["8b"]
+    weights = make_weights("8b", cfg)
+    folder = str(tmp_path / "m")
+    P.write_model(folder, cfg, weights)
+    eng = lib.load(folder, dtype="float16", max_tokens=20 * 192, n_slots=24)     # 20 live rows run as 24
+    g = torch.Generator().manual_seed(5)
+    lengths = [3, 70, 17, 64, 33, 5, 48, 65, 9, 100, 2, 31, 80, 12, 57, 24, 6, 90, 40, 1]
+    budgets = [40, 6, 22, 9, 35, 14, 4, 28, 11, 19, 38, 7, 25, 16, 3, 31, 13, 21, 5, 36]
+    prompts = [torch.randint(0, cfg["vocab_size"], (n,), generator=g).tolist() for n in lengths]
+    eager = eng.generate(prompts, max_new_tokens=budgets, temperature=0.0, use_graph=False, stop_token_ids=())
+    assert [len(o) for o in eager] == budgets
+    first = eng.generate(prompts, max_new_tokens=budgets, temperature=0.0, use_graph=True, stop_token_ids=())
+    again = eng.generate(prompts, max_new_tokens=budgets, temperature=0.0, use_graph=True, stop_token_ids=())
+    assert first == eager and again == eager
+    assert sorted({k[0] for k in eng._graphs}) == [1, 2, 4, 8, 12, 16, 24]
+    assert eng.decode_counts["replayed"] > eng.decode_counts["recorded"] > 0
+    checked = 0
+    for i in (0, 4, 10):                                   # the three that decode longest, from short prompts
+        whole = prompts[i] + eager[i]
+        ref = P.forward(weights, cfg, whole, torch.float64)
+        own = (P.forward(weights, cfg, whole, torch.float64, torch.float16) - ref).abs().max().item()
+        tol = 3 * own + 1e-6 * ref.std().item()
+        for j, tok in enumerate(eager[i]):
+            top = torch.topk(ref[len(prompts[i]) + j - 1], 2)
+            if (top.values[0] - top.values[1]).item() > 2 * tol:
+                assert tok == top.indices[0].item(), (i, j)
+                checked += 1
+    assert checked >= 60, checked
+    assert eng.cache.slots.n_free == eng.cache.n_slots
