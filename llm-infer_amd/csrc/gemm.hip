@@ -290,33 +290,6 @@ __global__ void tile_weight_kernel(const T* __restrict__ W, T* __restrict__ out,
     *(v8*)(out + i * 8) = n < N ? *(const v8*)(W + (int64_t)n * K + k) : z;
 }
 
-// A norm split over two products of a decode step (up to 16 rows), so that no norm kernel runs between
-// them.  The product that adds into the residual stream (EPI_ADD) also leaves, for the rows x it has
-// just completed, (a) the sums of squares as one partial sum per workgroup and row, `ss` [blocks, 16], and
-// (b) x * w * scale rounded to the 16-bit type, `xw` [M, N], w being the weight of the norm that reads
-// x next (RowsOut).  The next product takes `xw` as its X and multiplies its sums by
-// 1 / (scale * sqrt(mean(x^2) + eps)) from the partial sums (RowScale): together  W . (x / rms * w),
-// the norm of include/kernels_cpu.hpp:43-54 in another order of rounding.  `scale` keeps x * w inside
-// float16's range: one power of two for each row, near 1 / (8 rms) of the row as it was when a norm was last
-// taken of it (`row_scale`, written by the norm kernel or by the product that finished that norm:
-// row_scale_for in common.h), so that the rounding is as fine for a model whose residual stream is of the
-// order of 0.01 or 1000 as for one of the order of 1; without it the fixed `scale`.
-struct RowsOut {
-    float* ss;               // [gridDim.x, 16]
-    void* xw;                // [M, N] in the product's 16-bit type
-    const float* w;          // [N] weight of the next norm
-    float scale;
-    const float* row_scale;  // [16] or null
-};
-struct RowScale {
-    const float* ss;         // [P, 16]
-    int P;
-    float eps;               // of the norm
-    float inv_scale;         // 1 / RowsOut.scale
-    const float* row_scale;  // [16] the scales RowsOut used, or null (then inv_scale)
-    float* next_scale;       // [16] or null: row_scale_for(rms) of these rows, for the product that adds into them next
-};
-
 template <class T, int NT, int MT, int KW>
 __global__ __launch_bounds__(64 * KW) void gemv_tiled_kernel(const T* __restrict__ X, const T* __restrict__ Wt,
                                                              int K, Epilogue e, RowsOut ro, RowScale rsc) {
@@ -763,7 +736,7 @@ extern "C" int li_tile_weight(const void* W, void* out, int dt, int N, int K, hi
 static void gemv_tiled_shape(int M, int N, int K, int& nt, int& kw, int& blocks) {
     const int n_tiles = (N + 15) / 16;
     const int mt = (M + 15) / 16;
-    if (nt <= 0) nt = (mt >= 2 || (M > 12 && N >= 16384)) ? 2 : 1;           // measured on MI355X
+    if (nt <= 0) nt = (mt >= 2 || (M > 12 && N >= 6144)) ? 2 : 1;            // measured on MI355X (16 rows, 6,144 x 4,096: 14.5 against 16.3 us)
     if (mt >= 3) nt = 2;
     blocks = (n_tiles + nt - 1) / nt;
     if (kw <= 0) kw = (K >= 8192 || blocks < 320 || blocks > 4096) ? 8 : 4;   // measured on MI355X

@@ -195,6 +195,33 @@ static __global__ void splitk_reduce_kernel(const float* __restrict__ ws, int sp
 }
 
 
+// A norm split over two products of a decode step (up to 16 rows), so that no norm kernel runs between
+// them.  The product that adds into the residual stream (EPI_ADD) also leaves, for the rows x it has
+// just completed, (a) the sums of squares as one partial sum per workgroup and row, `ss` [blocks, 16], and
+// (b) x * w * scale rounded to the 16-bit type, `xw` [M, N], w being the weight of the norm that reads
+// x next (RowsOut).  The next product takes `xw` as its X and multiplies its sums by
+// 1 / (scale * sqrt(mean(x^2) + eps)) from the partial sums (RowScale; gemv_tiled, and gemm_wreg's kernel of every epilogue): together  W . (x / rms * w),
+// the norm of include/kernels_cpu.hpp:43-54 in another order of rounding.  `scale` keeps x * w inside
+// float16's range: one power of two for each row, near 1 / (8 rms) of the row as it was when a norm was last
+// taken of it (`row_scale`, written by the norm kernel or by the product that finished that norm:
+// row_scale_for in common.h), so that the rounding is as fine for a model whose residual stream is of the
+// order of 0.01 or 1000 as for one of the order of 1; without it the fixed `scale`.
+struct RowsOut {
+    float* ss;               // [gridDim.x, 16]
+    void* xw;                // [M, N] in the product's 16-bit type
+    const float* w;          // [N] weight of the next norm
+    float scale;
+    const float* row_scale;  // [16] or null
+};
+struct RowScale {
+    const float* ss;         // [P, 16]
+    int P;
+    float eps;               // of the norm
+    float inv_scale;         // 1 / RowsOut.scale
+    const float* row_scale;  // [16] the scales RowsOut used, or null (then inv_scale)
+    float* next_scale;       // [16] or null: row_scale_for(rms) of these rows, for the product that adds into them next
+};
+
 // The RMS norm that reads the rows of a residual sum next (src/model/block.cpp:127, 191): weight [N], eps, and
 // where its result goes ([M, N] of out_dt).
 struct NormAfter {

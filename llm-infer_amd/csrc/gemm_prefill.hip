@@ -230,7 +230,7 @@ __global__ __launch_bounds__(256) void gemm_big_kernel(const T* __restrict__ X, 
 template <class T, int NI, int MODE, int MJ = 8, int A = 2>
 __global__ __launch_bounds__(256) void gemm_wreg_kernel(const T* __restrict__ X, const T* __restrict__ Wt,
                                                         int K, int k_per_split, float* __restrict__ ws, Epilogue e,
-                                                        int wg_blocks) {
+                                                        int wg_blocks, RowScale rsc) {
     typedef typename Vec<T>::v8 v8;
     // A step is 64 of K: two halves of 32, each one matrix instruction deep.
     // MJ: fragments of X (16 rows each) per wave and half step; every wave takes all the tile's rows of X
@@ -358,8 +358,32 @@ __global__ __launch_bounds__(256) void gemm_wreg_kernel(const T* __restrict__ X,
         fetch_w(2 * a, ring[2 * a]);
         fetch_w(2 * a + 1, ring[2 * a + 1]);
     }
+    // RowScale (MODE -1, at most 16 rows of X, K whole; the host sees to it): the partial sums of squares of row
+    // tid % 16 are dealt to the 16 groups of 16 threads; they are fetched behind the first loads, and everything is
+    // waited for once (the loop's counts are upper bounds and stay right with fewer loads in flight).  The groups'
+    // sums lie behind the stages of X, where the epilogue finds them.
+    constexpr int STRIPS_BYTES = 4 * 2 * 16 * (16 * NI + 4) * 4;
+    constexpr int INFO = XBUFS * STAGE > STRIPS_BYTES ? XBUFS * STAGE : STRIPS_BYTES;     // behind the stages and the strips
+    float* row_ss = (float*)(smem_raw + INFO + 2 * BM * 4);                               // [16 groups][16 rows], then [16] factors
+    bool scaled = false;
+    if constexpr (MODE == -1) {
+        scaled = rsc.ss != nullptr;
+        if (scaled) {
+            const int r = tid & 15, grp = tid >> 4;
+            float sum = 0.f;
+            for (int p0 = grp; p0 < rsc.P; p0 += 16 * 8) {
+                float v[8];
+#pragma unroll
+                for (int c = 0; c < 8; ++c) v[c] = rsc.ss[min(p0 + 16 * c, rsc.P - 1) * 16 + r];
+#pragma unroll
+                for (int c = 0; c < 8; ++c) sum += (p0 + 16 * c < rsc.P) ? v[c] : 0.f;
+            }
+            row_ss[grp * 16 + r] = sum;                     // (the compiler waits for the loads it issued: all of them)
+            __builtin_amdgcn_s_waitcnt(0x0070);             // vmcnt(0): the first loads too
+        }
+    }
     // X of step 0 has landed (and W of step 0 with it)
-    __builtin_amdgcn_s_waitcnt(0x0F70 | (((A - 1) * PER_STEP) & 15) | ((((A - 1) * PER_STEP) >> 4) << 14));
+    if (!scaled) __builtin_amdgcn_s_waitcnt(0x0F70 | (((A - 1) * PER_STEP) & 15) | ((((A - 1) * PER_STEP) >> 4) << 14));
     __builtin_amdgcn_s_barrier();
     WREG_EIGHT(WREG_READ, lds_lane)
     int cur = 0;                                                   // byte offset of the buffer of step s
@@ -406,7 +430,7 @@ __global__ __launch_bounds__(256) void gemm_wreg_kernel(const T* __restrict__ X,
     // block is W row 4 (lane / 16) + q, X row lane % 16; read back, consecutive lanes hold consecutive
     // quads of columns of one row.  A wave has room for two strips.
     constexpr int SLD = 16 * NI + 4, QUADS = 4 * NI, STRIP = 16 * SLD;
-    constexpr int INFO = XBUFS * STAGE > 4 * 2 * STRIP * 4 ? XBUFS * STAGE : 4 * 2 * STRIP * 4;   // behind the stages and the strips
+    static_assert(STRIPS_BYTES == 4 * 2 * STRIP * 4, "the strips' size");
     int* row_pos = (int*)(smem_raw + INFO);
     int* row_page = row_pos + BM;
     if constexpr (MODE == EPI_ROPE) {
@@ -416,6 +440,16 @@ __global__ __launch_bounds__(256) void gemm_wreg_kernel(const T* __restrict__ X,
             row_pos[tid] = p;
             row_page[tid] = (e.rs.K > 0 && n0 + BN > e.rs.H * e.rs.hd)
                                 ? e.rs.page_table[(int64_t)e.rs.tok_slot[m] * e.rs.max_pages + p / PAGE] : 0;
+        }
+    }
+    if constexpr (MODE == -1) {
+        if (scaled && tid < 16) {
+            // this row: the groups' sums in the order of the groups, then 1 / (scale * rms)
+            float ss = row_ss[tid];
+            for (int grp = 1; grp < 16; ++grp) ss += row_ss[grp * 16 + tid];
+            const float rms = sqrtf(ss / (float)K + rsc.eps);
+            row_ss[256 + tid] = (rsc.row_scale ? 1.f / rsc.row_scale[tid] : rsc.inv_scale) / rms;
+            if (rsc.next_scale && blockIdx.x == 0 && blockIdx.y == 0 && blockIdx.z == 0) rsc.next_scale[tid] = row_scale_for(rms);
         }
     }
     __syncthreads();
@@ -506,7 +540,11 @@ __global__ __launch_bounds__(256) void gemm_wreg_kernel(const T* __restrict__ X,
                 } else {
                     if (q + 64 < 2 * 16 * QUADS) place_of(q + 64, row, n);
                     if (col >= n_end) continue;
-                    if (gridDim.z == 1) epilogue4(e, m, col, vv);
+                    if (scaled) {
+                        const float f = row_ss[256 + min(m, 15)];
+                        const float sv[4] = {vv[0] * f, vv[1] * f, vv[2] * f, vv[3] * f};
+                        epilogue4(e, m, col, sv);
+                    } else if (gridDim.z == 1) epilogue4(e, m, col, vv);
                     else if (m < e.M) {
                         float* p = ws + ((int64_t)bz * e.M + m) * e.N + col;
 #pragma unroll
@@ -577,7 +615,7 @@ extern "C" int li_gemm_big(const void* X, const void* W, int tiled, int dt, void
 // more workgroups of a product whose full tiles would leave CUs without one.
 extern "C" int li_gemm_wreg(const void* X, const void* Wt, int dt, void* C, int out_dt, int mode,
                             int M, int N, int K, int tile, int splits, float* ws, const RopeStore* rs,
-                            const NormAfter* na, int few_rows, int wg_blocks, hipStream_t stream) {
+                            const NormAfter* na, int few_rows, int wg_blocks, const RowScale* rsc, hipStream_t stream) {
     int rc = check_common(X, Wt, C, M, N, K, mode, out_dt);
     if (rc) return rc;
     if (dt != DT_F16 && dt != DT_BF16) return LI_BAD_ARG;
@@ -595,11 +633,16 @@ extern "C" int li_gemm_wreg(const void* X, const void* Wt, int dt, void* C, int 
     int k_per_split = ((K + splits - 1) / splits + bk - 1) / bk * bk;
     splits = (K + k_per_split - 1) / k_per_split;
     if (na && !(splits > 1 && norm_after_fits(na, e, ws))) return LI_BAD_ARG;
+    // rsc (or null): these rows are x * weight of a norm that the product before left unfinished (RowScale); up to
+    // 16 rows, K whole, not with the epilogues that have kernels of their own
+    if (rsc && (M > 16 || splits > 1 || !rsc->ss || rsc->P <= 0 || !(rsc->inv_scale > 0.f) || mode == EPI_ADD || mode == EPI_ROPE))
+        return LI_BAD_ARG;
+    const RowScale no_scale{};
     dim3 grid((M + bm - 1) / bm, ((N + 15) / 16 + wg_blocks - 1) / wg_blocks, splits), block(256);
     // ahead + 1 stages of X (a step is 64 of K); the epilogue stages two strips of 16 x (bn / 4 + 4) floats a wave
     // in the same LDS, and behind both lie a position and a page for each of the tile's rows
     const size_t stages = (size_t)(ahead + 1) * 2 * (bm / 16) * 1024, strips = (size_t)4 * 2 * 16 * (bn / 4 + 4) * 4;
-    const size_t lds = (stages > strips ? stages : strips) + (size_t)2 * bm * 4;
+    const size_t lds = (stages > strips ? stages : strips) + (size_t)2 * bm * 4 + (256 + 16) * 4;   // and the sums of squares of RowScale
     // the kernels of one epilogue: the residual sum into float32 with whole quads of columns; the
     // rotation with a table of angles
     const int one = splits > 1 ? -1 : (mode == EPI_ADD && N % 4 == 0) ? EPI_ADD : (mode == EPI_ROPE && e.rs.cos_sin) ? EPI_ROPE : -1;
@@ -612,7 +655,8 @@ extern "C" int li_gemm_wreg(const void* X, const void* Wt, int dt, void* C, int 
                 return LI_HIP_ERROR;                                                                      \
             allowed = true;                                                                               \
         }                                                                                                 \
-        kfn<<<grid, block, lds, stream>>>((const T*)X, (const T*)Wt, K, k_per_split, ws, e, wg_blocks);   \
+        kfn<<<grid, block, lds, stream>>>((const T*)X, (const T*)Wt, K, k_per_split, ws, e, wg_blocks,     \
+                                          rsc ? *rsc : no_scale);                                         \
     } while (0)
 #define BY_MODE(T, NI, MJ, A)                             \
     do {                                                  \

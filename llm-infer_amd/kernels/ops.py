@@ -286,7 +286,12 @@ def linear(x: torch.Tensor, w, mode: int = EPI_STORE, out: torch.Tensor | None =
         _need(fast_ok and kind != "fma", "a tiled weight needs 16-bit activations of its dtype")
         # up to 16 rows (32 for a small matrix) every wave fetches the rows of X itself; beyond that
         # the tiled GEMM is faster
-        if kind == "gemv_mfma" or (force is None and (m <= 16 or (m <= 32 and n * k <= (1 << 25)))):
+        # 9 to 16 rows against a wide matrix with an activation (gate and up): the tiled GEMM's tile of 64 rows of X
+        # fetches the rows of X once per 112 rows of W, gemv_tiled once per 16 or 32 (measured at 16 rows and
+        # 28,672 x 4,096: 44.6 against 51.7 us, at 12 rows 44.2 against 48.7, at 8 rows 44.0 against 43.5)
+        wide = (force is None and 8 < m <= 16 and mode in GATED and n * k >= (1 << 26) and m * k * 2 < (1 << 32)
+                and _wreg_plan(m, n, k) == (2, 1))
+        if not wide and (kind == "gemv_mfma" or (force is None and (m <= 16 or (m <= 32 and n * k <= (1 << 25))))):
             ro = rsc = None
             nxt = getattr(out, "_li_next_norm", None) if mode == EPI_ADD else None
             if (nxt is not None and m <= 16 and n % 32 == 0 and out.data_ptr() % 16 == 0 and nxt.dtype == torch.float32
@@ -300,21 +305,15 @@ def linear(x: torch.Tensor, w, mode: int = EPI_STORE, out: torch.Tensor | None =
                 ro = _RowsOut(ss.data_ptr(), xw.data_ptr(), nxt.data_ptr(), scale,
                               row_scales.data_ptr() if row_scales is not None else None)
             if lazy is not None:
-                # in float16 the kernel also leaves the scales for the product that adds into these rows next
-                nxt_scale = torch.empty((16,), dtype=torch.float32, device=x.device) if x.dtype == torch.float16 else None
-                rsc = _RowScale(lazy.ss.data_ptr(), lazy.ss.shape[0], lazy.eps, 1.0 / lazy.scale,
-                                lazy.row_scales.data_ptr() if lazy.row_scales is not None else None,
-                                nxt_scale.data_ptr() if nxt_scale is not None else None)
-                if nxt_scale is not None:
-                    lazy.x._li_row_scale = nxt_scale
+                rsc = _finish_norm(lazy, x)
             _check(lib.li_gemv_tiled(_ptr(x), _ptr(wd), DT[x.dtype], _ptr(out), out_dt, mode, m, n, k, 0, 0, rs,
                                      ctypes.byref(ro) if ro is not None else None,
                                      ctypes.byref(rsc) if rsc is not None else None, _stream()), "gemv_tiled")
             if ro is not None:
                 out._li_rows = (xw, ss, scale, nxt, out._version, row_scales)
             return out
-        _need(lazy is None, "a norm is finished by gemv_tiled alone")
-        if force is None and m <= 128:
+        _need(lazy is None or wide, "a norm is finished by gemv_tiled, or by gemm_wreg for gate and up")
+        if force is None and m <= 128 and not wide:
             # 17 to 128 rows: all of K in one workgroup and every epilogue the product's own (gemm_rows), where
             # that is estimated faster than the tiled GEMM with K split and its second kernel
             norm_rides = mode == EPI_ADD and getattr(out, "_li_next_norm", None) is not None
@@ -355,9 +354,10 @@ def linear(x: torch.Tensor, w, mode: int = EPI_STORE, out: torch.Tensor | None =
                 and (ws.data_ptr() | out.data_ptr() | nxt.data_ptr()) % 16 == 0):
             normed = torch.empty((m, n), dtype=x.dtype, device=x.device)
             na = _NormAfter(nxt.data_ptr(), normed.data_ptr(), DT[x.dtype], eps)
+        rsc = _finish_norm(lazy, x) if lazy is not None else None
         _check(lib.li_gemm_wreg(_ptr(x), _ptr(wd), DT[x.dtype], _ptr(out), out_dt, mode, m, n, k, tile, splits,
                                 _ptr(ws), rs, ctypes.byref(na) if na is not None else None, few_rows, wg_blocks,
-                                _stream()),
+                                ctypes.byref(rsc) if rsc is not None else None, _stream()),
                "gemm_wreg")
         if na is not None:
             out._li_normed = (normed, nxt, eps, out._version)
@@ -393,6 +393,18 @@ def linear(x: torch.Tensor, w, mode: int = EPI_STORE, out: torch.Tensor | None =
         _check(lib.li_gemm_mfma(_ptr(x), _ptr(wd), int(tiled), DT[x.dtype], _ptr(out), out_dt, mode, m, n, k,
                                 tile, splits, _ptr(ws), rs, _stream()), "gemm_mfma")
     return out
+
+
+def _finish_norm(lazy: "LazyNorm", x: torch.Tensor) -> _RowScale:
+    """What the product that reads an unfinished norm needs of it.  In float16 its kernel also leaves the scales
+    for the product that adds into these rows next."""
+    nxt_scale = torch.empty((16,), dtype=torch.float32, device=x.device) if x.dtype == torch.float16 else None
+    rsc = _RowScale(lazy.ss.data_ptr(), lazy.ss.shape[0], lazy.eps, 1.0 / lazy.scale,
+                    lazy.row_scales.data_ptr() if lazy.row_scales is not None else None,
+                    nxt_scale.data_ptr() if nxt_scale is not None else None)
+    if nxt_scale is not None:
+        lazy.x._li_row_scale = nxt_scale
+    return rsc
 
 
 # rows of W x rows of X of a workgroup of gemm_wreg

@@ -160,12 +160,14 @@ def test_linear_tiled_weights(ops, M, N, K, dt):
 
 
 @pytest.mark.parametrize("dt", F16S)
-@pytest.mark.parametrize("M,d,K2,N2", [(1, 4096, 4096, 6144), (8, 4096, 14336, 28672), (16, 96, 160, 200), (5, 2048, 64, 128256)])
+@pytest.mark.parametrize("M,d,K2,N2", [(1, 4096, 4096, 6144), (8, 4096, 14336, 28672), (16, 96, 160, 200), (5, 2048, 64, 128256),
+                                       (12, 4096, 14336, 28672), (16, 4096, 4096, 22016), (14, 4096, 4096, 6144)])
 def test_norm_split_over_two_products(ops, M, d, K2, N2, dt):
     """A decode step's product that adds into the residual stream prepares the norm that reads the rows
     next (x * weight in 16 bits, sums of squares), and the product behind the norm finishes it: the same
     result as norm kernel + product, without the kernel.  The preparation is void as soon as anything
-    else writes to the rows, and for any other norm."""
+    else writes to the rows, and for any other norm.  (From 9 rows on, gate and up against a wide matrix finish
+    the norm in the tiled GEMM's epilogue instead of gemv_tiled's: the last two cases.)"""
     g = torch.Generator().manual_seed(M + d)
     x0 = torch.randn(M, d, generator=g) * 3
     a = (torch.randn(M, K2, generator=g) * 0.5).to(dt)
@@ -222,14 +224,20 @@ def test_norm_split_over_two_products(ops, M, d, K2, N2, dt):
 
 
 @pytest.mark.parametrize("dt", F16S)
+@pytest.mark.parametrize("M,N2", [(7, 768), (12, 65536)])
 @pytest.mark.parametrize("rms,wscale", [(1e-2, 0.02), (1e3, 0.02), (1e3, 4.0), (3.0, 1.0)])
-def test_norm_split_over_two_products_at_a_models_own_scale(ops, rms, wscale, dt):
+def test_norm_split_over_two_products_at_a_models_own_scale(ops, rms, wscale, M, N2, dt):
     """The rows that travel in 16 bits between the two products are x * weight; a checkpoint's residual stream
     may be of the order of 0.01 or of 1000 and its norm weights of 0.02.  In float16 each row is scaled by a
     power of two taken from the norm before (left by the norm kernel, then by each product that finishes a
     norm), so the split norm is as exact as norm kernel + product at every scale, down a chain of layers in
-    which the rows grow; a view of the rows that a kernel writes through voids the preparation too."""
-    M, d, K2, N2 = 7, 1024, 512, 768
+    which the rows grow; a view of the rows that a kernel writes through voids the preparation too.  The second
+    shape is gate and up of 12 rows against a wide matrix, where the tiled GEMM finishes the norm and leaves the
+    scales."""
+    d, K2 = 1024, 512
+    gated = N2 > 768
+    assert not gated or ops._wreg_plan(M, N2, d) == (2, 1)
+    mode = ops.EPI_SWIGLU if gated else ops.EPI_STORE
     g = torch.Generator().manual_seed(3)
     x0 = torch.randn(M, d, generator=g) * rms
     x0[2, 5] = 40 * rms                                            # a row with one large element
@@ -249,13 +257,19 @@ def test_norm_split_over_two_products_at_a_models_own_scale(ops, rms, wscale, dt
         ln = ops.lazy_rmsnorm(x, wn, eps, dt)
         assert ln is not None and (ln.row_scales is not None) == (dt == torch.float16)
         assert torch.isfinite(ln.xw.float()).all()
-        fused = ops.linear(ln, w2t, out_dtype=torch.float32)
+        fused = ops.linear(ln, w2t, mode, out_dtype=torch.float32)
+        assert (getattr(x, "_li_row_scale", None) is not None) == (dt == torch.float16)
         xd = x.double().cpu()
         ref = (xd / torch.sqrt((xd ** 2).mean(1, keepdim=True) + eps) * wn.double().cpu()) @ w2.double().t()
-        plain = ops.linear(ops.rmsnorm(x.clone(), wn, eps, dt), w2t, out_dtype=torch.float32)
-        own = (plain.double().cpu() - ref).abs().max().item()
-        err = (fused.double().cpu() - ref).abs().max().item()
-        assert err < 1.5 * own + 1e-6 * ref.abs().max().item(), (layer, err, own)
+        if gated:
+            ref = torch.nn.functional.silu(ref[:, 0::2]) * ref[:, 1::2]
+        plain = ops.linear(ops.rmsnorm(x.clone(), wn, eps, dt), w2t, mode, out_dtype=torch.float32)
+        # (a gated product's largest errors sit at its few largest outputs, and the largest of them differs by a
+        # factor of two between two roundings of the same quality: there the root mean square is compared)
+        size = (lambda e: e.pow(2).mean().sqrt().item()) if gated else (lambda e: e.abs().max().item())
+        own = size(plain.double().cpu() - ref)
+        err = size(fused.double().cpu() - ref)
+        assert err < 1.5 * own + 1e-6 * size(ref), (layer, err, own)
     # a kernel that writes through a view of the rows voids what was prepared for the rows themselves
     ops.expect_norm(x, wn)
     ops.linear(a.to(DEV), wot, ops.EPI_ADD, out=x)
