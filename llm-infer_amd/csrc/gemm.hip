@@ -450,7 +450,7 @@ static __device__ __attribute__((aligned(1024))) unsigned char zero_kib[1024];  
 
 template <class T, int NT, int MT, int KW, int D>
 __global__ __launch_bounds__(64 * KW) void gemm_rows_kernel(const T* __restrict__ X, const T* __restrict__ Wt,
-                                                            int K, int ldx, Epilogue e) {
+                                                            int K, int ldx, Epilogue e, RowsOut ro) {
     typedef typename Vec<T>::v8 v8;
     constexpr int UNITS = 2 * MT, STAGE = UNITS * 1024, REGION = D * STAGE;     // bytes of LDS: a stage, a wave's stages
     static_assert(REGION >= NT * MT * 1024, "a wave's partial tiles lie in its own stages");
@@ -606,10 +606,26 @@ __global__ __launch_bounds__(64 * KW) void gemm_rows_kernel(const T* __restrict_
         const int m = 16 * j + r, col = (tile0 + t) * 16 + 4 * g;
         const float vv[4] = {v[0], v[1], v[2], v[3]};
         if (e.mode == EPI_ADD && quads) {
-            if (m < e.M && col < e.N) {
-                f32x4 o = res[i];
-                o[0] += v[0]; o[1] += v[1]; o[2] += v[2]; o[3] += v[3];
-                *(f32x4*)((float*)e.C + (int64_t)m * e.N + col) = o;
+            f32x4 o = res[i];
+            o[0] += v[0]; o[1] += v[1]; o[2] += v[2]; o[3] += v[3];
+            if (m < e.M && col < e.N) *(f32x4*)((float*)e.C + (int64_t)m * e.N + col) = o;
+            if (NT * MT == 1 && ro.ss) {
+                // RowsOut (one tile a workgroup, at most 16 rows: the host sees to it), as gemv_tiled leaves it
+                float sq = 0.f;
+                if (m < e.M && col < e.N) {
+                    const float scale = ro.row_scale ? ro.row_scale[m] : ro.scale;
+                    const f32x4 wv = *(const f32x4*)(ro.w + col);
+                    typename Vec<T>::v4 xw;
+#pragma unroll
+                    for (int q = 0; q < 4; ++q) {
+                        sq = fmaf(o[q], o[q], sq);
+                        xw[q] = from_f32<T>(o[q] * wv[q] * scale);
+                    }
+                    *(typename Vec<T>::v4*)((T*)ro.xw + (int64_t)m * e.N + col) = xw;
+                }
+                sq += __shfl_xor(sq, 16, WAVE);
+                sq += __shfl_xor(sq, 32, WAVE);
+                if (g == 0) ro.ss[(int64_t)blockIdx.x * 16 + r] = sq;          // (rows beyond M: zeros)
             }
         } else if (e.mode == EPI_ROPE && e.rs.cos_sin) {
             if (m < e.M && col < e.N) {
@@ -799,11 +815,13 @@ extern "C" int li_gemv_tiled(const void* X, const void* Wt, int dt, void* C, int
 }
 
 
-// 17 to 128 rows of X against a tiled weight, every epilogue its own (gemm_rows).  nt: 1 or 2 tiles of 16 rows
+// Up to 128 rows of X against a tiled weight, every epilogue its own (gemm_rows).  nt: 1 or 2 tiles of 16 rows
 // of W a workgroup, kw: 4 or 8 waves that share K (8: up to 64 rows of X) (0: chosen here); ldx: elements from
-// one row of X to the next.
+// one row of X to the next.  ro (or null; mode EPI_ADD, at most 16 rows, one tile a workgroup): RowsOut, with one
+// partial sum a row for each of the N / 16 workgroups.
 extern "C" int li_gemm_rows(const void* X, const void* Wt, int dt, void* C, int out_dt, int mode,
-                            int M, int N, int K, int ldx, int nt, int kw, const RopeStore* rs, hipStream_t stream) {
+                            int M, int N, int K, int ldx, int nt, int kw, const RopeStore* rs, const RowsOut* ro,
+                            hipStream_t stream) {
     int rc = check_common(X, Wt, C, M, N, K, mode, out_dt);
     if (rc) return rc;
     if (dt != DT_F16 && dt != DT_BF16) return LI_BAD_ARG;
@@ -813,11 +831,15 @@ extern "C" int li_gemm_rows(const void* X, const void* Wt, int dt, void* C, int 
     Epilogue e;
     rc = make_epilogue(e, C, mode, out_dt, M, N, rs);
     if (rc) return rc;
-    const int mt = M <= 32 ? 2 : (M <= 64 ? 4 : (M <= 96 ? 6 : 8));
+    const int mt = M <= 16 ? 1 : (M <= 32 ? 2 : (M <= 64 ? 4 : (M <= 96 ? 6 : 8)));
     const int tiles = (N + 15) / 16;
     if (nt <= 0) nt = tiles >= 1024 ? 2 : 1;          // enough workgroups for 256 CUs either way
     if (kw <= 0) kw = 4;
     if ((nt != 1 && nt != 2) || (kw != 4 && kw != 8) || (kw == 8 && mt > 4)) return LI_BAD_ARG;
+    if (ro && (mode != EPI_ADD || M > 16 || nt != 1 || (N & 15) || !ro->ss || !ro->xw || !ro->w || !(ro->scale > 0.f) ||
+               (((uintptr_t)C | (uintptr_t)ro->w) & 15) || ((uintptr_t)ro->xw & 7)))
+        return LI_BAD_ARG;
+    const RowsOut no_out{};
     const int blocks = (tiles + nt - 1) / nt;
     // stages of 64 of K a wave: what 128 KiB of LDS hold for the workgroup's waves
 #define GO(T, NT, MT, KW, D)                                                                              \
@@ -830,11 +852,13 @@ extern "C" int li_gemm_rows(const void* X, const void* Wt, int dt, void* C, int 
                 return LI_HIP_ERROR;                                                                      \
             allowed = true;                                                                               \
         }                                                                                                 \
-        kfn<<<blocks, 64 * KW, lds, stream>>>((const T*)X, (const T*)Wt, K, ldx, e);                      \
+        kfn<<<blocks, 64 * KW, lds, stream>>>((const T*)X, (const T*)Wt, K, ldx, e, ro ? *ro : no_out);   \
     } while (0)
 #define BY_MT(T, NT)                                            \
     do {                                                        \
-        if (mt == 2 && kw == 4) GO(T, NT, 2, 4, 6);             \
+        if (mt == 1 && kw == 4) GO(T, NT, 1, 4, 8);             \
+        else if (mt == 1) GO(T, NT, 1, 8, 8);                   \
+        else if (mt == 2 && kw == 4) GO(T, NT, 2, 4, 6);        \
         else if (mt == 2) GO(T, NT, 2, 8, 4);                   \
         else if (mt == 4 && kw == 4) GO(T, NT, 4, 4, 4);        \
         else if (mt == 4) GO(T, NT, 4, 8, 2);                   \

@@ -293,12 +293,18 @@ def linear(x: torch.Tensor, w, mode: int = EPI_STORE, out: torch.Tensor | None =
                 and _wreg_plan(m, n, k) == (2, 1))
         if not wide and (kind == "gemv_mfma" or (force is None and (m <= 16 or (m <= 32 and n * k <= (1 << 25))))):
             ro = rsc = None
+            # 9 to 16 rows with the residual sum against a matrix with a long K (down): gemm_rows, one tile of W a
+            # workgroup (measured at 16 rows and 4,096 x 14,336: 25.5 against 30.3 us, at 12 rows 24.4 against 27.1, at 8
+            # rows the same; against 4,096 x 4,096 gemv_tiled is as fast)
+            tall = (force is None and 8 < m <= 16 and mode == EPI_ADD and lazy is None and k >= 8192 and n % 16 == 0
+                    and x.stride(0) % 8 == 0 and x.stride(1) == 1)
             nxt = getattr(out, "_li_next_norm", None) if mode == EPI_ADD else None
             if (nxt is not None and m <= 16 and n % 32 == 0 and out.data_ptr() % 16 == 0 and nxt.dtype == torch.float32
                     and nxt.shape == (n,) and nxt.is_cuda and nxt.data_ptr() % 16 == 0):
                 # the rows of `out` are about to be complete rows of a residual stream that this norm reads
                 # next: leave x * weight in 16 bits and the sums of squares for the product behind the norm
-                ss = torch.empty((lib.li_gemv_tiled_blocks(m, n, k, 0, 0), 16), dtype=torch.float32, device=x.device)
+                blocks = n // 16 if tall else lib.li_gemv_tiled_blocks(m, n, k, 0, 0)
+                ss = torch.empty((blocks, 16), dtype=torch.float32, device=x.device)
                 xw = torch.empty((m, n), dtype=x.dtype, device=x.device)
                 scale = 0.125 if x.dtype == torch.float16 else 1.0        # x * w stays inside float16's range
                 row_scales = getattr(out, "_li_row_scale", None) if x.dtype == torch.float16 else None
@@ -306,9 +312,13 @@ def linear(x: torch.Tensor, w, mode: int = EPI_STORE, out: torch.Tensor | None =
                               row_scales.data_ptr() if row_scales is not None else None)
             if lazy is not None:
                 rsc = _finish_norm(lazy, x)
-            _check(lib.li_gemv_tiled(_ptr(x), _ptr(wd), DT[x.dtype], _ptr(out), out_dt, mode, m, n, k, 0, 0, rs,
-                                     ctypes.byref(ro) if ro is not None else None,
-                                     ctypes.byref(rsc) if rsc is not None else None, _stream()), "gemv_tiled")
+            if tall:
+                _check(lib.li_gemm_rows(_ptr(x), _ptr(wd), DT[x.dtype], _ptr(out), out_dt, mode, m, n, k, x.stride(0), 1, 4,
+                                        rs, ctypes.byref(ro) if ro is not None else None, _stream()), "gemm_rows")
+            else:
+                _check(lib.li_gemv_tiled(_ptr(x), _ptr(wd), DT[x.dtype], _ptr(out), out_dt, mode, m, n, k, 0, 0, rs,
+                                         ctypes.byref(ro) if ro is not None else None,
+                                         ctypes.byref(rsc) if rsc is not None else None, _stream()), "gemv_tiled")
             if ro is not None:
                 out._li_rows = (xw, ss, scale, nxt, out._version, row_scales)
             return out
@@ -327,7 +337,7 @@ def linear(x: torch.Tensor, w, mode: int = EPI_STORE, out: torch.Tensor | None =
         parts = kind.split(":")
         _check(lib.li_gemm_rows(_ptr(x), _ptr(wd), DT[x.dtype], _ptr(out), out_dt, mode, m, n, k, x.stride(0),
                                 int(parts[1]) if len(parts) > 1 else 0, int(parts[2]) if len(parts) > 2 else 0,
-                                rs, _stream()), "gemm_rows")
+                                rs, None, _stream()), "gemm_rows")
         return out
     if kind.startswith("wreg"):                                # "wreg[:<tile>[:<splits>[:<few rows>]]]" (a test's choice)
         _need(tiled and fast_ok and m * k * 2 < (1 << 32), "gemm_wreg: a tiled weight, X below 4 GiB")
