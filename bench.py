@@ -55,7 +55,7 @@ def main() -> int:
                     help="also time one step of this many prompts with lengths uniform in 16..2048")
     ap.add_argument("--dtype", default="fp16", choices=["fp16", "bf16"])
     ap.add_argument("--prefill-tokens", type=int, default=2048)
-    ap.add_argument("--points", default="1,64", help="further decode batch sizes, comma separated ('' for none)")
+    ap.add_argument("--points", default="1,16,64", help="further decode batch sizes, comma separated ('' for none)")
     ap.add_argument("--no-other-shapes", action="store_true",
                     help="leave out the 1B ragged step and the 7B batch-64 decode that the default run adds to points")
     ap.add_argument("--no-further-sizes", action="store_true",
