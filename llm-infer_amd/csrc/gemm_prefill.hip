@@ -225,8 +225,8 @@ __global__ __launch_bounds__(256) void gemm_big_kernel(const T* __restrict__ X, 
 // no spills (the build checks that the kernel uses no scratch memory).
 // MJ: the tile's rows of X in blocks of 16 (8: 128 rows; 4: 64 rows, for products of up to 64 rows, which then
 // fetch and multiply no rows that are not there).  A: how many steps ahead of their use the loads of W are
-// issued (2, or 4 for products of few rows, where one workgroup a CU has to keep enough of W in flight by itself:
-// 8 NI KiB a wave instead of 4 NI).
+// issued (2; 4 for products of few rows, where one workgroup a CU has to keep enough of W in flight by itself:
+// 8 NI KiB a wave instead of 4 NI; 3 for 65 to 128 rows, where two workgroups may share a CU).
 template <class T, int NI, int MODE, int MJ = 8, int A = 2>
 __global__ __launch_bounds__(256) void gemm_wreg_kernel(const T* __restrict__ X, const T* __restrict__ Wt,
                                                         int K, int k_per_split, float* __restrict__ ws, Epilogue e,
@@ -610,7 +610,8 @@ extern "C" int li_gemm_big(const void* X, const void* W, int tiled, int dt, void
 // `na` (or null): with K split and the residual sum as epilogue, the kernel that adds the partial sums also
 // takes the norm of the finished rows; it must fit (norm_after_fits), the caller has checked the same.
 // few_rows (tile 2 only): 1 = the tile has 64 rows of X, 2 = 128 rows; either way W is fetched four steps ahead
-// instead of two (for products of up to 128 rows, where a workgroup has a CU to itself); 0 = neither.
+// instead of two (for products of up to 128 rows, where a workgroup has a CU to itself); 3 = 128 rows of X and W
+// three steps ahead (two workgroups still fit a CU); 0 = none of these.
 // wg_blocks: blocks of 16 rows of W a workgroup, from 1 to the tile's own number (0: that number); fewer make
 // more workgroups of a product whose full tiles would leave CUs without one.
 extern "C" int li_gemm_wreg(const void* X, const void* Wt, int dt, void* C, int out_dt, int mode,
@@ -620,14 +621,14 @@ extern "C" int li_gemm_wreg(const void* X, const void* Wt, int dt, void* C, int 
     if (rc) return rc;
     if (dt != DT_F16 && dt != DT_BF16) return LI_BAD_ARG;
     if (K % 32 != 0 || ((uintptr_t)X & 15) || ((uintptr_t)Wt & 15)) return LI_UNSUPPORTED;
-    if (tile < 0 || tile > 2 || few_rows < 0 || few_rows > 2 || (few_rows && tile != 2)) return LI_BAD_ARG;
+    if (tile < 0 || tile > 2 || few_rows < 0 || few_rows > 3 || (few_rows && tile != 2)) return LI_BAD_ARG;
     if ((int64_t)M * K * 2 >= ((int64_t)1 << 32)) return LI_UNSUPPORTED;
     if (splits < 1 || (splits > 1 && !ws)) return LI_BAD_ARG;
     if (M == 0) return LI_OK;
     Epilogue e;
     rc = make_epilogue(e, C, mode, out_dt, M, N, rs);
     if (rc) return rc;
-    const int bn = 256 - 64 * tile, bm = few_rows == 1 ? 64 : 128, bk = 32, ahead = few_rows ? 4 : 2;
+    const int bn = 256 - 64 * tile, bm = few_rows == 1 ? 64 : 128, bk = 32, ahead = few_rows == 3 ? 3 : (few_rows ? 4 : 2);
     if (wg_blocks == 0) wg_blocks = bn / 16;
     if (wg_blocks < 1 || wg_blocks > bn / 16) return LI_BAD_ARG;
     int k_per_split = ((K + splits - 1) / splits + bk - 1) / bk * bk;
@@ -670,6 +671,7 @@ extern "C" int li_gemm_wreg(const void* X, const void* Wt, int dt, void* C, int 
         else if (tile == 1) BY_MODE(T, 3, 8, 2);        \
         else if (few_rows == 1) BY_MODE(T, 2, 4, 4);    \
         else if (few_rows == 2) BY_MODE(T, 2, 8, 4);    \
+        else if (few_rows == 3) BY_MODE(T, 2, 8, 3);    \
         else BY_MODE(T, 2, 8, 2);                       \
     } while (0)
     if (dt == DT_F16) LAUNCH(f16); else LAUNCH(bf16);

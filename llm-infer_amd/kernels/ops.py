@@ -345,9 +345,11 @@ def linear(x: torch.Tensor, w, mode: int = EPI_STORE, out: torch.Tensor | None =
         tile, splits = _wreg_plan(m, n, k)
         # up to 64 rows against the narrowest tile: a tile of 64 rows of X (none fetched or multiplied that is not
         # there) with W four steps ahead (measured at 64 rows: gate/up 53.9 -> 46.0 us, down 35.9 -> 35.0 and 29.5
-        # with K in 8; the same depth with 128 rows of X: by itself gate/up at 128 rows 61.5 -> 53.6 us, in a decode
-        # step at batch 128 nothing (11.41 and 11.47 ms), and is not used)
-        few_rows = 1 if (tile == 2 and m <= 64) else 0
+        # with K in 8; the same depth with 128 rows of X leaves room for one workgroup a CU and gained nothing in a
+        # decode step at batch 128: 11.41 and 11.47 ms).  65 to 128 rows: W three steps ahead, which still lets two
+        # workgroups share a CU (by itself gate/up at 96 rows 58.9 -> 52.1 us, at 128 rows 60.6 -> 54.1; in a decode
+        # step at batch 96 9.68 -> 9.55 ms, at batch 128 11.52 -> 11.46; from 192 rows on it gains nothing)
+        few_rows = (1 if m <= 64 else (3 if m <= 128 else 0)) if tile == 2 else 0
         wg_blocks = _wreg_blocks(tile, splits, m, n)
         if len(parts) > 1:                                     # "wreg:<tile>:<splits>:<few rows>:<blocks of W>"
             tile, splits = int(parts[1]), int(parts[2]) if len(parts) > 2 else 1

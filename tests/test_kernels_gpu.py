@@ -127,7 +127,7 @@ def test_linear_tiled_weights(ops, M, N, K, dt):
     # W into registers (tiles of 256, 192, 128 rows of W): the planner's choice and every tile, K whole and split
     kinds += ["wreg", "wreg:0", "wreg:1", "wreg:2", "wreg:0:2", "wreg:1:5", "wreg:2:3"]
     # the narrowest tile with W four steps ahead, with 64 rows of X (:1) and with 128 (:2), K whole and split
-    kinds += ["wreg:2:1:1", "wreg:2:3:1", "wreg:2:1:2", "wreg:2:4:2"]
+    kinds += ["wreg:2:1:1", "wreg:2:3:1", "wreg:2:1:2", "wreg:2:4:2", "wreg:2:1:3", "wreg:2:4:3"]        # (:3: three steps ahead)
     # workgroups that take fewer blocks of 16 rows of W than their tile has (the last field), for every tile
     kinds += ["wreg:2:1:1:7", "wreg:2:3:1:5", "wreg:2:1:2:6", "wreg:0:2:0:13", "wreg:1:1:0:9", "wreg:2:1:0:1"]
     # all of K in one workgroup, the rows of X through LDS of each wave's own (up to 128 rows): one and two tiles of W
