@@ -295,8 +295,9 @@ def linear(x: torch.Tensor, w, mode: int = EPI_STORE, out: torch.Tensor | None =
             ro = rsc = None
             # 9 to 16 rows with the residual sum against a matrix with a long K (down): gemm_rows, one tile of W a
             # workgroup (measured at 16 rows and 4,096 x 14,336: 25.5 against 30.3 us, at 12 rows 24.4 against 27.1, at 8
-            # rows the same; against 4,096 x 4,096 gemv_tiled is as fast)
-            tall = (force is None and 8 < m <= 16 and mode == EPI_ADD and lazy is None and k >= 8192 and n >= 4096 and n % 16 == 0
+            # rows the same; 4,096 x 11,008 at 16 rows 20.9 against 25.9, 2,048 x 8,192 10.2 against 11.9; against
+            # 4,096 x 4,096 gemv_tiled is as fast)
+            tall = (force is None and 8 < m <= 16 and mode == EPI_ADD and lazy is None and k >= 8192 and n >= 2048 and n % 16 == 0
                     and x.stride(0) % 8 == 0 and x.stride(1) == 1)
             nxt = getattr(out, "_li_next_norm", None) if mode == EPI_ADD else None
             if (nxt is not None and m <= 16 and n % 32 == 0 and out.data_ptr() % 16 == 0 and nxt.dtype == torch.float32
